@@ -1,0 +1,155 @@
+"""ctypes binding of libmellin_hip.so (the C ABI declared in include/mellin_hip.h).
+
+The library is the only compute back end of this package: if it has not been
+built, importing this module raises, and nothing falls back to PyTorch or CPU
+code.  Build it with ``python cnn-mellin_amd/build.py`` (hipcc, gfx950).
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmellin_hip.so")
+
+AX_MCORR, AX_MCONV, AX_LCORR, AX_LCONV = 0, 1, 2, 3
+
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_ptr = ctypes.c_void_p
+_size_t = ctypes.c_size_t
+
+if not os.path.isfile(LIB_PATH):
+    raise ImportError(
+        "%s is missing: build the HIP library first (python %s)"
+        % (LIB_PATH, os.path.join(_HERE, "build.py"))
+    )
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+
+# name -> (restype, argtypes); every symbol include/mellin_hip.h declares
+_ACC1D = [_ptr, _ptr] + [_i64] * 10 + [_int] * 3 + [_ptr, _ptr]
+_ACC2D = [_ptr, _ptr] + [_i64] * 17 + [_int] * 3 + [_ptr, _ptr]
+_DIMS = [_i64] * 17
+SYMBOLS = {
+    "mellin_version": (_int, []),
+    "mellin_last_error": (ctypes.c_char_p, []),
+    "mellin_last_variant": (ctypes.c_char_p, []),
+    "mellin_set_variant": (_int, [ctypes.c_char_p]),
+    "mellin_corr2d_backward_weight_workspace": (_size_t, [_int, _int] + _DIMS),
+}
+for _t in ("f32", "f64"):
+    for _n in ("mcorr1d", "mconv1d"):
+        SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC1D)
+    for _n in ("mcorrlcorr", "mconvlconv", "lcorrlcorr", "lconvlconv"):
+        SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC2D)
+    SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
+    SYMBOLS["mellin_corr2d_backward_input_" + _t] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
+    SYMBOLS["mellin_corr2d_backward_weight_" + _t] = (
+        _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
+
+for _name, (_res, _args) in SYMBOLS.items():
+    _fn = getattr(lib, _name)          # AttributeError if the library lacks a declared symbol
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+
+def last_error():
+    return lib.mellin_last_error().decode()
+
+
+def last_variant():
+    return lib.mellin_last_variant().decode()
+
+
+def set_variant(name=None):
+    _check(lib.mellin_set_variant((name or "").encode()))
+
+
+def _check(code):
+    if code != 0:
+        raise RuntimeError("libmellin_hip: %s (code %d)" % (last_error(), code))
+
+
+def suffix(dtype):
+    try:
+        return _SUFFIX[dtype]
+    except KeyError:
+        raise RuntimeError(
+            "libmellin_hip computes in float32 or float64, got %s" % dtype) from None
+
+
+def require_device(*tensors):
+    """All tensors must live on one HIP device; returns it."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "this build runs on AMD GPUs only: expected a HIP ('cuda') tensor, got a "
+                "tensor on %s (there is no CPU path)" % t.device)
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("tensors are on different devices: %s and %s" % (dev, t.device))
+    return dev
+
+
+def _stream(dev):
+    return _ptr(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _dp(t):
+    return _ptr(t.data_ptr()) if t is not None and t.numel() else _ptr(0)
+
+
+def accumulate(name, f, g, h, c_out, c_in, batch, nf, ng, nh, s, d, p, u, tf, tg, th):
+    """Call one of the accumulate-into-h kernels; sizes/params are ints (1-D) or pairs (2-D)."""
+    dev = require_device(f, g, h)
+    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(h.dtype)))
+    with torch.cuda.device(dev):
+        if isinstance(nf, int):
+            code = fn(_dp(f), _dp(g), c_out, c_in, batch, nf, ng, nh, s, d, p, u,
+                      int(tf), int(tg), int(th), _dp(h), _stream(dev))
+        else:
+            code = fn(_dp(f), _dp(g), c_out, c_in, batch, nf[0], nf[1], ng[0], ng[1],
+                      nh[0], nh[1], s[0], s[1], d[0], d[1], p[0], p[1], u[0], u[1],
+                      int(tf), int(tg), int(th), _dp(h), _stream(dev))
+    _check(code)
+    return h
+
+
+def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):
+    return (batch, c_in, c_out, nf[0], nf[1], ng[0], ng[1], nh[0], nh[1],
+            s[0], s[1], d[0], d[1], p[0], p[1], u[0], u[1])
+
+
+def corr2d_forward(kind_x, input, weight, bias, out, dims):
+    dev = require_device(input, weight, bias, out)
+    fn = getattr(lib, "mellin_corr2d_forward_" + suffix(out.dtype))
+    with torch.cuda.device(dev):
+        _check(fn(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))
+    return out
+
+
+def corr2d_backward_input(kind_x, weight, grad_out, grad_input, dims):
+    dev = require_device(weight, grad_out, grad_input)
+    fn = getattr(lib, "mellin_corr2d_backward_input_" + suffix(grad_input.dtype))
+    with torch.cuda.device(dev):
+        _check(fn(kind_x, _dp(weight), _dp(grad_out), *dims, _dp(grad_input), _stream(dev)))
+    return grad_input
+
+
+def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims):
+    dev = require_device(input, grad_out, grad_weight)
+    suf = suffix(grad_weight.dtype)
+    nbytes = lib.mellin_corr2d_backward_weight_workspace(kind_x, grad_weight.element_size(), *dims)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    fn = getattr(lib, "mellin_corr2d_backward_weight_" + suf)
+    with torch.cuda.device(dev):
+        _check(fn(kind_x, _dp(input), _dp(grad_out), *dims, _dp(grad_weight),
+                  _dp(ws), nbytes, _stream(dev)))
+    return grad_weight

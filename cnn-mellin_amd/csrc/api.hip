@@ -1,0 +1,279 @@
+// extern "C" surface of libmellin_hip (declared in include/mellin_hip.h):
+// argument validation, descriptor construction and kernel-variant dispatch.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/mellin_hip.h"
+#include "mellin_common.hpp"
+
+using namespace mellin;
+
+namespace {
+
+thread_local char g_error[512] = "";
+thread_local const char *g_variant = "";
+thread_local int g_forced = 0;   // 0 automatic, 1 generic
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_hip(hipError_t e, const char *what) {
+  if (e == hipSuccess) return MELLIN_OK;
+  return fail(MELLIN_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool mellin_kind(int k) { return k == AX_MCORR || k == AX_MCONV; }
+
+// Parameter domain of one axis.  s, d, u divide or scale indices and must be
+// positive; on a Mellin axis p + 1 is a divisor so p >= 0.
+int check_axis(const char *fn, const char *ax, int kind, i64 nf, i64 ng, i64 nh,
+               i64 s, i64 d, i64 p, i64 u) {
+  if (nf < 0 || ng < 0 || nh < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: negative size on the %s axis (nf=%lld ng=%lld nh=%lld)",
+                fn, ax, (long long)nf, (long long)ng, (long long)nh);
+  if (s < 1 || d < 1 || u < 1)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: s, d and u must be >= 1 on the %s axis (s=%lld d=%lld u=%lld)",
+                fn, ax, (long long)s, (long long)d, (long long)u);
+  if (mellin_kind(kind) && p < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: p must be >= 0 on the Mellin axis (p=%lld)", fn, (long long)p);
+  // keep index products inside 62 bits
+  const i64 lim = (i64)1 << 30;
+  if (nf > lim || ng > lim || nh > lim || s > lim || d > lim || u > lim || p > lim || p < -lim)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: size or parameter too large on the %s axis", fn, ax);
+  return MELLIN_OK;
+}
+
+int check_channels(const char *fn, i64 c_out, i64 c_in, i64 batch) {
+  if (c_out < 0 || c_in < 0 || batch < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: negative channel or batch count (c_out=%lld c_in=%lld batch=%lld)",
+                fn, (long long)c_out, (long long)c_in, (long long)batch);
+  return MELLIN_OK;
+}
+
+// ---- section 1: accumulate-into-h kernels ---------------------------------
+template <typename T>
+int accumulate_2d(const char *fn, int kind_x, int kind_y, const T *f, const T *g,
+                  i64 c_out, i64 c_in, i64 batch, i64 nfx, i64 nfy, i64 ngx,
+                  i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy,
+                  i64 px, i64 py, i64 ux, i64 uy, int tf, int tg, int th, T *h,
+                  void *stream) {
+  int rc;
+  if ((rc = check_channels(fn, c_out, c_in, batch))) return rc;
+  if ((rc = check_axis(fn, "x", kind_x, nfx, ngx, nhx, sx, dx, px, ux))) return rc;
+  if ((rc = check_axis(fn, "y", kind_y, nfy, ngy, nhy, sy, dy, py, uy))) return rc;
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  if (batch * c_out * nh == 0) return MELLIN_OK;               // nothing to write
+  if (c_in * nf * ng == 0) return MELLIN_OK;                   // empty sum: h unchanged
+  if (!f || !g || !h) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  SepConv pr;
+  pr.x = make_axis(kind_x, nfx, ngx, nhx, sx, dx, px, ux);
+  pr.y = make_axis(kind_y, nfy, ngy, nhy, sy, dy, py, uy);
+  pr.batch = batch; pr.c_out = c_out; pr.c_in = c_in;
+  pr.f_m = tf ? nf : c_in * nf;   pr.f_c = tf ? c_out * nf : nf;
+  pr.g_n = tg ? ng : c_in * ng;   pr.g_c = tg ? batch * ng : ng;
+  pr.h_n = th ? nh : c_out * nh;  pr.h_m = th ? batch * nh : nh;
+  pr.accumulate = 1;
+  g_variant = "generic";
+  return check_hip(launch_sepconv_generic<T>(pr, f, g, (const T *)nullptr, h,
+                                             (hipStream_t)stream), fn);
+}
+
+// ---- section 2: operator-level entry points -------------------------------
+int check_corr2d(const char *fn, int kind_x, i64 batch, i64 c_in, i64 c_out,
+                 i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy, i64 sx,
+                 i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy) {
+  int rc;
+  if (kind_x != AX_MCORR && kind_x != AX_LCORR)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: kind_x must be MELLIN_AXIS_MCORR or MELLIN_AXIS_LCORR", fn);
+  if ((rc = check_channels(fn, c_out, c_in, batch))) return rc;
+  if ((rc = check_axis(fn, "x", kind_x, nfx, ngx, nhx, sx, dx, px, ux))) return rc;
+  if ((rc = check_axis(fn, "y", AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy))) return rc;
+  return MELLIN_OK;
+}
+
+template <typename T>
+int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
+                   const T *bias, i64 batch, i64 c_in, i64 c_out, i64 nfx,
+                   i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy,
+                   i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, T *out,
+                   void *stream) {
+  int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
+                        nhy, sx, sy, dx, dy, px, py, ux, uy);
+  if (rc) return rc;
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  if (batch * c_out * nh == 0) return MELLIN_OK;
+  if (!out || (c_in * nf * ng != 0 && (!input || !weight)))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  SepConv pr;
+  pr.x = make_axis(kind_x, nfx, ngx, nhx, sx, dx, px, ux);
+  pr.y = make_axis(AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy);
+  if (c_in * nf * ng == 0) pr.x.nh_eff = 0;                   // empty sum: out = bias
+  pr.batch = batch; pr.c_out = c_out; pr.c_in = c_in;
+  pr.f_m = c_in * nf; pr.f_c = nf;
+  pr.g_n = c_in * ng; pr.g_c = ng;
+  pr.h_n = c_out * nh; pr.h_m = nh;
+  pr.accumulate = 0;
+  g_variant = "generic";
+  return check_hip(launch_sepconv_generic<T>(pr, weight, input, bias, out,
+                                             (hipStream_t)stream), fn);
+}
+
+// grad_input[n, ci, gx, gy] = sum_{co, fx, fy} weight[co, ci, fx, fy] *
+//   grad_out[n, co, hx, hy] over the (hx, hy) whose forward taps land on
+// (gx, gy).  Solving the forward relations for the output index gives the
+// convolution relations with s and u exchanged:
+//   x (Mellin): hx = (p + 1)(gx + u)/(fx + d) - s
+//   x (linear): hx = (u gx - d fx + p)/s
+//   y (linear): hy = (u gy - d fy + p)/s
+template <typename T>
+int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
+                          const T *grad_out, i64 batch, i64 c_in, i64 c_out,
+                          i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy,
+                          i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux,
+                          i64 uy, T *grad_input, void *stream) {
+  int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
+                        nhy, sx, sy, dx, dy, px, py, ux, uy);
+  if (rc) return rc;
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  if (batch * c_in * ng == 0) return MELLIN_OK;
+  if (!grad_input || (c_out * nf * nh != 0 && (!weight || !grad_out)))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  SepConv pr;
+  const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
+  // roles: "signal" = grad_out (length nh), "output" = grad_input (length ng)
+  pr.x = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
+  pr.y = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
+  if (c_out * nf * nh == 0) pr.x.nh_eff = 0;
+  pr.batch = batch; pr.c_out = c_in; pr.c_in = c_out;
+  pr.f_m = nf; pr.f_c = c_in * nf;                              // weight read transposed
+  pr.g_n = c_out * nh; pr.g_c = nh;
+  pr.h_n = c_in * ng; pr.h_m = ng;
+  pr.accumulate = 0;
+  g_variant = "generic";
+  return check_hip(launch_sepconv_generic<T>(pr, weight, grad_out, (const T *)nullptr,
+                                             grad_input, (hipStream_t)stream), fn);
+}
+
+template <typename T>
+int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
+                           const T *grad_out, i64 batch, i64 c_in, i64 c_out,
+                           i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy,
+                           i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux,
+                           i64 uy, T *grad_weight, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+  int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
+                        nhy, sx, sy, dx, dy, px, py, ux, uy);
+  if (rc) return rc;
+  (void)workspace; (void)workspace_bytes;
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  if (c_out * c_in * nf == 0) return MELLIN_OK;
+  if (!grad_weight || (batch * ng * nh != 0 && (!input || !grad_out)))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  SepReduce pr;
+  pr.x = make_axis(kind_x, nfx, ngx, nhx, sx, dx, px, ux);
+  pr.y = make_axis(AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy);
+  if (batch * ng * nh == 0) pr.x.nh_eff = 0;
+  pr.batch = batch; pr.c_out = c_out; pr.c_in = c_in;
+  g_variant = "generic";
+  return check_hip(launch_sepreduce_generic<T>(pr, grad_out, input, grad_weight,
+                                               (hipStream_t)stream), fn);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mellin_version(void) { return 100; }
+
+const char *mellin_last_error(void) { return g_error; }
+
+const char *mellin_last_variant(void) { return g_variant; }
+
+int mellin_set_variant(const char *name) {
+  if (!name || !*name) { g_forced = 0; return MELLIN_OK; }
+  if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
+  return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
+}
+
+#define DEFINE_1D(NAME, T, KX, KY)                                             \
+  MELLIN_DECL_1D(NAME, T) {                                                    \
+    return accumulate_2d<T>(#NAME, KX, KY, f, g, c_out, c_in, batch, nf, 1,    \
+                            ng, 1, nh, 1, s, 1, d, 1, p, 0, u, 1,              \
+                            transposed_f, transposed_g, transposed_h, h,       \
+                            stream);                                           \
+  }
+#define DEFINE_2D(NAME, T, KX, KY)                                             \
+  MELLIN_DECL_2D(NAME, T) {                                                    \
+    return accumulate_2d<T>(#NAME, KX, KY, f, g, c_out, c_in, batch, nfx, nfy, \
+                            ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py, ux,    \
+                            uy, transposed_f, transposed_g, transposed_h, h,   \
+                            stream);                                           \
+  }
+
+DEFINE_1D(mellin_mcorr1d_f32, float, AX_MCORR, AX_LCORR)
+DEFINE_1D(mellin_mcorr1d_f64, double, AX_MCORR, AX_LCORR)
+DEFINE_1D(mellin_mconv1d_f32, float, AX_MCONV, AX_LCONV)
+DEFINE_1D(mellin_mconv1d_f64, double, AX_MCONV, AX_LCONV)
+DEFINE_2D(mellin_mcorrlcorr_f32, float, AX_MCORR, AX_LCORR)
+DEFINE_2D(mellin_mcorrlcorr_f64, double, AX_MCORR, AX_LCORR)
+DEFINE_2D(mellin_mconvlconv_f32, float, AX_MCONV, AX_LCONV)
+DEFINE_2D(mellin_mconvlconv_f64, double, AX_MCONV, AX_LCONV)
+DEFINE_2D(mellin_lcorrlcorr_f32, float, AX_LCORR, AX_LCORR)
+DEFINE_2D(mellin_lcorrlcorr_f64, double, AX_LCORR, AX_LCORR)
+DEFINE_2D(mellin_lconvlconv_f32, float, AX_LCONV, AX_LCONV)
+DEFINE_2D(mellin_lconvlconv_f64, double, AX_LCONV, AX_LCONV)
+
+#define CORR2D_ARGS                                                            \
+  batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
+  ux, uy
+
+int mellin_corr2d_forward_f32(int kind_x, const float *input, const float *weight,
+                              const float *bias, MELLIN_CORR2D_DIMS, float *out,
+                              void *stream) {
+  return corr2d_forward<float>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream);
+}
+int mellin_corr2d_forward_f64(int kind_x, const double *input, const double *weight,
+                              const double *bias, MELLIN_CORR2D_DIMS, double *out,
+                              void *stream) {
+  return corr2d_forward<double>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream);
+}
+int mellin_corr2d_backward_input_f32(int kind_x, const float *weight,
+                                     const float *grad_out, MELLIN_CORR2D_DIMS,
+                                     float *grad_input, void *stream) {
+  return corr2d_backward_input<float>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input, stream);
+}
+int mellin_corr2d_backward_input_f64(int kind_x, const double *weight,
+                                     const double *grad_out, MELLIN_CORR2D_DIMS,
+                                     double *grad_input, void *stream) {
+  return corr2d_backward_input<double>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input, stream);
+}
+size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
+                                               MELLIN_CORR2D_DIMS) {
+  (void)kind_x; (void)elem_bytes;
+  (void)batch; (void)c_in; (void)c_out; (void)nfx; (void)nfy; (void)ngx; (void)ngy;
+  (void)nhx; (void)nhy; (void)sx; (void)sy; (void)dx; (void)dy; (void)px; (void)py;
+  (void)ux; (void)uy;
+  return 0;
+}
+int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,
+                                      const float *grad_out, MELLIN_CORR2D_DIMS,
+                                      float *grad_weight, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return corr2d_backward_weight<float>(__func__, kind_x, input, grad_out, CORR2D_ARGS,
+                                       grad_weight, workspace, workspace_bytes, stream);
+}
+int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
+                                      const double *grad_out, MELLIN_CORR2D_DIMS,
+                                      double *grad_weight, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return corr2d_backward_weight<double>(__func__, kind_x, input, grad_out, CORR2D_ARGS,
+                                        grad_weight, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

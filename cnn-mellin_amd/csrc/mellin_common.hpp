@@ -1,0 +1,90 @@
+// Shared declarations of libmellin_hip: problem descriptors, the per-axis tap
+// relation, and the launchers each translation unit exports to the C API.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mellin {
+
+typedef int64_t i64;
+
+enum AxisKind : int { AX_MCORR = 0, AX_MCONV = 1, AX_LCORR = 2, AX_LCONV = 3 };
+
+// One axis of a separable tap structure: output index h and filter index f
+// select signal index g, or nothing.
+struct Axis {
+  int kind;
+  i64 nf, ng, nh;    // filter, signal, allocated output lengths
+  i64 s, d, p, u;
+  i64 nh_eff;        // min(nh, support size): outputs at or past it have no tap
+};
+
+// h[n, m, hx, hy] (+)= sum_{c, fx, fy} f[m, c, fx, fy] * g[n, c, tap_x(hx, fx), tap_y(hy, fy)]
+// with every tensor addressed through explicit element strides so that the
+// transposed layouts of the reference contract and the role swaps of the
+// backward passes need no copies.
+struct SepConv {
+  Axis x, y;
+  i64 batch, c_out, c_in;        // c_out: output channels (m), c_in: contracted channels (c)
+  i64 f_m, f_c;                  // filter strides; spatial part is dense (nfx, nfy)
+  i64 g_n, g_c;                  // signal strides; spatial part is dense (ngx, ngy)
+  i64 h_n, h_m;                  // output strides; spatial part is dense (nhx, nhy)
+  int accumulate;                // 1: h += result (h pre-initialised); 0: h = bias + result
+};
+
+// Reduction form used by the weight gradient:
+// w[m, c, fx, fy] = sum_{n, hx, hy} a[n, m, hx, hy] * g[n, c, tap_x(hx, fx), tap_y(hy, fy)]
+struct SepReduce {
+  Axis x, y;                     // nf = filter size (output of the reduction), nh = size of `a`
+  i64 batch, c_out, c_in;
+};
+
+__host__ __device__ inline i64 floor_div(i64 a, i64 b) {
+  i64 q = a / b;
+  return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
+
+// Signal index chosen by (h, f) on one axis, or -1.  p1 = p + 1.
+__host__ __device__ inline i64 tap_index(int kind, i64 h, i64 f, i64 ng, i64 s,
+                                         i64 d, i64 p, i64 u) {
+  i64 num, den, off = 0;
+  switch (kind) {
+    case AX_MCORR: num = (h + s) * (f + d); den = p + 1; off = u; break;
+    case AX_MCONV: num = (p + 1) * (h + s); den = f + d; off = u; break;
+    case AX_LCORR: num = s * h + d * f - p; den = u; break;
+    default:       num = s * h - d * f + p; den = u; break;
+  }
+  if (num % den != 0) return -1;
+  const i64 g = num / den - off;
+  return (g >= 0 && g < ng) ? g : -1;
+}
+
+inline i64 support_size(int kind, i64 nf, i64 ng, i64 s, i64 d, i64 p, i64 u) {
+  i64 v;
+  switch (kind) {
+    case AX_MCORR: v = floor_div((ng + u - 1) * (p + 1), d) - s + 1; break;
+    case AX_MCONV: v = floor_div((nf + d - 1) * (ng + u - 1), p + 1) - s + 1; break;
+    case AX_LCORR: v = floor_div(u * (ng - 1) + p, s) + 1; break;
+    default:       v = floor_div(u * (ng - 1) + d * (nf - 1) - p, s) + 1; break;
+  }
+  return v > 0 ? v : 0;
+}
+
+inline Axis make_axis(int kind, i64 nf, i64 ng, i64 nh, i64 s, i64 d, i64 p, i64 u) {
+  Axis a;
+  a.kind = kind; a.nf = nf; a.ng = ng; a.nh = nh; a.s = s; a.d = d; a.p = p; a.u = u;
+  const i64 sup = support_size(kind, nf, ng, s, d, p, u);
+  a.nh_eff = sup < nh ? sup : nh;
+  return a;
+}
+
+// ---- launchers (each returns the hipError_t of the launch) ----------------
+template <typename T>
+hipError_t launch_sepconv_generic(const SepConv &pr, const T *f, const T *g,
+                                  const T *bias, T *h, hipStream_t stream);
+template <typename T>
+hipError_t launch_sepreduce_generic(const SepReduce &pr, const T *a, const T *g,
+                                    T *w, hipStream_t stream);
+
+}  // namespace mellin

@@ -1,0 +1,168 @@
+/*
+ * mellin_hip.h -- C ABI of libmellin_hip.so: Mellin / linear convolution
+ * kernels for AMD MI355X (gfx950), hand-written in HIP.
+ *
+ * The library replaces the device half of the reference's PyTorch extension:
+ * the CUDA adapters of ext/torch_cuda.cu:45-303 and the kernels of
+ * c/cuda/include/cdrobert/mellin/mconv_cuda.cuh that those adapters launch.
+ * All pointers are DEVICE pointers owned by the caller; the library keeps no
+ * reference to them after a call returns.  Every call is asynchronous on the
+ * HIP stream passed as `stream` (NULL = the default stream), performs no
+ * synchronisation, and allocates no memory.  Every function returns MELLIN_OK
+ * or an error code; mellin_last_error() gives the message of the calling
+ * thread's most recent failure.
+ *
+ * Index relations (h = output index, f = filter index, g = signal index; a tap
+ * exists only if the division is exact and 0 <= g < ng):
+ *
+ *   Mellin correlation  g = (h + s)(f + d)/(p + 1) - u     (mconv.h:65)
+ *   Mellin convolution  g = (p + 1)(h + s)/(f + d) - u     (mconv.h:24-25)
+ *   linear correlation  g = (s h + d f - p)/u              (mconv.h:168-171)
+ *   linear convolution  g = (s h - d f + p)/u              (mconv.h:105-107)
+ *
+ * with s, d, u >= 1 and p >= 0 on a Mellin axis.  "x" is the first spatial
+ * axis (time), "y" the second (frequency).
+ */
+#ifndef MELLIN_HIP_H_
+#define MELLIN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MELLIN_OK 0
+#define MELLIN_ERR_ARGUMENT 1    /* inconsistent sizes / parameters / null pointer */
+#define MELLIN_ERR_RUNTIME 2     /* the HIP runtime reported an error */
+#define MELLIN_ERR_WORKSPACE 3   /* workspace missing or too small */
+
+/* Axis kinds for the functions that take one. */
+#define MELLIN_AXIS_MCORR 0
+#define MELLIN_AXIS_MCONV 1
+#define MELLIN_AXIS_LCORR 2
+#define MELLIN_AXIS_LCONV 3
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int mellin_version(void);
+
+/* Message for the calling thread's most recent non-OK return ("" if none). */
+const char *mellin_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * 1. Accumulating kernels: the reference's kernel-level contract.
+ *
+ * Same argument meaning and order as the reference's host launchers
+ *   MCorr1D     mconv.h:92-100   / mconv_cuda.cuh MCorr1DCuda
+ *   MConv1D     mconv.h:52-60    / MConv1DCuda
+ *   MCorrLCorr  mconv.h:218-227  / MCorrLCorrCuda
+ *   MConvLConv  mconv.h:154-163  / MConvLConvCuda
+ * which ext/torch_cuda.cu:45-177 binds, plus the trailing stream:
+ *   f   filter, (c_out, c_in, nfx[, nfy]) or (c_in, c_out, ...) if transposed_f
+ *   g   signal, (batch, c_in, ngx[, ngy]) or (c_in, batch, ...) if transposed_g
+ *   h   output, (batch, c_out, nhx[, nhy]) or (c_out, batch, ...) if transposed_h;
+ *       caller-allocated and initialised (bias or zeros); results are ADDED
+ *       to it.  nh may be smaller or larger than the support size; outputs
+ *       at or beyond the support size are left untouched.
+ * All three buffers are dense (C-contiguous) in the stated layout.
+ * The *_lcorrlcorr / *_lconvlconv variants use the linear relations on both
+ * axes; the reference has no such kernel (its non-Mellin model calls
+ * torch.nn.Conv2d, models.py:334-336).
+ * ------------------------------------------------------------------------ */
+#define MELLIN_DECL_1D(NAME, T)                                                \
+  int NAME(const T *f, const T *g, int64_t c_out, int64_t c_in, int64_t batch, \
+           int64_t nf, int64_t ng, int64_t nh, int64_t s, int64_t d,           \
+           int64_t p, int64_t u, int transposed_f, int transposed_g,           \
+           int transposed_h, T *h, void *stream)
+#define MELLIN_DECL_2D(NAME, T)                                                \
+  int NAME(const T *f, const T *g, int64_t c_out, int64_t c_in, int64_t batch, \
+           int64_t nfx, int64_t nfy, int64_t ngx, int64_t ngy, int64_t nhx,    \
+           int64_t nhy, int64_t sx, int64_t sy, int64_t dx, int64_t dy,        \
+           int64_t px, int64_t py, int64_t ux, int64_t uy, int transposed_f,   \
+           int transposed_g, int transposed_h, T *h, void *stream)
+
+MELLIN_DECL_1D(mellin_mcorr1d_f32, float);
+MELLIN_DECL_1D(mellin_mcorr1d_f64, double);
+MELLIN_DECL_1D(mellin_mconv1d_f32, float);
+MELLIN_DECL_1D(mellin_mconv1d_f64, double);
+MELLIN_DECL_2D(mellin_mcorrlcorr_f32, float);
+MELLIN_DECL_2D(mellin_mcorrlcorr_f64, double);
+MELLIN_DECL_2D(mellin_mconvlconv_f32, float);
+MELLIN_DECL_2D(mellin_mconvlconv_f64, double);
+MELLIN_DECL_2D(mellin_lcorrlcorr_f32, float);
+MELLIN_DECL_2D(mellin_lcorrlcorr_f64, double);
+MELLIN_DECL_2D(mellin_lconvlconv_f32, float);
+MELLIN_DECL_2D(mellin_lconvlconv_f64, double);
+
+/* ------------------------------------------------------------------------
+ * 2. Operator-level entry points: one launch per pass of a correlation layer.
+ *
+ * These replace the adapter + autograd glue of the reference for the two
+ * layer types (x axis Mellin or linear correlation, y axis always linear
+ * correlation):
+ *   forward          mcorrlcorr_cuda, ext/torch_cuda.cu:144-177, with
+ *                    BuildOutput (ext/torch.cpp:88-101) folded in: `out` is
+ *                    WRITTEN, out = bias + correlation (bias may be NULL);
+ *   backward_input   the mconvlconv(weight^T, grad_out, u, s, p, d) call of
+ *                    MCorrLCorrOp::backward, ext/torch.cpp:284-290;
+ *                    `grad_input` is written;
+ *   backward_weight  the mcorrlcorr(input^T, grad_out^T, d, s, p, u) call,
+ *                    ext/torch.cpp:292-298; `grad_weight` is written.  The
+ *                    reduction over batch and output positions runs in a
+ *                    fixed order (no floating-point atomics), so results are
+ *                    bit-reproducible from run to run.
+ * Layouts are the natural dense ones:
+ *   input (batch, c_in, ngx, ngy)    weight (c_out, c_in, nfx, nfy)
+ *   out / grad_out (batch, c_out, nhx, nhy)      bias (c_out)
+ * kind_x is MELLIN_AXIS_MCORR or MELLIN_AXIS_LCORR.  1-D layers pass a unit
+ * y axis (nfy = ngy = nhy = 1, sy = dy = uy = 1, py = 0).
+ *
+ * backward_weight needs scratch memory for partial sums: ask
+ * mellin_corr2d_backward_weight_workspace() for the byte count and pass a
+ * device buffer of at least that size (256-byte aligned); its contents on
+ * entry do not matter and are garbage on exit.
+ * ------------------------------------------------------------------------ */
+#define MELLIN_CORR2D_DIMS                                                     \
+  int64_t batch, int64_t c_in, int64_t c_out, int64_t nfx, int64_t nfy,        \
+  int64_t ngx, int64_t ngy, int64_t nhx, int64_t nhy, int64_t sx, int64_t sy,  \
+  int64_t dx, int64_t dy, int64_t px, int64_t py, int64_t ux, int64_t uy
+
+int mellin_corr2d_forward_f32(int kind_x, const float *input,
+                              const float *weight, const float *bias,
+                              MELLIN_CORR2D_DIMS, float *out, void *stream);
+int mellin_corr2d_forward_f64(int kind_x, const double *input,
+                              const double *weight, const double *bias,
+                              MELLIN_CORR2D_DIMS, double *out, void *stream);
+
+int mellin_corr2d_backward_input_f32(int kind_x, const float *weight,
+                                     const float *grad_out, MELLIN_CORR2D_DIMS,
+                                     float *grad_input, void *stream);
+int mellin_corr2d_backward_input_f64(int kind_x, const double *weight,
+                                     const double *grad_out, MELLIN_CORR2D_DIMS,
+                                     double *grad_input, void *stream);
+
+size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
+                                               MELLIN_CORR2D_DIMS);
+int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,
+                                      const float *grad_out, MELLIN_CORR2D_DIMS,
+                                      float *grad_weight, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
+                                      const double *grad_out, MELLIN_CORR2D_DIMS,
+                                      double *grad_weight, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
+/* Name of the kernel variant the most recent operator-level call on this
+ * thread dispatched to (for tests and profiling), e.g. "generic". */
+const char *mellin_last_variant(void);
+
+/* Force a variant for subsequent operator-level calls on this thread:
+ * NULL or "" = automatic choice; "generic" = the one-thread-per-output
+ * kernels.  Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
+int mellin_set_variant(const char *name);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MELLIN_HIP_H_ */

@@ -1,0 +1,129 @@
+"""Host-side behaviour of the drop-in module that needs no GPU: output-length
+rules, argument checks and their messages, layer construction, and the
+C-ABI's own argument validation (which returns before any kernel launch)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import mconv
+import _mellin_hip as hip
+from oracle import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SIZE_FUNCS = ["lconv_support", "lconv_valid", "lcorr_support", "lcorr_valid",
+              "mconv_support", "mconv_valid", "mcorr_support", "mcorr_valid"]
+
+
+def test_public_names_match_reference():
+    # mconv.py:22-37 of the reference
+    ref_all = ["lconv_support_size", "lconv_valid_size", "lcorr_support_size", "lcorr_valid_size",
+               "mconv_support_size", "mconv_valid_size", "mcorr_support_size", "mcorr_valid_size",
+               "mcorr1d", "MCorr1d", "mcorrlcorr", "MCorrLCorr", "snd2col", "spec2col"]
+    for name in ref_all:
+        assert name in mconv.__all__ and hasattr(mconv, name)
+
+
+@pytest.mark.parametrize("name", SIZE_FUNCS)
+def test_size_functions_equal_checker(name):
+    g = torch.Generator().manual_seed(3)
+    fn, ofn = getattr(mconv, name + "_size"), getattr(oracle, name + "_size")
+    for _ in range(2000):
+        nf, ng = int(torch.randint(1, 20, (1,), generator=g)), int(torch.randint(1, 900, (1,), generator=g))
+        s, d, u = (int(v) for v in torch.randint(1, 6, (3,), generator=g))
+        p = int(torch.randint(0, 6, (1,), generator=g))
+        assert fn(nf, ng, s, d, p, u) == ofn(nf, ng, s, d, p, u), (name, nf, ng, s, d, p, u)
+
+
+def test_size_values_of_benchmark_configs():
+    # the table of output lengths the survey derives for the BASELINE configs
+    assert mconv.mcorr_valid_size(16, 256) == 16 and mconv.mconv_valid_size(16, 256) == 256
+    grid = [(s, d, p) for s in (1, 2) for d in (1, 2) for p in (0, 3)]
+    assert [mconv.mcorr_valid_size(8, 780, s, d, p) for s, d, p in grid] == [97, 390, 86, 346, 96, 389, 85, 345]
+    assert [mconv.lcorr_valid_size(8, 780, s, d, p) for s, d, p in grid] == [773, 776, 766, 769, 387, 388, 383, 385]
+    assert (mconv.mcorr_valid_size(8, 512), mconv.lcorr_valid_size(4, 41)) == (64, 38)
+    assert (mconv.lcorr_valid_size(3, 256, 1, 2, 2), mconv.lcorr_valid_size(3, 41, 1, 1, 1)) == (254, 40)
+
+
+def test_argument_errors_have_reference_wording():
+    w = torch.zeros(4, 3, 5)
+    with pytest.raises(RuntimeError, match=r"Expected 3-dimensional arg\[0\], but got 4-dimensional tensor "
+                                           r"for argument #1 'input' \(while checking arguments for mcorr1d\)"):
+        mconv.mcorr1d(torch.zeros(2, 3, 9, 1), w)
+    with pytest.raises(RuntimeError, match=r"Expected tensor to have size 3 at dimension 1, but got size 2 "
+                                           r"for argument #1 'input'"):
+        mconv.mcorr1d(torch.zeros(2, 2, 9), w)
+    with pytest.raises(RuntimeError, match=r"Expected tensor to have size 4 at dimension 0, but got size 5 "
+                                           r"for argument #3 'bias'"):
+        mconv.mcorr1d(torch.zeros(2, 3, 9), w, torch.zeros(5))
+    with pytest.raises(RuntimeError, match="either an integer or a tuple of 2 integers"):
+        mconv.mcorrlcorr(torch.zeros(1, 3, 9, 9), torch.zeros(4, 3, 2, 2), None, s=(1, 2, 3))
+    with pytest.raises(NotImplementedError, match='_impl "fft" not supported'):
+        mconv.mcorr1d(torch.zeros(2, 3, 9), w, _impl="fft")
+
+
+def test_cpu_tensors_are_refused_loudly():
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mconv.mcorr1d(torch.zeros(2, 3, 9), torch.zeros(4, 3, 5))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mconv.MCorrLCorr(3, 4, (2, 2))(torch.zeros(1, 3, 9, 9))
+
+
+def test_layers_keep_reference_parameter_layout():
+    torch.manual_seed(0)
+    m = mconv.MCorrLCorr(3, 64, (8, 4), p=(3, 1), r=(0, 2), bias=True)
+    assert list(m.state_dict()) == ["weight", "bias"]
+    assert m.weight.shape == (64, 3, 8, 4) and m.bias.shape == (64,)
+    bound = (3 * 8 * 4) ** -0.5          # U(+-1/sqrt(fan_in)), mconv.py:1062-1067
+    assert float(m.weight.abs().max()) <= bound and float(m.bias.abs().max()) <= bound
+    assert float(m.weight.abs().max()) > 0.9 * bound
+    assert (m.s, m.d, m.p, m.r) == ((1, 1), (1, 1), (3, 1), (0, 2))
+    m1 = mconv.MCorr1d(5, 7, 3, bias=False)
+    assert m1.bias is None and m1.weight.shape == (7, 5, 3) and m1.s == (1,)
+    assert "kernel_size=" in repr(m)
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mellin_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    names = set(re.findall(r"\b(mellin_[a-z0-9_]+)\s*\(", text))
+    names |= set(re.findall(r"MELLIN_DECL_[12]D\((mellin_[a-z0-9_]+)\s*,", text))
+    return sorted(names)
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 23, names
+    lib = ctypes.CDLL(hip.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), "libmellin_hip.so lacks %s" % n
+    assert set(hip.SYMBOLS) == set(names)
+    assert lib.mellin_version() >= 100
+
+
+def test_cabi_rejects_bad_arguments_before_launch():
+    lib = hip.lib
+    dims_ok = [1, 1, 1, 2, 2, 4, 4, 2, 3] + [1, 1, 1, 1, 0, 0, 1, 1]
+    null = ctypes.c_void_p(0)
+    # kind_x must be a correlation kind
+    assert lib.mellin_corr2d_forward_f32(hip.AX_MCONV, null, null, null, *dims_ok, null, null) == 1
+    assert "kind_x" in hip.last_error()
+    bad = list(dims_ok)
+    bad[9] = 0                                          # sx = 0
+    assert lib.mellin_corr2d_forward_f32(hip.AX_MCORR, null, null, null, *bad, null, null) == 1
+    assert "s, d and u must be >= 1" in hip.last_error()
+    bad = list(dims_ok)
+    bad[13] = -1                                        # px = -1 on the Mellin axis
+    assert lib.mellin_corr2d_forward_f32(hip.AX_MCORR, null, null, null, *bad, null, null) == 1
+    assert "p must be >= 0" in hip.last_error()
+    # null pointers with non-empty sizes
+    assert lib.mellin_corr2d_forward_f32(hip.AX_MCORR, null, null, null, *dims_ok, null, null) == 1
+    assert "null pointer" in hip.last_error()
+    # empty problems are fine and launch nothing
+    empty = list(dims_ok)
+    empty[0] = 0
+    assert lib.mellin_corr2d_forward_f32(hip.AX_MCORR, null, null, null, *empty, null, null) == 0
+    assert lib.mellin_set_variant(b"no-such-variant") == 1
+    assert lib.mellin_set_variant(b"") == 0
