@@ -143,13 +143,19 @@ def corr2d_backward_input(kind_x, weight, grad_out, grad_input, dims):
     return grad_input
 
 
-def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims):
+def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims, workspace=None,
+                           workspace_bytes=None):
+    """Weight gradient; scratch memory comes from `workspace` or, if None, from torch's
+    caching allocator on the launch stream."""
     dev = require_device(input, grad_out, grad_weight)
     suf = suffix(grad_weight.dtype)
-    nbytes = lib.mellin_corr2d_backward_weight_workspace(kind_x, grad_weight.element_size(), *dims)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    if workspace is None:
+        workspace_bytes = lib.mellin_corr2d_backward_weight_workspace(
+            kind_x, grad_weight.element_size(), *dims)
+        workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=dev)
+                     if workspace_bytes else None)
     fn = getattr(lib, "mellin_corr2d_backward_weight_" + suf)
     with torch.cuda.device(dev):
         _check(fn(kind_x, _dp(input), _dp(grad_out), *dims, _dp(grad_weight),
-                  _dp(ws), nbytes, _stream(dev)))
+                  _dp(workspace), workspace_bytes, _stream(dev)))
     return grad_weight

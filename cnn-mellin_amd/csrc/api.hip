@@ -6,6 +6,7 @@
 
 #include "../../include/mellin_hip.h"
 #include "mellin_common.hpp"
+#include "tile_gemm.hpp"
 
 using namespace mellin;
 
@@ -56,6 +57,31 @@ int check_channels(const char *fn, i64 c_out, i64 c_in, i64 batch) {
   return MELLIN_OK;
 }
 
+// Gather-form dispatch: the matrix-core tile kernel when it applies (fp32,
+// sizes within its plan limits), otherwise one thread per output.
+template <typename T>
+hipError_t run_sepconv(const SepConv &pr, const T *f, const T *g, const T *bias,
+                       T *h, hipStream_t stream) {
+  g_variant = "generic";
+  return launch_sepconv_generic<T>(pr, f, g, bias, h, stream);
+}
+
+template <>
+hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
+                              const float *bias, float *h, hipStream_t stream) {
+  if (g_forced != 1) {
+    TilePlan pl;
+    size_t lds = 0;
+    int mt = 0, nt = 0;
+    if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
+      g_variant = "mfma";
+      return launch_tile_gemm(pl, lds, mt, nt, f, g, bias, h, stream);
+    }
+  }
+  g_variant = "generic";
+  return launch_sepconv_generic<float>(pr, f, g, bias, h, stream);
+}
+
 // ---- section 1: accumulate-into-h kernels ---------------------------------
 template <typename T>
 int accumulate_2d(const char *fn, int kind_x, int kind_y, const T *f, const T *g,
@@ -79,9 +105,7 @@ int accumulate_2d(const char *fn, int kind_x, int kind_y, const T *f, const T *g
   pr.g_n = tg ? ng : c_in * ng;   pr.g_c = tg ? batch * ng : ng;
   pr.h_n = th ? nh : c_out * nh;  pr.h_m = th ? batch * nh : nh;
   pr.accumulate = 1;
-  g_variant = "generic";
-  return check_hip(launch_sepconv_generic<T>(pr, f, g, (const T *)nullptr, h,
-                                             (hipStream_t)stream), fn);
+  return check_hip(run_sepconv<T>(pr, f, g, (const T *)nullptr, h, (hipStream_t)stream), fn);
 }
 
 // ---- section 2: operator-level entry points -------------------------------
@@ -119,9 +143,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
   pr.g_n = c_in * ng; pr.g_c = ng;
   pr.h_n = c_out * nh; pr.h_m = nh;
   pr.accumulate = 0;
-  g_variant = "generic";
-  return check_hip(launch_sepconv_generic<T>(pr, weight, input, bias, out,
-                                             (hipStream_t)stream), fn);
+  return check_hip(run_sepconv<T>(pr, weight, input, bias, out, (hipStream_t)stream), fn);
 }
 
 // grad_input[n, ci, gx, gy] = sum_{co, fx, fy} weight[co, ci, fx, fy] *
@@ -155,9 +177,8 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   pr.g_n = c_out * nh; pr.g_c = nh;
   pr.h_n = c_in * ng; pr.h_m = ng;
   pr.accumulate = 0;
-  g_variant = "generic";
-  return check_hip(launch_sepconv_generic<T>(pr, weight, grad_out, (const T *)nullptr,
-                                             grad_input, (hipStream_t)stream), fn);
+  return check_hip(run_sepconv<T>(pr, weight, grad_out, (const T *)nullptr, grad_input,
+                                  (hipStream_t)stream), fn);
 }
 
 template <typename T>
@@ -198,6 +219,7 @@ const char *mellin_last_variant(void) { return g_variant; }
 int mellin_set_variant(const char *name) {
   if (!name || !*name) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
+  if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
   return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
 }
 

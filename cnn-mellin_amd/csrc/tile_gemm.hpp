@@ -1,0 +1,39 @@
+// Descriptor of one launch of the matrix-core gather-GEMM (tile_gemm.hip).
+#pragma once
+
+#include "mellin_common.hpp"
+
+namespace mellin {
+
+struct TilePlan {
+  // problem (all fit 32 bits; checked by make_tile_plan)
+  int batch, M, C;                 // images, output channels, contracted channels
+  int nfx, nfy, nf;                // filter extent and nfx * nfy
+  int ngx, ngy;                    // signal extent
+  int nox, noy, Q;                 // allocated output extent and nox * noy
+  int nox_eff, noy_eff;            // outputs at or past these have no tap
+  i64 f_m, f_c, g_n, g_c, h_n, h_m;
+  int accumulate;
+  // x axis: Mellin kinds evaluate taps per (row, filter row); linear kinds use
+  // the coordinate ax * ox + bx * fx + cx (divided by ux)
+  int kind_x, sx, dx, px, ux;
+  int ax, bx, cx, bx_min, bx_span;
+  int Ax, Bx, Cx0;                 // LDS row = Ax * (ox - ox_lo) + Bx * fx + Cx0
+  // y axis: coordinate ay * oy + by * fy + cy (divided by uy)
+  int ay, by, cy, uy, by_min, by_span;
+  // tiling
+  int segment, chunks_per_row, tiles_per_image, total_tiles;
+  int R, RS;                       // virtual rows per channel and their stride (words)
+  int CP, CP_log2;                 // staged columns rounded up to a power of two
+  int CC;                          // channels staged per chunk
+  int KCp;                         // CC * nf rounded up to even
+  int WSS;                         // stride of the K-major filter block (words)
+};
+
+bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt);
+
+hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
+                            const float *f, const float *g, const float *bias,
+                            float *h, hipStream_t stream);
+
+}  // namespace mellin

@@ -49,6 +49,7 @@
  */
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 typedef int64_t i64;
 
@@ -152,6 +153,12 @@ static i64 support_clip(int kind, i64 nf, i64 ng, i64 nh, i64 s, i64 d, i64 p,
     const i64 total = batch * c_out * nhx * nhy;                               \
     const i64 Nhx = support_clip(kind_x, nfx, ngx, nhx, sx, dx, px, ux);       \
     const i64 Nhy = support_clip(kind_y, nfy, ngy, nhy, sy, dy, py, uy);       \
+    if (total <= 0 || Nhx <= 0 || Nhy <= 0) return;                            \
+    /* index maps first, as MCorr1D v3 does (mconv.h:1100-1113) */             \
+    i64 *xmap = (i64 *)malloc(sizeof(i64) * (size_t)(Nhx * nfx + 1));          \
+    i64 *ymap = (i64 *)malloc(sizeof(i64) * (size_t)(Nhy * nfy + 1));          \
+    oracle_tap_map(kind_x, nfx, ngx, Nhx, sx, dx, px, ux, xmap);               \
+    oracle_tap_map(kind_y, nfy, ngy, Nhy, sy, dy, py, uy, ymap);               \
     _Pragma("omp parallel for schedule(static)")                               \
     for (i64 i = 0; i < total; ++i) {                                          \
       const i64 hy = i % nhy, hx = (i / nhy) % nhx, ip = i / (nhy * nhx);      \
@@ -160,12 +167,13 @@ static i64 support_clip(int kind, i64 nf, i64 ng, i64 nh, i64 s, i64 d, i64 p,
       const i64 bt = transposed_h ? ip % batch : ip / c_out;                   \
       const T *f_co = f + (transposed_f ? co : co * c_in) * nf;                \
       const T *g_bt = g + (transposed_g ? bt : bt * c_in) * ng;                \
+      const i64 *xm = xmap + hx * nfx, *ym = ymap + hy * nfy;                  \
       ACC acc = 0;                                                             \
       for (i64 fx = 0; fx < nfx; ++fx) {                                       \
-        const i64 gx = oracle_tap(kind_x, hx, fx, ngx, sx, dx, px, ux);        \
+        const i64 gx = xm[fx];                                                 \
         if (gx < 0) continue;                                                  \
         for (i64 fy = 0; fy < nfy; ++fy) {                                     \
-          const i64 gy = oracle_tap(kind_y, hy, fy, ngy, sy, dy, py, uy);      \
+          const i64 gy = ym[fy];                                               \
           if (gy < 0) continue;                                                \
           const T *fp = f_co + fx * nfy + fy, *gp = g_bt + gx * ngy + gy;      \
           for (i64 ci = 0; ci < c_in; ++ci)                                    \
@@ -174,6 +182,8 @@ static i64 support_clip(int kind, i64 nf, i64 ng, i64 nh, i64 s, i64 d, i64 p,
       }                                                                        \
       h[i] += acc;                                                             \
     }                                                                          \
+    free(xmap);                                                                \
+    free(ymap);                                                                \
   }
 
 DEFINE_SEPCONV(oracle_sepconv_f32, float, float)
