@@ -121,6 +121,21 @@ int check_corr2d(const char *fn, int kind_x, i64 batch, i64 c_in, i64 c_out,
   return MELLIN_OK;
 }
 
+SepConv forward_problem(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
+                        i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px,
+                        i64 py, i64 ux, i64 uy) {
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  SepConv pr;
+  pr.x = make_axis(kind_x, nfx, ngx, nhx, sx, dx, px, ux);
+  pr.y = make_axis(AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy);
+  pr.batch = batch; pr.c_out = c_out; pr.c_in = c_in;
+  pr.f_m = c_in * nf; pr.f_c = nf;
+  pr.g_n = c_in * ng; pr.g_c = ng;
+  pr.h_n = c_out * nh; pr.h_m = nh;
+  pr.accumulate = 0;
+  return pr;
+}
+
 template <typename T>
 int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
                    const T *bias, i64 batch, i64 c_in, i64 c_out, i64 nfx,
@@ -191,11 +206,23 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
-  (void)workspace; (void)workspace_bytes;
   const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
   if (c_out * c_in * nf == 0) return MELLIN_OK;
   if (!grad_weight || (batch * ng * nh != 0 && (!input || !grad_out)))
     return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  if (sizeof(T) == 4 && g_forced != 1 && batch * ng * nh != 0) {
+    WgradPlan wp;
+    if (make_wgrad_plan(forward_problem(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy,
+                                        sx, sy, dx, dy, px, py, ux, uy), wp)) {
+      if (!workspace || workspace_bytes < wp.ws_bytes)
+        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
+                    wp.ws_bytes, workspace_bytes);
+      g_variant = "mfma";
+      return check_hip(launch_wgrad(wp, (const float *)grad_out, (const float *)input,
+                                    (float *)grad_weight, (float *)workspace,
+                                    (hipStream_t)stream), fn);
+    }
+  }
   SepReduce pr;
   pr.x = make_axis(kind_x, nfx, ngx, nhx, sx, dx, px, ux);
   pr.y = make_axis(AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy);
@@ -277,11 +304,12 @@ int mellin_corr2d_backward_input_f64(int kind_x, const double *weight,
 }
 size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
                                                MELLIN_CORR2D_DIMS) {
-  (void)kind_x; (void)elem_bytes;
-  (void)batch; (void)c_in; (void)c_out; (void)nfx; (void)nfy; (void)ngx; (void)ngy;
-  (void)nhx; (void)nhy; (void)sx; (void)sy; (void)dx; (void)dy; (void)px; (void)py;
-  (void)ux; (void)uy;
-  return 0;
+  if (elem_bytes != 4 || g_forced == 1) return 0;
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
+  WgradPlan wp;
+  if (!make_wgrad_plan(forward_problem(kind_x, CORR2D_ARGS), wp)) return 0;
+  return wp.ws_bytes;
 }
 int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,
                                       const float *grad_out, MELLIN_CORR2D_DIMS,

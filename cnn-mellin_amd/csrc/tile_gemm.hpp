@@ -30,10 +30,31 @@ struct TilePlan {
   int WSS;                         // stride of the K-major filter block (words)
 };
 
-bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt);
+// force_nt: 0 lets the plan pick the number of 32-position tiles per wavefront
+bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt,
+                    int force_nt = 0);
 
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
                             float *h, hipStream_t stream);
+
+// Weight gradient (wgrad_gemm.hip): position tiling and signal staging of the
+// forward problem in `t`, plus the blocking of the (c_out) x (c_in * taps) output.
+struct WgradPlan {
+  TilePlan t;
+  i64 a_n, a_m;                    // grad_out strides: image, channel (positions are dense)
+  int J;                           // c_in * nfx * nfy
+  int mt, jt, nt;                  // 32-wide tiles per workgroup: channels, columns, positions per wave
+  int m_groups, j_groups, M_pad, J_pad;
+  int CCj;                         // input channels a column block can touch
+  int GSS;                         // row stride of the staged grad_out tile (words)
+  int S;                           // position shares = persistent workgroups per output block
+  size_t lds_bytes, ws_bytes;
+};
+
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp);
+
+hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float *input,
+                        float *grad_weight, float *workspace, hipStream_t stream);
 
 }  // namespace mellin

@@ -1,0 +1,147 @@
+// Device-side pieces shared by the matrix-core kernels: direct global->LDS
+// loads, division-free index splitting, position-tile geometry, and the staging
+// of signal rows into affine "virtual rows" (see tile_gemm.hip).
+#pragma once
+
+#include "mellin_common.hpp"
+#include "tile_gemm.hpp"
+
+namespace mellin {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+
+typedef __attribute__((address_space(3))) float *lds_float_ptr;
+
+// One dword per active lane from `src` (per-lane address) straight to LDS at
+// `row` + 4 * lane id; `row` must be wave-uniform.  Completion is counted by
+// vmcnt.  Written as inline assembly on purpose: the compiler then does not
+// order later LDS reads after these loads, which is what lets the loads of the
+// next stage stay in flight during the matrix loop; every consumer waits
+// explicitly (wait_all_memory + barrier).  m0 carries the LDS base.
+__device__ __forceinline__ void load_to_lds(const float *src, float *row) {
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_float_ptr)row);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :: "s"(lds_addr), "v"(src) : "memory");
+}
+
+__device__ __forceinline__ void wait_all_memory() {
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+}
+
+// Signal row chosen by (output row, filter row) on a Mellin axis, in 32-bit
+// arithmetic (the plan guarantees that the products fit).  p1 = p + 1.
+__device__ __forceinline__ int mellin_tap32(int kind, int h, int f, int ng, int s, int d, int p1, int u) {
+  int num, den;
+  if (kind == AX_MCORR) { num = (h + s) * (f + d); den = p1; }
+  else { num = p1 * (h + s); den = f + d; }
+  const int q = num / den;
+  if (q * den != num) return -1;
+  const int g = q - u;
+  return (g >= 0 && g < ng) ? g : -1;
+}
+
+// n / d and n % d for 0 <= n < 2^22, d >= 1, without an integer divide.
+struct FastDiv {
+  int d;
+  float inv;
+  __device__ explicit FastDiv(int d_) : d(d_), inv(1.0f / (float)d_) {}
+  __device__ __forceinline__ void divmod(int n, int &q, int &r) const {
+    q = (int)((float)n * inv);
+    r = n - q * d;
+    if (r < 0) { --q; r += d; }
+    else if (r >= d) { ++q; r -= d; }
+  }
+};
+
+// Uniform description of one position tile.
+struct TileGeom {
+  int n, q0, count, ox_lo, oy_lo, R_tile, RSL, vx_min, vy_min;
+};
+
+template <int P>
+__device__ __forceinline__ TileGeom tile_geometry(const TilePlan &pl, int tile_id, bool mellin_x) {
+  TileGeom g;
+  g.n = tile_id / pl.tiles_per_image;
+  const int tile = tile_id - g.n * pl.tiles_per_image;
+  int ox_hi, oy_hi;
+  if (pl.segment) {
+    g.ox_lo = ox_hi = tile / pl.chunks_per_row;
+    g.oy_lo = (tile - g.ox_lo * pl.chunks_per_row) * P;
+    g.count = min(P, pl.noy - g.oy_lo);
+    oy_hi = g.oy_lo + g.count - 1;
+    g.q0 = g.ox_lo * pl.noy + g.oy_lo;
+  } else {
+    g.q0 = tile * P;
+    g.count = min(P, pl.Q - g.q0);
+    g.ox_lo = g.q0 / pl.noy;
+    ox_hi = (g.q0 + g.count - 1) / pl.noy;
+    g.oy_lo = 0;
+    oy_hi = pl.noy - 1;
+  }
+  const int rows = ox_hi - g.ox_lo + 1;
+  g.R_tile = mellin_x ? rows * pl.nfx : pl.ax * (rows - 1) + pl.bx_span + 1;
+  g.vx_min = pl.ax * g.ox_lo + pl.cx + pl.bx_min;         // linear x only
+  g.vy_min = pl.ay * g.oy_lo + pl.cy + pl.by_min;
+  g.RSL = pl.ay * (oy_hi - g.oy_lo) + pl.by_span + 1;     // staged columns
+  return g;
+}
+
+
+// ---- signal rows of one (tile, channel range) --------------------------------
+// wave w owns virtual rows w, w + 4, ...; 64 lanes first work out the source of
+// 64 such rows, then one direct load per row is issued with the lanes on
+// columns; columns or rows without a source are written as zeros.
+__device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom &tg,
+                                             const float *__restrict__ G, int c0, int cc,
+                                             float *Gs, bool mellin_x, int lane, int wave) {
+  const int total_rows = cc * tg.R_tile;
+  const float *Gimg = G + (i64)tg.n * pl.g_n + (i64)c0 * pl.g_c;
+  const int g_c = (int)pl.g_c;                         // fits: c_in * ngx * ngy < 2^31
+  const FastDiv by_rows(tg.R_tile), by_nfx(pl.nfx);
+  for (int base = 0; base < total_rows; base += 64 * kWaves) {
+    // per-lane: row base + 4 * lane + wave
+    const int rr = base + kWaves * lane + wave;
+    int src_off = -1, dst_off = 0;
+    if (rr < total_rows) {
+      int cl, r;
+      by_rows.divmod(rr, cl, r);
+      int gx = -1;
+      if (mellin_x) {
+        int oxl, fx;
+        by_nfx.divmod(r, oxl, fx);
+        gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
+      } else {
+        const int vx = tg.vx_min + r;
+        if (vx >= 0) {
+          if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
+          else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
+        }
+      }
+      if (gx >= 0) src_off = cl * g_c + gx * pl.ngy;
+      dst_off = (cl * pl.R + r) * pl.RS;
+    }
+    const int mine = min(64, (total_rows - base - wave + kWaves - 1) / kWaves);
+    for (int cb = 0; cb < tg.RSL; cb += 64) {
+      const int col = cb + lane;
+      const int vy = tg.vy_min + col;
+      int gy = -1;
+      if (col < tg.RSL && vy >= 0) {
+        if (pl.uy == 1) gy = vy;
+        else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
+        if (gy >= pl.ngy) gy = -1;
+      }
+      for (int j = 0; j < mine; ++j) {
+        const int s_src = __builtin_amdgcn_readlane(src_off, j);
+        const int s_dst = __builtin_amdgcn_readlane(dst_off, j);
+        float *row = Gs + s_dst + cb;
+        if (s_src >= 0 && gy >= 0) load_to_lds(Gimg + s_src + gy, row);
+        else if (col < tg.RSL) row[lane] = 0.f;
+      }
+    }
+  }
+}
+
+}  // namespace mellin

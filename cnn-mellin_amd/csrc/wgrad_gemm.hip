@@ -1,0 +1,314 @@
+// Weight gradient on the fp32 matrix cores.
+//
+//   W[m, (c, fx, fy)] = sum_{n, ox, oy} A[n, m, ox, oy] *
+//                       G[n, c, tap_x(ox, fx), tap_y(oy, fy)]
+//
+// (A = grad_out, G = layer input) is a (M x positions) * (positions x J)
+// product, J = c_in * nfx * nfy, whose long dimension is the reduction.  The
+// reduction is split over persistent workgroups in a FIXED way: workgroup s
+// takes position tiles s, s + S, ... of the same (image, position) tiling the
+// forward kernel uses, each wavefront a quarter of every tile, and keeps its
+// MT x JT accumulator tiles in registers for its whole life.  At the end the
+// four wavefronts are summed through LDS in wave order, the workgroup writes
+// one partial block to the workspace, and a second kernel adds the S partials
+// in index order.  No floating-point atomics: the result is bit-reproducible.
+//
+// Operands are staged exactly as in the forward kernel (direct global->LDS
+// loads, two buffers): the input as affine "virtual rows", so that the B
+// operand of lane (column j) at position q is the LDS word
+// col_offset[j] + pos_offset[q], and grad_out as one dense row of P positions
+// per output channel (the A operand).
+#include <algorithm>
+
+#include "mellin_common.hpp"
+#include "tile_gemm.hpp"
+#include "tile_stage.hpp"
+
+namespace mellin {
+
+namespace {
+
+template <int MT, int JT, int NT>
+__global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
+    WgradPlan wp, const float *__restrict__ A, const float *__restrict__ G,
+    float *__restrict__ ws) {
+  extern __shared__ float lds[];
+  const TilePlan &pl = wp.t;
+  constexpr int M_T = MT * 32, J_T = JT * 32;
+  constexpr int PW = NT * 32;                        // positions per wavefront and tile
+  constexpr int P = kWaves * PW;
+  constexpr int GS = 4;                              // position pairs per operand group
+  const int x_words = wp.CCj * pl.R * pl.RS;
+  const int a_words = M_T * wp.GSS;
+  float *Xs0 = lds;                                  // [2][CCj][R][RS]
+  float *As0 = Xs0 + 2 * x_words;                    // [2][M_T][GSS]
+  int *posoff0 = (int *)(As0 + 2 * a_words);         // [2][P]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+
+  // block of the output this workgroup owns
+  const int mg = blockIdx.y / wp.j_groups, jg = blockIdx.y - mg * wp.j_groups;
+  const int m0 = mg * M_T, j0 = jg * J_T;
+  const int c_lo = j0 / pl.nf;
+  const int j_last = min(wp.J, j0 + J_T) - 1;
+  const int ccj = j_last / pl.nf - c_lo + 1;
+
+  // LDS word of column j's tap relative to a position's base (constant per lane)
+  int col_off[JT];
+  {
+    const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
+#pragma unroll
+    for (int t = 0; t < JT; ++t) {
+      const int j = min(j0 + t * 32 + l32, wp.J - 1);   // columns past J are computed but never stored
+      int c, tt, fx, fy;
+      by_nf.divmod(j, c, tt);
+      by_nfy.divmod(tt, fx, fy);
+      col_off[t] = (c - c_lo) * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+    }
+  }
+
+  const FastDiv by_noy(pl.noy);
+  const int my_tiles = (int)blockIdx.x < pl.total_tiles
+                           ? (pl.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+
+  auto issue_stage = [&](int ti) {
+    const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
+    const int b = ti & 1;
+    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, mellin_x, lane, wave);
+    // grad_out rows: P consecutive positions per output channel, zeros past the tile
+    const float *An = A + (i64)tg.n * wp.a_n + tg.q0;
+    float *As = As0 + b * a_words;
+    for (int m = wave; m < M_T; m += kWaves) {
+      const bool mv = m0 + m < pl.M;
+      const float *src = An + (i64)(m0 + (mv ? m : 0)) * wp.a_m;
+      for (int pb = 0; pb < P; pb += 64) {
+        float *row = As + m * wp.GSS + pb;
+        if (mv && pb + lane < tg.count) load_to_lds(src + pb + lane, row);
+        else row[lane] = 0.f;
+      }
+    }
+    // LDS word of every position's (fx = 0, fy = 0) tap
+    int *posoff = posoff0 + b * P;
+    for (int p = tid; p < P; p += kThreads) {
+      const int q = tg.q0 + (p < tg.count ? p : 0);       // past the tile: any valid position
+      int ox, oy;
+      by_noy.divmod(q, ox, oy);
+      posoff[p] = (pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min;
+    }
+  };
+
+  floatx16 acc[MT][JT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
+
+  if (my_tiles > 0) issue_stage(0);
+
+  for (int ti = 0; ti < my_tiles; ++ti) {
+    wait_all_memory();
+    __syncthreads();
+    if (ti + 1 < my_tiles) issue_stage(ti + 1);
+
+    const int tile_id = blockIdx.x + ti * gridDim.x;
+    const int n = tile_id / pl.tiles_per_image, tile = tile_id - n * pl.tiles_per_image;
+    int count;
+    if (pl.segment) count = min(P, pl.noy - (tile % pl.chunks_per_row) * P);
+    else count = min(P, pl.Q - tile * P);
+    const int cnt_w = max(0, min(PW, count - wave * PW));  // this wavefront's live positions
+    const int steps = (cnt_w + 1) >> 1;
+    const int full = cnt_w >> 1;                           // pairs with both positions live
+
+    const float *Xs = Xs0 + (ti & 1) * x_words;
+    const float *ap = As0 + (ti & 1) * a_words + l32 * wp.GSS + wave * PW + half;
+    const int *pp = posoff0 + (ti & 1) * P + wave * PW + half;
+    const int arow = 32 * wp.GSS;
+    const int groups = full / GS;
+    float a0[GS][MT], b0[GS][JT], a1[GS][MT], b1[GS][JT];
+    auto fetch = [&](int g, float (&a)[GS][MT], float (&b)[GS][JT]) {
+      int po[GS];
+#pragma unroll
+      for (int k = 0; k < GS; ++k) po[k] = pp[2 * (g * GS + k)];
+#pragma unroll
+      for (int k = 0; k < GS; ++k) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a[k][i] = ap[2 * (g * GS + k) + i * arow];
+#pragma unroll
+        for (int t = 0; t < JT; ++t) b[k][t] = Xs[col_off[t] + po[k]];
+      }
+    };
+    auto multiply = [&](float (&a)[GS][MT], float (&b)[GS][JT]) {
+#pragma unroll
+      for (int k = 0; k < GS; ++k)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int t = 0; t < JT; ++t)
+            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[k][i], b[k][t], acc[i][t], 0, 0, 0);
+    };
+    int g = 0;
+    if (groups > 0) fetch(0, a0, b0);
+    for (; g + 1 < groups; g += 2) {
+      fetch(g + 1, a1, b1);
+      multiply(a0, b0);
+      if (g + 2 < groups) fetch(g + 2, a0, b0);
+      multiply(a1, b1);
+    }
+    if (g < groups) multiply(a0, b0);
+    for (int s = groups * GS; s < steps; ++s) {
+      const int po = pp[2 * s];
+      float a[MT], b[JT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) a[i] = ap[2 * s + i * arow];
+      // the odd last position of a tile multiplies a zero of grad_out; force the
+      // other operand to zero as well so that a non-finite input cannot leak in
+#pragma unroll
+      for (int t = 0; t < JT; ++t) b[t] = (s >= full && half) ? 0.f : Xs[col_off[t] + po];
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < JT; ++t)
+          acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+    }
+  }
+
+  // ---- sum the four wavefronts in wave order, then write the partial block ------
+  __syncthreads();
+  float *red = lds;                                   // [M_T][J_T]
+  for (int w = 0; w < kWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < JT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float *dst = red + m * J_T + t * 32 + l32;
+            if (w == 0) *dst = acc[i][t][r];
+            else *dst += acc[i][t][r];
+          }
+    }
+    __syncthreads();
+  }
+  float *out = ws + (i64)blockIdx.x * wp.M_pad * wp.J_pad + (i64)m0 * wp.J_pad + j0;
+  for (int e = tid; e < M_T * J_T; e += kThreads) {
+    const int m = e / J_T, jj = e - m * J_T;
+    out[(i64)m * wp.J_pad + jj] = red[e];
+  }
+}
+
+// W[m, j] = sum over the S partial blocks, in index order.  A block of 256
+// threads handles 16 outputs: 16 threads per output add every 16th partial,
+// then thread 0 of each output adds the 16 sums in order.
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ ws,
+                                                           float *__restrict__ W, int S, int M,
+                                                           int J, int M_pad, int J_pad) {
+  __shared__ float part[16][17];
+  const int el = threadIdx.x & 15, ph = threadIdx.x >> 4;
+  const int e = blockIdx.x * 16 + el;
+  float sum = 0.f;
+  if (e < M * J) {
+    const int m = e / J, j = e - m * J;
+    const float *src = ws + (i64)m * J_pad + j;
+    const i64 stride = (i64)M_pad * J_pad;
+    int s = ph;
+    for (; s + 48 < S; s += 64) {
+      const float v0 = src[(i64)s * stride], v1 = src[(i64)(s + 16) * stride];
+      const float v2 = src[(i64)(s + 32) * stride], v3 = src[(i64)(s + 48) * stride];
+      sum += v0; sum += v1; sum += v2; sum += v3;
+    }
+    for (; s < S; s += 16) sum += src[(i64)s * stride];
+  }
+  part[ph][el] = sum;
+  __syncthreads();
+  if (ph == 0 && e < M * J) {
+    float tot = part[0][el];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) tot += part[k][el];
+    W[e] = tot;
+  }
+}
+
+template <int MT, int JT, int NT>
+hipError_t launch_variant(const WgradPlan &wp, size_t lds_bytes, dim3 grid, const float *a,
+                          const float *g, float *ws, hipStream_t stream) {
+  auto kern = wgrad_gemm_kernel<MT, JT, NT>;
+  if (lds_bytes > 64 * 1024) {
+    static thread_local size_t granted = 0;
+    if (granted < lds_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds_bytes);
+      if (e != hipSuccess) return e;
+      granted = lds_bytes;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, wp, a, g, ws);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+// Plan the weight gradient of the layer whose FORWARD problem is `fwd`
+// (filter = weight, signal = input, output = grad_out, write mode).
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp) {
+  size_t lds_fwd;
+  int mt, nt;
+  // 128 positions per tile: the staged grad_out tile (channels x positions, two
+  // buffers) is what fills LDS here
+  if (!make_tile_plan(fwd, wp.t, &lds_fwd, &mt, &nt, 1)) return false;
+  TilePlan &pl = wp.t;
+  wp.J = pl.C * pl.nf;
+  wp.mt = 1;
+  wp.jt = wp.J > 64 ? 3 : (wp.J > 32 ? 2 : 1);
+  const int M_T = wp.mt * 32, J_T = wp.jt * 32;
+  wp.m_groups = (pl.M + M_T - 1) / M_T;
+  wp.j_groups = (wp.J + J_T - 1) / J_T;
+  wp.M_pad = wp.m_groups * M_T;
+  wp.J_pad = wp.j_groups * J_T;
+  wp.a_n = (i64)pl.M * pl.Q;
+  wp.a_m = pl.Q;
+  // the forward plan fixed the position tiling (nt) and the row geometry
+  wp.nt = nt;
+  const int P = kWaves * nt * 32;
+  wp.GSS = P + 1;
+  wp.CCj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
+  const size_t words = 2 * (size_t)wp.CCj * pl.R * pl.RS + 2 * (size_t)M_T * wp.GSS + 2 * (size_t)P;
+  const size_t red_words = (size_t)M_T * J_T;
+  wp.lds_bytes = 4 * std::max(words, red_words);
+  if (wp.lds_bytes > 96 * 1024) return false;
+  // position shares: persistent workgroups, at most two per CU over all output blocks
+  const int blocks_y = wp.m_groups * wp.j_groups;
+  int per_cu = (int)((160 * 1024) / (wp.lds_bytes + 512));
+  per_cu = std::max(1, std::min(per_cu, 2));
+  int S = std::max(1, (256 * per_cu) / blocks_y);
+  S = std::min(S, pl.total_tiles);
+  wp.S = S;
+  wp.ws_bytes = (size_t)S * wp.M_pad * wp.J_pad * sizeof(float);
+  return true;
+}
+
+hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float *input,
+                        float *grad_weight, float *workspace, hipStream_t stream) {
+  dim3 grid((unsigned)wp.S, (unsigned)(wp.m_groups * wp.j_groups));
+  hipError_t e = hipErrorInvalidValue;
+#define MELLIN_WGRAD_CASE(MT_, JT_, NT_)                                                   \
+  if (wp.mt == MT_ && wp.jt == JT_ && wp.nt == NT_)                                          \
+    e = launch_variant<MT_, JT_, NT_>(wp, wp.lds_bytes, grid, grad_out, input, workspace, stream);
+  MELLIN_WGRAD_CASE(1, 3, 1)
+  MELLIN_WGRAD_CASE(1, 2, 1)
+  MELLIN_WGRAD_CASE(1, 1, 1)
+#undef MELLIN_WGRAD_CASE
+  if (e != hipSuccess) return e;
+  const int outputs = wp.t.M * wp.J;
+  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((outputs + 15) / 16)), dim3(256), 0, stream,
+                     (const float *)workspace, grad_weight, wp.S, wp.t.M, wp.J, wp.M_pad, wp.J_pad);
+  return hipGetLastError();
+}
+
+}  // namespace mellin
