@@ -85,6 +85,9 @@ class Layer:
         nbytes = hip.lib.mellin_corr2d_backward_weight_workspace(kind_x, 4, *self.dims)
         self.ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
         self.ws_bytes = nbytes
+        nbytes = hip.lib.mellin_corr2d_backward_input_workspace(kind_x, 4, *self.dims)
+        self.ws_in = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        self.ws_in_bytes = nbytes
         self.bytes_per_pass = pass_bytes_flops(self.nhx, self.nhy)
         self.macs_per_pass = count_macs(kind_x, self.nhx, self.nhy)
 
@@ -94,7 +97,8 @@ class Layer:
 
     def backward_input(self):
         import _mellin_hip as hip
-        hip.corr2d_backward_input(self.kind_x, self.w, self.go, self.gi, self.dims)
+        hip.corr2d_backward_input(self.kind_x, self.w, self.go, self.gi, self.dims,
+                                  workspace=self.ws_in, workspace_bytes=self.ws_in_bytes)
 
     def backward_weight(self):
         import _mellin_hip as hip

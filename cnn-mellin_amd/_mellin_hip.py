@@ -39,6 +39,7 @@ SYMBOLS = {
     "mellin_last_variant": (ctypes.c_char_p, []),
     "mellin_set_variant": (_int, [ctypes.c_char_p]),
     "mellin_corr2d_backward_weight_workspace": (_size_t, [_int, _int] + _DIMS),
+    "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
 }
 for _t in ("f32", "f64"):
     for _n in ("mcorr1d", "mconv1d"):
@@ -46,7 +47,8 @@ for _t in ("f32", "f64"):
     for _n in ("mcorrlcorr", "mconvlconv", "lcorrlcorr", "lconvlconv"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC2D)
     SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
-    SYMBOLS["mellin_corr2d_backward_input_" + _t] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
+    SYMBOLS["mellin_corr2d_backward_input_" + _t] = (
+        _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
     SYMBOLS["mellin_corr2d_backward_weight_" + _t] = (
         _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 
@@ -135,11 +137,26 @@ def corr2d_forward(kind_x, input, weight, bias, out, dims):
     return out
 
 
-def corr2d_backward_input(kind_x, weight, grad_out, grad_input, dims):
+def _workspace(kind_x, which, out, dims, workspace, workspace_bytes):
+    if workspace is None:
+        query = getattr(lib, "mellin_corr2d_backward_%s_workspace" % which)
+        workspace_bytes = query(kind_x, out.element_size(), *dims)
+        workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=out.device)
+                     if workspace_bytes else None)
+    return workspace, workspace_bytes
+
+
+def corr2d_backward_input(kind_x, weight, grad_out, grad_input, dims, workspace=None,
+                          workspace_bytes=None):
+    """Input gradient; scratch memory comes from `workspace` or, if None, from torch's
+    caching allocator on the launch stream."""
     dev = require_device(weight, grad_out, grad_input)
+    workspace, workspace_bytes = _workspace(kind_x, "input", grad_input, dims, workspace,
+                                            workspace_bytes)
     fn = getattr(lib, "mellin_corr2d_backward_input_" + suffix(grad_input.dtype))
     with torch.cuda.device(dev):
-        _check(fn(kind_x, _dp(weight), _dp(grad_out), *dims, _dp(grad_input), _stream(dev)))
+        _check(fn(kind_x, _dp(weight), _dp(grad_out), *dims, _dp(grad_input),
+                  _dp(workspace), workspace_bytes, _stream(dev)))
     return grad_input
 
 
@@ -148,13 +165,9 @@ def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims, workspace
     """Weight gradient; scratch memory comes from `workspace` or, if None, from torch's
     caching allocator on the launch stream."""
     dev = require_device(input, grad_out, grad_weight)
-    suf = suffix(grad_weight.dtype)
-    if workspace is None:
-        workspace_bytes = lib.mellin_corr2d_backward_weight_workspace(
-            kind_x, grad_weight.element_size(), *dims)
-        workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=dev)
-                     if workspace_bytes else None)
-    fn = getattr(lib, "mellin_corr2d_backward_weight_" + suf)
+    workspace, workspace_bytes = _workspace(kind_x, "weight", grad_weight, dims, workspace,
+                                            workspace_bytes)
+    fn = getattr(lib, "mellin_corr2d_backward_weight_" + suffix(grad_weight.dtype))
     with torch.cuda.device(dev):
         _check(fn(kind_x, _dp(input), _dp(grad_out), *dims, _dp(grad_weight),
                   _dp(workspace), workspace_bytes, _stream(dev)))

@@ -168,12 +168,52 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
 //   x (Mellin): hx = (p + 1)(gx + u)/(fx + d) - s
 //   x (linear): hx = (u gx - d fx + p)/s
 //   y (linear): hy = (u gy - d fy + p)/s
+// Two-pass input gradient for layers with few input channels.  With c_in output
+// channels the matrix-core tile would be mostly padding, so the first pass runs
+// the gather-GEMM over the y axis only, with one output channel per
+// (input channel, filter row) pair, into a workspace
+//   Y[n, ci * nfx + fx, hx, gy] = sum_{co, fy} weight[co, ci, fx, fy] * grad_out[n, co, hx, .]
+// and the second pass (fold_x.hip) adds the filter rows whose x tap exists.
+struct TwoPassInput {
+  TilePlan plan;
+  size_t lds, ws_bytes;
+  int mt, nt;
+  Axis fold;
+};
+
+bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
+                         i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px,
+                         i64 py, i64 ux, i64 uy, TwoPassInput &tp) {
+  (void)sx;
+  const i64 m2 = c_in * nfx;
+  // worth it when c_in alone would leave most of a 32-row tile empty and the
+  // (c_in, filter row) pairs fill tiles reasonably
+  if (c_in >= 16 || nfx < 2) return false;
+  const i64 pad = ((m2 + 31) / 32) * 32;
+  if (pad * 2 > m2 * 3) return false;
+  const i64 nf = nfx * nfy, nh = nhx * nhy;
+  SepConv pr;
+  pr.x = make_axis(AX_LCORR, 1, nhx, nhx, 1, 1, 0, 1);                 // rows pass through
+  pr.y = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
+  pr.batch = batch; pr.c_out = m2; pr.c_in = c_out;
+  pr.f_m = nfy; pr.f_c = c_in * nf;
+  pr.g_n = c_out * nh; pr.g_c = nh;
+  pr.h_n = m2 * nhx * ngy; pr.h_m = nhx * ngy;
+  pr.accumulate = 0;
+  if (!make_tile_plan(pr, tp.plan, &tp.lds, &tp.mt, &tp.nt)) return false;
+  const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
+  tp.fold = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
+  tp.ws_bytes = (size_t)(batch * m2 * nhx * ngy) * sizeof(float);
+  return true;
+}
+
 template <typename T>
 int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
                           const T *grad_out, i64 batch, i64 c_in, i64 c_out,
                           i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy,
                           i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux,
-                          i64 uy, T *grad_input, void *stream) {
+                          i64 uy, T *grad_input, void *workspace, size_t workspace_bytes,
+                          void *stream) {
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
@@ -181,8 +221,25 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   if (batch * c_in * ng == 0) return MELLIN_OK;
   if (!grad_input || (c_out * nf * nh != 0 && (!weight || !grad_out)))
     return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  SepConv pr;
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
+  if (sizeof(T) == 4 && g_forced != 1 && c_out * nf * nh != 0) {
+    TwoPassInput tp;
+    if (plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy,
+                            dx, dy, px, py, ux, uy, tp)) {
+      if (!workspace || workspace_bytes < tp.ws_bytes)
+        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
+                    tp.ws_bytes, workspace_bytes);
+      g_variant = "mfma+fold";
+      hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight,
+                                      (const float *)grad_out, nullptr, (float *)workspace,
+                                      (hipStream_t)stream);
+      if (e == hipSuccess)
+        e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)workspace,
+                          (float *)grad_input, (hipStream_t)stream);
+      return check_hip(e, fn);
+    }
+  }
+  SepConv pr;
   // roles: "signal" = grad_out (length nh), "output" = grad_input (length ng)
   pr.x = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
   pr.y = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
@@ -235,6 +292,10 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
 
 }  // namespace
 
+#define CORR2D_ARGS                                                            \
+  batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
+  ux, uy
+
 extern "C" {
 
 int mellin_version(void) { return 100; }
@@ -278,10 +339,6 @@ DEFINE_2D(mellin_lcorrlcorr_f64, double, AX_LCORR, AX_LCORR)
 DEFINE_2D(mellin_lconvlconv_f32, float, AX_LCONV, AX_LCONV)
 DEFINE_2D(mellin_lconvlconv_f64, double, AX_LCONV, AX_LCONV)
 
-#define CORR2D_ARGS                                                            \
-  batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
-  ux, uy
-
 int mellin_corr2d_forward_f32(int kind_x, const float *input, const float *weight,
                               const float *bias, MELLIN_CORR2D_DIMS, float *out,
                               void *stream) {
@@ -292,15 +349,28 @@ int mellin_corr2d_forward_f64(int kind_x, const double *input, const double *wei
                               void *stream) {
   return corr2d_forward<double>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream);
 }
+size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
+                                              MELLIN_CORR2D_DIMS) {
+  if (elem_bytes != 4 || g_forced == 1) return 0;
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
+  TwoPassInput tp;
+  if (!plan_two_pass_input(kind_x, CORR2D_ARGS, tp)) return 0;
+  return tp.ws_bytes;
+}
 int mellin_corr2d_backward_input_f32(int kind_x, const float *weight,
                                      const float *grad_out, MELLIN_CORR2D_DIMS,
-                                     float *grad_input, void *stream) {
-  return corr2d_backward_input<float>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input, stream);
+                                     float *grad_input, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return corr2d_backward_input<float>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input,
+                                      workspace, workspace_bytes, stream);
 }
 int mellin_corr2d_backward_input_f64(int kind_x, const double *weight,
                                      const double *grad_out, MELLIN_CORR2D_DIMS,
-                                     double *grad_input, void *stream) {
-  return corr2d_backward_input<double>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input, stream);
+                                     double *grad_input, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return corr2d_backward_input<double>(__func__, kind_x, weight, grad_out, CORR2D_ARGS, grad_input,
+                                       workspace, workspace_bytes, stream);
 }
 size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
                                                MELLIN_CORR2D_DIMS) {

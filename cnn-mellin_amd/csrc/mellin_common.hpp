@@ -87,4 +87,7 @@ template <typename T>
 hipError_t launch_sepreduce_generic(const SepReduce &pr, const T *a, const T *g,
                                     T *w, hipStream_t stream);
 
+hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
+                         float *grad_input, hipStream_t stream);
+
 }  // namespace mellin

@@ -118,10 +118,12 @@ MELLIN_DECL_2D(mellin_lconvlconv_f64, double);
  * kind_x is MELLIN_AXIS_MCORR or MELLIN_AXIS_LCORR.  1-D layers pass a unit
  * y axis (nfy = ngy = nhy = 1, sy = dy = uy = 1, py = 0).
  *
- * backward_weight needs scratch memory for partial sums: ask
- * mellin_corr2d_backward_weight_workspace() for the byte count and pass a
- * device buffer of at least that size (256-byte aligned); its contents on
- * entry do not matter and are garbage on exit.
+ * The backward passes may need scratch memory (partial sums of the weight
+ * gradient; the intermediate of the two-pass input gradient used for layers
+ * with few input channels): ask mellin_corr2d_backward_*_workspace() for the
+ * byte count (0 = none) and pass a device buffer of at least that size
+ * (256-byte aligned); its contents on entry do not matter and are garbage on
+ * exit.
  * ------------------------------------------------------------------------ */
 #define MELLIN_CORR2D_DIMS                                                     \
   int64_t batch, int64_t c_in, int64_t c_out, int64_t nfx, int64_t nfy,        \
@@ -135,12 +137,16 @@ int mellin_corr2d_forward_f64(int kind_x, const double *input,
                               const double *weight, const double *bias,
                               MELLIN_CORR2D_DIMS, double *out, void *stream);
 
+size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
+                                              MELLIN_CORR2D_DIMS);
 int mellin_corr2d_backward_input_f32(int kind_x, const float *weight,
                                      const float *grad_out, MELLIN_CORR2D_DIMS,
-                                     float *grad_input, void *stream);
+                                     float *grad_input, void *workspace,
+                                     size_t workspace_bytes, void *stream);
 int mellin_corr2d_backward_input_f64(int kind_x, const double *weight,
                                      const double *grad_out, MELLIN_CORR2D_DIMS,
-                                     double *grad_input, void *stream);
+                                     double *grad_input, void *workspace,
+                                     size_t workspace_bytes, void *stream);
 
 size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
                                                MELLIN_CORR2D_DIMS);
