@@ -160,7 +160,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--variant", default=None, help="force a kernel variant (e.g. generic)")
-    ap.add_argument("--cpu-slice", type=int, default=8, help="utterances in the CPU baseline sample")
+    ap.add_argument("--cpu-slice", type=int, default=32, help="utterances in the CPU baseline sample")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain device copy of known size (to scale profiler byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (got --gpus %d)" % args.gpus)
@@ -171,6 +173,16 @@ def main():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        # 256 MiB read + 256 MiB written per launch, ten launches
+        src = torch.randn(64 * 1024 * 1024, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4,
+                          "launches": 10}))
+        return
     hip.set_variant(args.variant)
     gen = torch.Generator().manual_seed(2)
     layers = [Layer(hip.AX_MCORR, "mconv2d", gen, dev), Layer(hip.AX_LCORR, "lconv2d", gen, dev)]
