@@ -43,6 +43,7 @@ namespace {
 
 #ifndef MELLIN_STAMP
 #define MELLIN_STAMP(i)
+#define MELLIN_PROBE_DECL
 #endif
 
 template <int MT, int NT, bool ACC>
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   int *tapoff = (int *)(Ws0 + (single_chunk ? 1 : 2) * w_words);   // [KCp]
   float *Bs = (float *)(tapoff + pl.KCp);            // [M_T] bias (zeros when accumulating)
 
+  MELLIN_PROBE_DECL
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
@@ -74,15 +76,18 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   auto issue_filter = [&](int c0, int cc, float *Ws) {
     const int KC = cc * pl.nf;
     const FastDiv by_nf(pl.nf);
+    const int m_live = max(0, min(M_T, pl.M - m0));       // channels of this block that exist
     for (int kb = 0; kb < pl.KCp; kb += 64) {
       const int k = kb + lane;
       int cl, t;
       by_nf.divmod(k, cl, t);
-      const float *Fk = F + (i64)(c0 + cl) * pl.f_c + t;
-      for (int m = wave; m < M_T; m += kWaves) {
-        float *row = Ws + m * pl.WSS + kb;
-        if (k < KC && m0 + m < pl.M) load_to_lds(Fk + (i64)(m0 + m) * pl.f_m, row);
-        else if (k < pl.KCp) row[lane] = 0.f;
+      const unsigned voff = (unsigned)(((i64)(c0 + cl) * pl.f_c + t) * 4);   // < 4 GB: checked by the plan
+      if (k < KC) {
+        for (int m = wave; m < m_live; m += kWaves)
+          load_to_lds(F + (i64)(m0 + m) * pl.f_m, voff, Ws + m * pl.WSS + kb);
+        for (int m = m_live + wave; m < M_T; m += kWaves) Ws[m * pl.WSS + k] = 0.f;
+      } else if (k < pl.KCp) {
+        for (int m = wave; m < M_T; m += kWaves) Ws[m * pl.WSS + k] = 0.f;
       }
     }
   };
@@ -348,6 +353,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     if (hmax * fmax >= lim || (X.p + 1) * hmax >= lim) return false;
   }
   if (Q >= ((i64)1 << 22) || pr.c_in * ng >= lim) return false;   // float-reciprocal index splits
+  if (pr.c_in * pr.f_c + nf >= lim || pr.f_c < 0 || pr.f_m < 0) return false;   // 32-bit byte offsets into the filter
   pl.R = (int)R;
   pl.RS = (int)RSL | 1;                                            // odd stride spreads LDS banks
 
@@ -383,7 +389,7 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   // persistent workgroups: as many as fit at once (by LDS, two per CU at most) on the 256 CUs
   const int m_tiles = (pl.M + M_T - 1) / M_T;
   int per_cu = (int)((160 * 1024) / (lds_bytes + 512));
-  per_cu = std::max(1, std::min(per_cu, 2));
+  per_cu = std::max(1, std::min(per_cu, nt == 2 ? 3 : 4));
   int gx = std::max(1, (256 * per_cu) / m_tiles);
   gx = std::min(gx, pl.total_tiles);
   dim3 grid((unsigned)gx, (unsigned)m_tiles);

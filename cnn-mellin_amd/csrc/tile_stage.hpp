@@ -15,16 +15,21 @@ constexpr int kThreads = kWaves * 64;
 
 typedef __attribute__((address_space(3))) float *lds_float_ptr;
 
-// One dword per active lane from `src` (per-lane address) straight to LDS at
-// `row` + 4 * lane id; `row` must be wave-uniform.  Completion is counted by
+// One dword per active lane straight from global memory to LDS: lane l reads
+// the dword at `base` + `byte_offset` (base wave-uniform, offset per lane) and
+// it lands at `row` + 4 * l (`row` wave-uniform).  Completion is counted by
 // vmcnt.  Written as inline assembly on purpose: the compiler then does not
 // order later LDS reads after these loads, which is what lets the loads of the
 // next stage stay in flight during the matrix loop; every consumer waits
 // explicitly (wait_all_memory + barrier).  m0 carries the LDS base.
-__device__ __forceinline__ void load_to_lds(const float *src, float *row) {
+__device__ __forceinline__ void load_to_lds(const float *base, unsigned byte_offset, float *row) {
   const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_float_ptr)row);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-               :: "s"(lds_addr), "v"(src) : "memory");
+  const unsigned long long b = (unsigned long long)base;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_addr), "v"(byte_offset), "s"(sbase) : "memory");
 }
 
 __device__ __forceinline__ void wait_all_memory() {
@@ -127,18 +132,31 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
     for (int cb = 0; cb < tg.RSL; cb += 64) {
       const int col = cb + lane;
       const int vy = tg.vy_min + col;
+      const bool in_row = col < tg.RSL;
       int gy = -1;
-      if (col < tg.RSL && vy >= 0) {
+      if (in_row && vy >= 0) {
         if (pl.uy == 1) gy = vy;
         else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
         if (gy >= pl.ngy) gy = -1;
       }
-      for (int j = 0; j < mine; ++j) {
-        const int s_src = __builtin_amdgcn_readlane(src_off, j);
-        const int s_dst = __builtin_amdgcn_readlane(dst_off, j);
-        float *row = Gs + s_dst + cb;
-        if (s_src >= 0 && gy >= 0) load_to_lds(Gimg + s_src + gy, row);
-        else if (col < tg.RSL) row[lane] = 0.f;
+      // lanes whose column has a source: one load per row that has a source
+      if (gy >= 0) {
+        const unsigned voff = (unsigned)gy * 4u;
+        for (int j = 0; j < mine; ++j) {
+          const int s_src = __builtin_amdgcn_readlane(src_off, j);
+          if (s_src >= 0) {
+            const int s_dst = __builtin_amdgcn_readlane(dst_off, j);
+            load_to_lds(Gimg + s_src, voff, Gs + s_dst + cb);
+          }
+        }
+      }
+      // zeros: padding columns of every row, and whole rows without a source
+      if (in_row) {
+        const bool pad_col = gy < 0;
+        for (int j = 0; j < mine; ++j) {
+          const int s_src = __builtin_amdgcn_readlane(src_off, j);
+          if (pad_col || s_src < 0) Gs[__builtin_amdgcn_readlane(dst_off, j) + col] = 0.f;
+        }
       }
     }
   }

@@ -81,13 +81,15 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
     // grad_out rows: P consecutive positions per output channel, zeros past the tile
     const float *An = A + (i64)tg.n * wp.a_n + tg.q0;
     float *As = As0 + b * a_words;
-    for (int m = wave; m < M_T; m += kWaves) {
-      const bool mv = m0 + m < pl.M;
-      const float *src = An + (i64)(m0 + (mv ? m : 0)) * wp.a_m;
-      for (int pb = 0; pb < P; pb += 64) {
-        float *row = As + m * wp.GSS + pb;
-        if (mv && pb + lane < tg.count) load_to_lds(src + pb + lane, row);
-        else row[lane] = 0.f;
+    const int m_live = min(M_T, pl.M - m0);
+    for (int pb = 0; pb < P; pb += 64) {
+      const int p = pb + lane;
+      if (p < tg.count) {
+        for (int m = wave; m < m_live; m += kWaves)
+          load_to_lds(An + (i64)(m0 + m) * wp.a_m, (unsigned)p * 4u, As + m * wp.GSS + pb);
+        for (int m = max(m_live, 0) + wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
+      } else {
+        for (int m = wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
       }
     }
     // LDS word of every position's (fx = 0, fy = 0) tap
