@@ -6,6 +6,7 @@
 
 #include "../../include/mellin_hip.h"
 #include "mellin_common.hpp"
+#include "igrad_gemm.hpp"
 #include "tile_gemm.hpp"
 
 using namespace mellin;
@@ -14,7 +15,7 @@ namespace {
 
 thread_local char g_error[512] = "";
 thread_local const char *g_variant = "";
-thread_local int g_forced = 0;   // 0 automatic, 1 generic
+thread_local int g_forced = 0;   // 0 automatic, 1 generic, 2 automatic without the fused input gradient
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -222,6 +223,15 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   if (!grad_input || (c_out * nf * nh != 0 && (!weight || !grad_out)))
     return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
+  if (sizeof(T) == 4 && g_forced == 0 && c_out * nf * nh != 0) {
+    IgradPlan ip;
+    if (make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
+                        px, py, ux, uy, ip)) {
+      g_variant = "mfma-fused";
+      return check_hip(launch_igrad(ip, (const float *)weight, (const float *)grad_out,
+                                    (float *)grad_input, (hipStream_t)stream), fn);
+    }
+  }
   if (sizeof(T) == 4 && g_forced != 1 && c_out * nf * nh != 0) {
     TwoPassInput tp;
     if (plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy,
@@ -308,6 +318,7 @@ int mellin_set_variant(const char *name) {
   if (!name || !*name) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
   if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
+  if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }
   return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
 }
 
@@ -354,6 +365,8 @@ size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
   if (elem_bytes != 4 || g_forced == 1) return 0;
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
+  IgradPlan ip;
+  if (g_forced == 0 && make_igrad_plan(kind_x, CORR2D_ARGS, ip)) return 0;
   TwoPassInput tp;
   if (!plan_two_pass_input(kind_x, CORR2D_ARGS, tp)) return 0;
   return tp.ws_bytes;

@@ -1,0 +1,38 @@
+// Descriptor of the fused input-gradient kernel for layers with few input
+// channels and a linear x axis (igrad_gemm.hip).
+#pragma once
+
+#include "mellin_common.hpp"
+
+namespace mellin {
+
+struct IgradPlan {
+  // problem: forward layer out[n, co, hx, hy] = sum w[co, ci, fx, fy] *
+  // in[n, ci, sx hx + dx fx - px, sy hy + dy fy - py]   (ux = uy = 1)
+  int batch, c_in, c_out;
+  int nfx, nfy, nf;
+  int nhx, nhy, nh;                // grad_out extent and nhx * nhy
+  int ngx, ngy;                    // grad_input extent
+  int sx, dx, px, sy, dy, py;
+  // blocking
+  int mtn;                         // 32-tap tiles per input channel
+  int units;                       // c_in * mtn: wavefronts per workgroup
+  int ksteps;                      // (c_out rounded up) / 2: template instance
+  int nt;                          // 32-position tiles per chunk: template instance
+  int T, strips;                   // grad_input rows per workgroup; workgroups per image
+  int Rp, Wp;                      // accumulator plane: rows and row length (words)
+  int batched_fold;                // taps with congruent matrix rows never share a word: fold them in batches
+  size_t lds_bytes;
+};
+
+// force_nt / force_T (0 = automatic) pin the chunk width and the strip height.
+// False when the layer does not suit the kernel (Mellin x axis, ux or uy != 1,
+// too many channels, planes that do not fit in LDS, sizes beyond 32-bit indexing).
+bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
+                     i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
+                     i64 ux, i64 uy, IgradPlan &pl, int force_nt = 0, int force_T = 0);
+
+hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
+                        float *grad_input, hipStream_t stream);
+
+}  // namespace mellin

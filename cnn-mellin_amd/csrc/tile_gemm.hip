@@ -260,6 +260,7 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
     MELLIN_STAMP(6);
   }
   if (my_stages > 0) epilogue();
+  MELLIN_STAMP(9);
 }
 
 template <int MT, int NT, bool ACC>

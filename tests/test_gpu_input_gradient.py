@@ -1,0 +1,105 @@
+"""Input gradient of layers with few input channels: the fused matrix-core
+kernel (linear x axis) and the two-pass path must both agree with the CPU
+checker, and with each other, through the C ABI.
+
+Tolerance: rtol 1e-5 / atol 1e-5 * sqrt(fan_in) against the float64 checker.
+"""
+import numpy as np
+import pytest
+import torch
+
+import _mellin_hip as hip
+from _gpu import assert_close, to_gpu
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _grad_input(kind_x, w, go, in_shape, s, d, p, u, variant):
+    """grad_input of the correlation layer through mellin_corr2d_backward_input_f32."""
+    n, c_in, ngx, ngy = in_shape
+    c_out, _, nfx, nfy = w.shape
+    nhx, nhy = go.shape[2:]
+    dims = hip._dims(n, c_in, c_out, (nfx, nfy), (ngx, ngy), (nhx, nhy), s, d, p, u)
+    gi = torch.full(in_shape, float("nan"), dtype=torch.float32, device="cuda")   # every word must be written
+    hip.set_variant(variant)
+    try:
+        hip.corr2d_backward_input(kind_x, to_gpu(w), to_gpu(go), gi, dims)
+        return gi, hip.last_variant()
+    finally:
+        hip.set_variant(None)
+
+
+def _expected(x_shape, w, go, s, d, p, u):
+    x = np.zeros(x_shape, dtype=np.float64)
+    gi, _, _ = oracle.lcorrlcorr_backward(x, w.astype(np.float64), go.astype(np.float64), s, d, p, u)
+    return gi
+
+
+CASES = [
+    # (n, c_in, c_out, nf, ng, s, d, p, r)   r: output rows/cols beyond the valid size
+    (2, 3, 64, (8, 4), (70, 41), (1, 1), (1, 1), (0, 0), (0, 0)),      # the benchmark layer, shortened
+    (3, 1, 7, (5, 5), (33, 29), (1, 1), (1, 1), (2, 1), (0, 0)),       # one input channel, padding
+    (2, 2, 33, (6, 4), (50, 20), (2, 1), (1, 2), (1, 0), (0, 0)),      # stride in x, dilation in y
+    (1, 4, 100, (4, 7), (41, 37), (1, 3), (2, 1), (3, 2), (0, 0)),     # c_out past 64, stride in y, dilation in x
+    (2, 3, 128, (7, 8), (64, 30), (3, 2), (2, 2), (0, 3), (0, 0)),     # two tap tiles per channel
+    (2, 5, 16, (3, 9), (25, 45), (1, 1), (3, 1), (1, 1), (2, 1)),      # outputs past the valid size
+    (1, 2, 5, (30, 1), (200, 1), (1, 1), (1, 1), (0, 0), (0, 0)),      # 1-D layer, long filter
+    (2, 3, 64, (8, 4), (9, 6), (1, 1), (1, 1), (0, 0), (0, 0)),        # image barely larger than the filter
+    (1, 1, 1, (6, 4), (300, 11), (4, 1), (1, 1), (5, 0), (0, 0)),      # stride larger than the strips' overlap
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_fused_and_two_pass_match_checker(case):
+    n, c_in, c_out, nf, ng, s, d, p, r = case
+    u = (1, 1)
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    nh = tuple(oracle.lcorr_valid_size(nf[i], ng[i], s[i], d[i], p[i], u[i]) + r[i] for i in range(2))
+    assert min(nh) > 0
+    w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    exp = _expected((n, c_in) + ng, w, go, s, d, p, u)
+    fan_in = c_out * nf[0] * nf[1]
+    fused, v1 = _grad_input(hip.AX_LCORR, w, go, (n, c_in) + ng, s, d, p, u, None)
+    assert v1 == "mfma-fused", v1
+    assert_close(fused, exp, fan_in, "fused %s" % (case,))
+    other, v2 = _grad_input(hip.AX_LCORR, w, go, (n, c_in) + ng, s, d, p, u, "two-pass")
+    assert v2 != "mfma-fused", v2
+    assert_close(other, exp, fan_in, "%s %s" % (v2, case))
+
+
+def test_fused_random_sweep():
+    rng = np.random.default_rng(77)
+    fused_seen = 0
+    for trial in range(40):
+        n, c_in = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+        c_out = int(rng.choice([1, 3, 20, 32, 40, 64, 65, 128]))
+        nf = (int(rng.integers(2, 9)), int(rng.integers(2, 9)))
+        ng = (int(rng.integers(nf[0], 90)), int(rng.integers(nf[1], 60)))
+        s = tuple(int(v) for v in rng.integers(1, 4, 2))
+        d = tuple(int(v) for v in rng.integers(1, 3, 2))
+        p = tuple(int(v) for v in rng.integers(0, 4, 2))
+        u = (1, 1)
+        nh = tuple(oracle.lcorr_valid_size(nf[i], ng[i], s[i], d[i], p[i], u[i]) for i in range(2))
+        if min(nh) <= 0:
+            continue
+        w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+        go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+        exp = _expected((n, c_in) + ng, w, go, s, d, p, u)
+        got, v = _grad_input(hip.AX_LCORR, w, go, (n, c_in) + ng, s, d, p, u, None)
+        fused_seen += v == "mfma-fused"
+        assert_close(got, exp, c_out * nf[0] * nf[1], "trial %d %s nf=%s ng=%s s=%s d=%s p=%s c=%d->%d" %
+                     (trial, v, nf, ng, s, d, p, c_in, c_out))
+    assert fused_seen >= 10, fused_seen
+
+
+def test_fused_is_run_to_run_deterministic():
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((64, 3, 8, 4)).astype(np.float32)
+    go = rng.standard_normal((4, 64, 121, 38)).astype(np.float32)
+    first, v = _grad_input(hip.AX_LCORR, w, go, (4, 3, 128, 41), (1, 1), (1, 1), (0, 0), (1, 1), None)
+    assert v == "mfma-fused"
+    for _ in range(3):
+        again, _ = _grad_input(hip.AX_LCORR, w, go, (4, 3, 128, 41), (1, 1), (1, 1), (0, 0), (1, 1), None)
+        assert torch.equal(first, again)
