@@ -227,9 +227,12 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
     IgradPlan ip;
     if (make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
                         px, py, ux, uy, ip)) {
+      if (ip.ws_bytes && (!workspace || workspace_bytes < ip.ws_bytes))
+        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
+                    ip.ws_bytes, workspace_bytes);
       g_variant = "mfma-fused";
       return check_hip(launch_igrad(ip, (const float *)weight, (const float *)grad_out,
-                                    (float *)grad_input, (hipStream_t)stream), fn);
+                                    (float *)grad_input, (float *)workspace, (hipStream_t)stream), fn);
     }
   }
   if (sizeof(T) == 4 && g_forced != 1 && c_out * nf * nh != 0) {
@@ -366,7 +369,7 @@ size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
   IgradPlan ip;
-  if (g_forced == 0 && make_igrad_plan(kind_x, CORR2D_ARGS, ip)) return 0;
+  if (g_forced == 0 && make_igrad_plan(kind_x, CORR2D_ARGS, ip)) return ip.ws_bytes;
   TwoPassInput tp;
   if (!plan_two_pass_input(kind_x, CORR2D_ARGS, tp)) return 0;
   return tp.ws_bytes;

@@ -15,20 +15,22 @@
 // grad_out as it lies in memory (no gather, no padding), and every element of
 // Z belongs to exactly one grad_input element, at (sx hx + dx fx - px,
 // sy hy + dy fy - py).  Z never leaves the chip: each wavefront adds its
-// accumulator tile straight into an LDS image of the grad_input rows its
-// workgroup owns.
+// accumulator tile straight into an LDS image ("plane") of the grad_input rows
+// its workgroup can reach.
 //
-// Work split: one workgroup per (image, strip of T grad_input rows).  It walks
-// the grad_out rows that have a tap in the strip, 32 * NT positions at a time
-// (two LDS buffers filled by direct global->LDS loads, the next chunk in flight
-// while this one multiplies).  One wavefront per (input channel, 32-tap tile):
-// its filter operand stays in registers for the whole kernel, and it alone
-// adds into its own LDS plane, in program order, so the result does not depend
-// on scheduling (no two wavefronts ever add to the same word; lanes of one
-// instruction that share a word are ordered by the hardware).  Rows of the
-// plane above and below the strip catch the taps that fall outside it: the
-// neighbouring strips recompute those.  At the end the planes of one input
-// channel are summed in tile order and written out, coalesced along gy.
+// Work split: one workgroup per (image, strip of Th grad_out rows), so every
+// grad_out element is read and multiplied once.  The strip is walked 32 * NT
+// positions at a time: all channels of the chunk are copied to LDS by direct
+// global->LDS loads (16 bytes per lane), then multiplied.  The buffer is single:
+// several small workgroups share a CU and cover each other's load latency.
+// One wavefront per (input channel, 32-tap tile): its filter operand stays in
+// registers for the whole kernel, and it alone adds into its own plane, in
+// program order, so the result does not depend on scheduling.
+//
+// A grad_input row whose taps all come from one strip is written by that
+// strip's workgroup.  The few rows fed by two neighbouring strips (dx (nfx - 1)
+// - sx + 1 rows per boundary) are written as two partial rows into a small
+// workspace and summed, upper strip first, by a second kernel.
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
@@ -40,34 +42,68 @@ namespace mellin {
 
 namespace {
 
-template <int KSTEPS, int NT>
-__global__ __launch_bounds__(512) void igrad_kernel(const IgradPlan pl, const float *__restrict__ W,
+// Strips [lo, hi] that feed grad_input row gx: the strips of the first and last
+// grad_out rows hx with sx hx + dx fx - px = gx for some fx in [0, nfx), clamped
+// to the rows that exist.  lo == hi for most rows; hi == lo + 1 next to a
+// strip boundary (the plan keeps strips taller than a filter's reach).  A row
+// that nothing feeds belongs to the strip of the last grad_out row before it.
+struct StripMap {
+  FastDiv by_sx, by_th;
+  int px, reach, sx, H;
+  __device__ explicit StripMap(const IgradPlan &pl)
+      : by_sx(pl.sx), by_th(pl.Th), px(pl.px), reach(pl.dx * (pl.nfx - 1)), sx(pl.sx), H(pl.H) {}
+  __device__ __forceinline__ void feeding(int gx, int &lo, int &hi) const {
+    int q, r;
+    const int a0 = gx + px - reach;                    // ceil(a0 / sx), clamped below at 0
+    int h0 = 0;
+    if (a0 > 0) { by_sx.divmod(a0 + sx - 1, q, r); h0 = q; }
+    by_sx.divmod(gx + px, q, r);                       // gx + px >= 0
+    int h1 = q;
+    h0 = min(h0, H - 1);
+    h1 = min(h1, H - 1);
+    if (h0 > h1) h0 = h1;                              // no row feeds gx (stride wider than the reach)
+    by_th.divmod(h0, lo, r);
+    by_th.divmod(h1, hi, r);
+  }
+};
+
+// Up to twelve wavefronts per workgroup (168 registers each) wherever the instance can live with that.
+template <int KSTEPS, int NT, bool PIPE>
+__global__ __launch_bounds__((KSTEPS * NT <= 128 ? 768 : 512)) void igrad_kernel(const IgradPlan pl, const float *__restrict__ W,
                                                     const float *__restrict__ GO,
-                                                    float *__restrict__ GI) {
+                                                    float *__restrict__ GI, float *__restrict__ WS) {
   extern __shared__ __align__(16) float lds[];
   constexpr int K = 2 * KSTEPS, P = NT * 32;
-  float *Bs0 = lds;                                    // [2][K][P] grad_out chunk, channel-major
-  float *planes = lds + 2 * K * P;                     // [units][Rp][Wp]
+  constexpr int BW = PIPE ? K * 96 : K * P;            // words of the chunk buffer
 
-  const int tid = threadIdx.x, nthreads = blockDim.x;
+  // A workgroup runs pl.jobs independent (image, strip) jobs side by side, one
+  // group of pl.units wavefronts each with its own slice of LDS: same strip,
+  // consecutive images, hence the same trip counts and barriers.  That makes the
+  // wavefront count a multiple of four (all four SIMDs of a CU equally loaded).
+  const int job = (int)(threadIdx.x >> 6) / pl.units;
+  const int tid = threadIdx.x - job * pl.units * 64, nthreads = pl.units * 64;
   const int lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
-  const int n = blockIdx.x / pl.strips, strip = blockIdx.x - n * pl.strips;
-  const int a = strip * pl.T, b = min(a + pl.T, pl.ngx);      // grad_input rows [a, b)
-
-  // grad_out rows hx with sx hx + dx fx - px inside [a, b) for some fx
-  const int reach = pl.dx * (pl.nfx - 1);
-  int hx_lo = a + pl.px - reach;
-  hx_lo = hx_lo > 0 ? (hx_lo + pl.sx - 1) / pl.sx : 0;
-  int hx_hi = b - 1 + pl.px;
-  hx_hi = hx_hi >= 0 ? min(pl.nhx - 1, hx_hi / pl.sx) : -1;
-  const int q_lo = hx_lo * pl.nhy, q_end = (hx_hi + 1) * pl.nhy;
-  const int nchunks = hx_hi >= hx_lo ? (q_end - q_lo + P - 1) / P : 0;
+  const int image_group = blockIdx.x / pl.strips, strip = blockIdx.x - image_group * pl.strips;
+  const int n_want = image_group * pl.jobs + job;
+  const bool active = n_want < pl.batch;               // a job past the last image only keeps the barriers
+  const int n = active ? n_want : pl.batch - 1;
+  const int ha = strip * pl.Th, hb = min(ha + pl.Th, pl.H);    // grad_out rows [ha, hb)
+  const int q_lo = ha * pl.nhy, q_end = hb * pl.nhy;
+  const int nchunks = (q_end - q_lo + P - 1) / P;
   const int plane_words = pl.Rp * pl.Wp;
+  float *job_lds = lds + job * (((BW + pl.units * plane_words) + 3) & ~3);
+  float *Bs = job_lds;                                 // grad_out chunk buffer, channel-major
+  float *planes = job_lds + BW;                        // [units][Rp][Wp]
 
   for (int i = tid; i < pl.units * plane_words; i += nthreads) planes[i] = 0.f;
-  // rows past c_out and lanes past the image are never loaded: keep them finite
-  for (int i = tid; i < 2 * K * P; i += nthreads) Bs0[i] = 0.f;
+  // channels past c_out are never loaded, nor are positions past the end of the
+  // image: keep what the multiply loop reads there finite
+  if (PIPE || q_lo + nchunks * P > pl.nh) {
+    for (int i = tid; i < BW; i += nthreads) Bs[i] = 0.f;
+  } else {
+    for (int i = pl.c_out * P + tid; i < BW; i += nthreads) Bs[i] = 0.f;
+  }
 
   // filter operand of this wavefront: A[tap m = l32][k = 2 s + half] = w[k, ci, m]
   const int ci = wave / pl.mtn, mt = wave - ci * pl.mtn;
@@ -81,142 +117,324 @@ __global__ __launch_bounds__(512) void igrad_kernel(const IgradPlan pl, const fl
     }
   }
   // accumulator register r of this lane holds tap m(r); its offset in the plane
+  // (-1: a matrix row past the last tap)
   int off[16];
+  {
+    const FastDiv by_nfy(pl.nfy);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int m = mt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-    const int fx = m / pl.nfy, fy = m - fx * pl.nfy;
-    off[r] = m < pl.nf ? pl.dx * fx * pl.Wp + pl.dy * fy : -1;
+    for (int r = 0; r < 16; ++r) {
+      const int m = mt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+      int fx, fy;
+      by_nfy.divmod(m, fx, fy);
+      off[r] = m < pl.nf ? pl.dx * fx * pl.Wp + pl.dy * fy : -1;
+    }
   }
   float *plane = planes + wave * plane_words;
   const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
   const FastDiv by_nhy(pl.nhy);
 
-  // Chunk c: channel k's P positions go to words [k * P, (k + 1) * P) of a buffer.
+  // Chunk c: channel k's P positions go to words [k * P, (k + 1) * P) of the buffer.
   // Odd channels are stored with every pair of 32-position halves exchanged, so
   // the two half-waves of the multiply loop (channels 2 s and 2 s + 1) read
   // disjoint banks.  Away from the end of the image one instruction moves
   // 16 bytes per lane: 1024 / (4 P) whole channels.
   constexpr int LPR = P / 4;                           // lanes per channel row
   constexpr int RPI = 64 / LPR;                        // channel rows per instruction
+  constexpr int KH = K / 2;                            // channels per half of the buffer
   const int row_in = lane / LPR, seg = lane - row_in * LPR;
-  auto issue = [&](int c) {
-    float *Bs = Bs0 + (c & 1) * K * P;
+  const unsigned bs_addr = lds_address(Bs);
+  auto issue = [&](int c, int k_lo) {                  // channels [k_lo, k_lo + KH) of chunk c
     const int q0 = q_lo + c * P;
+    const int k_hi = min(k_lo + KH, pl.c_out);
     if (q0 + P <= pl.nh) {
-      for (int k0 = wave * RPI; k0 < pl.c_out; k0 += pl.units * RPI) {
+      for (int k0 = k_lo + wave * RPI; k0 < k_hi; k0 += pl.units * RPI) {
         const int k = k0 + row_in;
         const unsigned voff = (unsigned)(row_in * pl.nh + q0 + 4 * (seg ^ ((k & 1) << 3))) * 4u;
-        if (k < pl.c_out) load16_to_lds(GOn + (i64)k0 * pl.nh, voff, Bs + k0 * P);
+        if (k < k_hi) load16_to_lds_at(GOn + (i64)k0 * pl.nh, voff, bs_addr + 4u * (unsigned)(k0 * P));
       }
     } else {
-      for (int k = wave; k < pl.c_out; k += pl.units)
+      for (int k = k_lo + wave; k < k_hi; k += pl.units)
 #pragma unroll
         for (int t2 = 0; t2 < P; t2 += 64) {
           const int q = q0 + t2 + (lane ^ ((k & 1) << 5));
-          if (q < pl.nh) load_to_lds(GOn + (i64)k * pl.nh, (unsigned)q * 4u, Bs + k * P + t2);
+          if (q < pl.nh) load_to_lds_at(GOn + (i64)k * pl.nh, (unsigned)q * 4u, bs_addr + 4u * (unsigned)(k * P + t2));
         }
     }
   };
 
-  __syncthreads();
-  if (nchunks > 0) issue(0);
+  // The buffer is single, but its two channel halves are refilled separately:
+  // as soon as every wavefront has multiplied a half, the same half of the next
+  // chunk is requested, so the loads fly during the other half's multiplies
+  // and the fold.
+  // this lane's channel of step s is 2 s + half; odd channels hold 32-position
+  // tile t where tile t ^ 1 would be
+  int bo[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) bo[t] = half * P + ((t ^ half) << 5) + l32;
+  // fold: Z[m, position] joins grad_input word base(position) + off(m), by plain
+  // read-add-write (this wavefront owns the plane).  The 32 lanes of a half-wave
+  // hold one tap at 32 different positions: never the same word.  Registers r
+  // with the same r % 4 (and the two half-waves) hold different taps; when the
+  // plan has shown that those cannot meet either, they go as one batch.
+  auto fold = [&](auto padded_rows, int c, const floatx16 (&acc)[NT]) {
+    constexpr bool kPadded = decltype(padded_rows)::value;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int rel = c * P + t * 32 + l32;              // position counted from q_lo
+      int hxr, hy;
+      by_nhy.divmod(rel, hxr, hy);
+      float *dst = plane + pl.sx * hxr * pl.Wp + pl.sy * hy;
+      if (q_lo + rel < q_end) {
+        if (pl.batched_fold) {
+#pragma unroll
+          for (int c4 = 0; c4 < 4; ++c4) {
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (!kPadded || off[4 * j + c4] >= 0) v[j] = dst[off[4 * j + c4]];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (!kPadded || off[4 * j + c4] >= 0) dst[off[4 * j + c4]] = v[j] + acc[t][4 * j + c4];
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            // one half-wave at a time; the wave barriers keep the two phases apart
+            if (half == 0 && (!kPadded || off[r] >= 0)) dst[off[r]] += acc[t][r];
+            __builtin_amdgcn_wave_barrier();
+            if (half == 1 && (!kPadded || off[r] >= 0)) dst[off[r]] += acc[t][r];
+            __builtin_amdgcn_wave_barrier();
+          }
+        }
+      }
+    }
+  };
+
+  if constexpr (PIPE) {
+    // Batched fold and every matrix row a tap: positions stream through in tiles
+    // of 32.  Tile p lives in block p % 3 of the buffer ([3][K][32] words); the
+    // block of tile p - 1 is refilled with tile p + 2 as soon as every wavefront
+    // has multiplied it, two tile phases before it is needed.  The fold of tile
+    // p - 1 is cut into its four batches and spread between the multiplies of
+    // tile p, so its LDS round trips hide behind the matrix pipe.
+    constexpr int NBUF = 3, SPB = KSTEPS / 4;            // multiply steps per fold batch
+    const int ntiles = (q_end - q_lo + 31) / 32;
+    const int row8 = lane >> 3, seg8 = lane & 7;         // 8 lanes x 16 bytes per channel row
+    auto issue_tile = [&](int p) {
+      const int q0 = q_lo + p * 32;
+      const unsigned blk = bs_addr + 4u * (unsigned)((p % NBUF) * K * 32);
+      if (q0 + 32 <= pl.nh) {
+        for (int k0 = wave * 8; k0 < pl.c_out; k0 += pl.units * 8) {
+          const unsigned voff = (unsigned)(row8 * pl.nh + q0 + 4 * seg8) * 4u;
+          if (k0 + row8 < pl.c_out) load16_to_lds_at(GOn + (i64)k0 * pl.nh, voff, blk + 4u * (unsigned)(k0 * 32));
+        }
+      } else {
+        for (int k = wave; k < pl.c_out; k += pl.units)
+          if (lane < 32 && q0 + lane < pl.nh)
+            load_to_lds_at(GOn + (i64)k * pl.nh, (unsigned)(q0 + lane) * 4u, blk + 4u * (unsigned)(k * 32));
+      }
+    };
+    floatx16 acc0, acc1;
+    const int bsrc = half * 32 + l32;                    // this lane's word of channel pair s: + 64 s
+    auto tile = [&](auto has_prev, int p, floatx16 &cur, const floatx16 &prev) {
+      constexpr bool kPrev = decltype(has_prev)::value;
+      int dprev = 0;                                     // plane word of tile p - 1's position
+      if (kPrev) {
+        int hxr, hy;
+        by_nhy.divmod((p - 1) * 32 + l32, hxr, hy);
+        dprev = pl.sx * hxr * pl.Wp + pl.sy * hy;
+      }
+      wait_all_memory();
+      __syncthreads();               // tile p has landed for every wavefront; the block of tile p - 1 is free
+      if (p >= 1 && p + 2 < ntiles) issue_tile(p + 2);
+      const float *blk = Bs + (p % NBUF) * K * 32 + bsrc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) cur[r] = 0.f;
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        float v[4];
+        if (kPrev) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = plane[dprev + off[4 * j + c4]];
+        }
+#pragma unroll
+        for (int s = c4 * SPB; s < (c4 + 1) * SPB; ++s)
+          cur = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], blk[64 * s], cur, 0, 0, 0);
+        if (kPrev) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) plane[dprev + off[4 * j + c4]] = v[j] + prev[4 * j + c4];
+        }
+      }
+    };
+    __syncthreads();                                     // zeroes are in place
+    issue_tile(0);
+    if (ntiles > 1) issue_tile(1);
+    if (ntiles > 2) issue_tile(2);
+    tile(std::false_type(), 0, acc0, acc1);
+    int p = 1;
+    for (; p + 1 < ntiles; p += 2) {
+      tile(std::true_type(), p, acc1, acc0);
+      tile(std::true_type(), p + 1, acc0, acc1);
+    }
+    if (p < ntiles) {
+      tile(std::true_type(), p, acc1, acc0);
+      acc0 = acc1;
+      ++p;
+    }
+    // the last tile: not every position need exist
+    {
+      const int rel = (p - 1) * 32 + l32;
+      int hxr, hy;
+      by_nhy.divmod(rel, hxr, hy);
+      const int d = pl.sx * hxr * pl.Wp + pl.sy * hy;
+      if (q_lo + rel < q_end) {
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4) {
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = plane[d + off[4 * j + c4]];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) plane[d + off[4 * j + c4]] = v[j] + acc0[4 * j + c4];
+        }
+      }
+    }
+  } else {
+  __syncthreads();                                     // zeroes are in place
+  issue(0, 0);
+  issue(0, KH);
   for (int c = 0; c < nchunks; ++c) {
-    // chunk c has landed for every wavefront, and nobody still reads the other buffer
     wait_all_memory();
-    __syncthreads();
-    if (c + 1 < nchunks) issue(c + 1);
+    __syncthreads();                                   // chunk c has landed for every wavefront
 
     floatx16 acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
-    // this lane's channel of step s is 2 s + half; odd channels hold 32-position
-    // tile t where tile t ^ 1 would be
-    const float *Bs[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) Bs[t] = Bs0 + (c & 1) * K * P + half * P + ((t ^ half) << 5) + l32;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s)
+    for (int s = 0; s < KSTEPS / 2; ++s)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[t][2 * s * P], acc[t], 0, 0, 0);
-
-    // fold: Z[m, position] joins grad_input word base(position) + off(m), by plain
-    // read-add-write (this wavefront owns the plane).  The 32 lanes of a half-wave
-    // hold one tap at 32 different positions: never the same word.  Registers r
-    // with the same r % 4 (and the two half-waves) hold different taps; when the
-    // plan has shown that those cannot meet either, they go as one batch.
-    // Matrix rows past the last tap (off < 0) hold zeros and must not touch the plane.
-    auto fold = [&](auto padded_rows) {
-      constexpr bool kPadded = decltype(padded_rows)::value;
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
+    __syncthreads();                                   // the first half is free
+    if (c + 1 < nchunks) issue(c + 1, 0);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const int rel = c * P + t * 32 + l32;              // position counted from q_lo
-        int hxr, hy;
-        by_nhy.divmod(rel, hxr, hy);
-        float *dst = plane + pl.sx * hxr * pl.Wp + pl.sy * hy;
-        if (q_lo + rel < q_end) {
-          if (pl.batched_fold) {
+    for (int s = KSTEPS / 2; s < KSTEPS; ++s)
 #pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-              float v[4];
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if (!kPadded || off[4 * j + c4] >= 0) v[j] = dst[off[4 * j + c4]];
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if (!kPadded || off[4 * j + c4] >= 0) dst[off[4 * j + c4]] = v[j] + acc[t][4 * j + c4];
-            }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              // one half-wave at a time; the wave barriers keep the two phases apart
-              if (half == 0 && (!kPadded || off[r] >= 0)) dst[off[r]] += acc[t][r];
-              __builtin_amdgcn_wave_barrier();
-              if (half == 1 && (!kPadded || off[r] >= 0)) dst[off[r]] += acc[t][r];
-              __builtin_amdgcn_wave_barrier();
-            }
-          }
-        }
-      }
-    };
-    if ((pl.nf & 31) == 0) fold(std::false_type());
-    else fold(std::true_type());
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
+    __syncthreads();                                   // the second half is free
+    if (c + 1 < nchunks) issue(c + 1, KH);
+    if ((pl.nf & 31) == 0) fold(std::false_type(), c, acc);
+    else fold(std::true_type(), c, acc);
+  }
   }
   __syncthreads();
 
-  // write the strip: plane row i is grad_input row g_lo + i, plane column j is gy = j - py
-  const int rows = b - a;
-  const int g_lo = pl.sx * hx_lo - pl.px;
-  const int total = pl.c_in * rows * pl.ngy;
-  const FastDiv by_ngy(pl.ngy), by_rows(rows);
-  for (int i = tid; i < total; i += nthreads) {
-    int r2, gy, cc, gxr;
-    by_ngy.divmod(i, r2, gy);
-    by_rows.divmod(r2, cc, gxr);
-    const int pi = a + gxr - g_lo, pj = gy + pl.py;
-    float v = 0.f;
-    if (nchunks > 0 && pi >= 0 && pi < pl.Rp && pj >= 0 && pj < pl.Wp) {
-      const float *src = planes + cc * pl.mtn * plane_words + pi * pl.Wp + pj;
-      for (int m2 = 0; m2 < pl.mtn; ++m2) v += src[m2 * plane_words];
+  // Write the rows this strip feeds: plane row i is grad_input row g0 + i, plane
+  // column j is gy = j - py.  First, one thread per plane row works out where the
+  // row goes: -1 nowhere (another strip owns it, or it lies outside grad_input),
+  // 2 gx straight to grad_input, or 2 (slot index) + 1 a partial row in the workspace.
+  // Rows between the reach of this strip and the first row of the next one (a
+  // stride wider than the filter) are nobody's: they get zeros from here too.
+  const int g0 = pl.sx * ha - pl.px;
+  const int rp_t = max(pl.Rp, pl.sx * pl.Th);
+  int *row_dst = (int *)Bs;                            // the chunk buffer is free now
+  const StripMap map(pl);
+  for (int pi = tid; pi < rp_t; pi += nthreads) {
+    const int gx = g0 + pi;
+    int code = -1;
+    if (gx >= 0 && gx < pl.ngx) {
+      int s_lo, s_hi;
+      map.feeding(gx, s_lo, s_hi);
+      if (s_lo == s_hi) {
+        if (s_lo == strip) code = 2 * gx;
+      } else if (strip == s_lo || strip == s_hi) {
+        // boundary s_hi, row number within the boundary's shared rows, upper or lower strip
+        const int r = gx - (pl.sx * s_hi * pl.Th - pl.px);
+        code = 2 * (((s_hi - 1) * pl.nshared + r) * 2 + (strip - s_lo)) + 1;
+      }
     }
-    GI[((i64)(n * pl.c_in + cc) * pl.ngx + a + gxr) * pl.ngy + gy] = v;
+    row_dst[pi] = code;
+  }
+  __syncthreads();
+  {
+    const int row_words = rp_t * pl.ngy;
+    const FastDiv by_ngy(pl.ngy), by_rp(rp_t);
+    const i64 nc0 = (i64)n * pl.c_in;
+    for (int i = tid; i < pl.c_in * row_words; i += nthreads) {
+      int r2, gy, cc, pi;
+      by_ngy.divmod(i, r2, gy);
+      by_rp.divmod(r2, cc, pi);
+      const int code = row_dst[pi];
+      if (code < 0 || !active) continue;
+      float v = 0.f;
+      if (pi < pl.Rp && gy + pl.py < pl.Wp) {
+        const float *src = planes + cc * pl.mtn * plane_words + pi * pl.Wp + pl.py + gy;
+        for (int m2 = 0; m2 < pl.mtn; ++m2) v += src[m2 * plane_words];
+      }
+      if (code & 1)
+        WS[((nc0 + cc) * (pl.strips - 1) * pl.nshared * 2 + (code >> 1)) * pl.ngy + gy] = v;
+      else
+        GI[((nc0 + cc) * pl.ngx + (code >> 1)) * pl.ngy + gy] = v;
+    }
+  }
+  // grad_input rows past the reach of the last grad_out row belong to the last strip: zeros
+  if (strip == pl.strips - 1 && active) {
+    const int z0 = max(0, g0 + rp_t);
+    const int zrows = pl.ngx - z0;
+    if (zrows > 0) {
+      const i64 per_c = (i64)zrows * pl.ngy;
+      for (i64 i = tid; i < pl.c_in * per_c; i += nthreads) {
+        const i64 cc = i / per_c, w = i - cc * per_c;
+        GI[(((i64)n * pl.c_in + cc) * pl.ngx + z0) * pl.ngy + w] = 0.f;
+      }
+    }
   }
 }
 
-template <int KSTEPS, int NT>
+// grad_input rows next to a strip boundary: upper strip's partial + lower strip's.
+// One workgroup per (boundary, image * c_in + channel) sums that boundary's rows.
+__global__ __launch_bounds__(256) void igrad_combine_kernel(const IgradPlan pl,
+                                                            const float *__restrict__ WS,
+                                                            float *__restrict__ GI) {
+  const int b = blockIdx.x + 1;                        // boundary between strips b - 1 and b
+  const i64 nc = blockIdx.y;
+  const int g_b = pl.sx * b * pl.Th - pl.px;           // first row the boundary can share
+  const float *src = WS + ((nc * (pl.strips - 1) + (b - 1)) * pl.nshared * 2) * pl.ngy;
+  float *out = GI + nc * pl.ngx * pl.ngy;
+  const StripMap map(pl);
+  const FastDiv by_ngy(pl.ngy);
+  for (int i = threadIdx.x; i < pl.nshared * pl.ngy; i += blockDim.x) {
+    int r, gy;
+    by_ngy.divmod(i, r, gy);
+    const int gx = g_b + r;
+    if (gx < 0 || gx >= pl.ngx) continue;
+    int s_lo, s_hi;
+    map.feeding(gx, s_lo, s_hi);
+    if (s_lo == s_hi) continue;                        // not shared after clamping: written directly
+    const float *p = src + (i64)r * 2 * pl.ngy + gy;
+    out[(i64)gx * pl.ngy + gy] = p[0] + p[pl.ngy];
+  }
+}
+
+template <int KSTEPS, int NT, bool PIPE>
 hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go, float *gi,
-                           hipStream_t stream) {
-  auto kern = igrad_kernel<KSTEPS, NT>;
+                           float *ws, hipStream_t stream) {
+  auto kern = igrad_kernel<KSTEPS, NT, PIPE>;
   if (pl.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)pl.lds_bytes);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(pl.batch * pl.strips)), dim3(64 * pl.units),
-                     pl.lds_bytes, stream, pl, w, go, gi);
+  const int groups = (pl.batch + pl.jobs - 1) / pl.jobs;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(groups * pl.strips)), dim3(64 * pl.units * pl.jobs),
+                     pl.lds_bytes, stream, pl, w, go, gi, ws);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || pl.ws_bytes == 0) return e;
+  hipLaunchKernelGGL(igrad_combine_kernel,
+                     dim3((unsigned)(pl.strips - 1), (unsigned)(pl.batch * pl.c_in)), dim3(256), 0,
+                     stream, pl, ws, gi);
   return hipGetLastError();
 }
 
@@ -224,14 +442,13 @@ hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go,
 
 bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                      i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
-                     i64 ux, i64 uy, IgradPlan &pl, int force_nt, int force_T) {
+                     i64 ux, i64 uy, IgradPlan &pl, int force_nt, int force_Th, int force_pipe) {
   if (kind_x != AX_LCORR || ux != 1 || uy != 1) return false;
   if (px < 0 || py < 0) return false;
   const i64 nf = nfx * nfy, nh = nhx * nhy, ng = ngx * ngy;
   if (batch < 1 || c_in < 1 || c_out < 1 || nf < 1 || nh < 1 || ng < 1) return false;
   const i64 lim = (i64)1 << 28;
-  if (batch * c_out * nh / nh != batch * c_out || nh >= lim || ng >= lim || c_out * c_in * nf >= lim)
-    return false;
+  if (nh >= lim || ng >= lim || c_out * c_in * nf >= lim) return false;
   if (sx >= 4096 || sy >= 4096 || dx >= 4096 || dy >= 4096 || px >= lim || py >= lim) return false;
   // few input channels, and taps that fill their 32-row tiles reasonably
   const i64 mtn = (nf + 31) / 32;
@@ -259,40 +476,62 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
       if (std::abs(ey) < nhy && std::abs(span) >= 1 && std::abs(span) <= 31) { pl.batched_fold = 0; break; }
     }
   pl.ksteps = c_out <= 32 ? 16 : c_out <= 64 ? 32 : 64;
+  // streaming variant: needs batches that cannot collide and no padded matrix rows
+  pl.pipe = pl.batched_fold && (nf & 31) == 0 && force_pipe != 0;
   const i64 K = 2 * pl.ksteps;
   const i64 Wp = sy * (nhy - 1) + dy * (nfy - 1) + 1;
   const i64 reach = dx * (nfx - 1);
   if (Wp >= 4096) return false;
-  // strip height: enough workgroups to fill the chip about three times over, but
-  // strips at least twice as tall as the rows recomputed at their borders
-  const i64 want_strips = std::max<i64>(1, (768 + batch - 1) / batch);
-  i64 T = std::max<i64>((ngx + want_strips - 1) / want_strips, std::max<i64>(2 * reach / sx, 4));
-  if (force_T > 0) T = force_T;
-  T = std::min(T, ngx);
-  // LDS tiers: three, two, one workgroup per CU; within a tier the wider chunk
-  const size_t tiers[3] = {53 * 1024, 80 * 1024, 160 * 1024 - 512};
-  for (i64 t = T; t >= 1; t = (t > 8 ? t * 3 / 4 : t - 1)) {
-    const i64 Rp = sx * ((t - 1 + reach) / sx) + reach + 1;
-    if ((t + reach + 2) * std::max(nhy, Wp) >= ((i64)1 << 22)) continue;   // float-reciprocal index splits
-    if (c_in * t * ngy >= ((i64)1 << 22)) continue;
-    for (int tier = 0; tier < 3; ++tier)
-      for (int nt = 4; nt >= 2; nt -= 2) {
-        if (force_nt > 0 && nt != force_nt) continue;
-        const size_t lds = 4 * (size_t)(2 * K * nt * 32 + units * Rp * Wp);
-        if (lds > tiers[tier]) continue;
-        pl.nt = nt; pl.T = (int)t; pl.strips = (int)((ngx + t - 1) / t);
-        pl.Rp = (int)Rp; pl.Wp = (int)Wp; pl.lds_bytes = lds;
-        return (i64)pl.batch * pl.strips < ((i64)1 << 31);
-      }
+  // grad_out rows with a tap inside grad_input
+  const i64 H = std::min(nhx, (ngx - 1 + px) / sx + 1);
+  if (H < 1) return false;
+  // Strip height: about four workgroups per CU (1024 in all), and taller than a
+  // filter's reach so that a grad_input row is fed by at most two strips.
+  const i64 min_th = reach / sx + 1;
+  const i64 want_strips = std::max<i64>(1, (1024 + batch - 1) / batch);
+  i64 Th = std::max<i64>((H + want_strips - 1) / want_strips, std::max<i64>(min_th, 2));
+  if (force_Th > 0) Th = std::max<i64>(force_Th, min_th);
+  Th = std::min(Th, std::max(H, min_th));
+  // jobs per workgroup: make the wavefront count a multiple of four when that fits
+  const int max_waves = pl.ksteps == 64 ? 8 : 12;      // registers: see the launch bounds
+  pl.jobs = 1;
+  for (int j = 1; j <= 4; ++j)
+    if ((j * units) % 4 == 0 && j * units <= max_waves && j <= batch) { pl.jobs = j; break; }
+  if (units > max_waves) return false;
+  for (; Th >= min_th; Th = (Th > 8 ? Th * 3 / 4 : Th - 1)) {
+    const i64 Rp = sx * (Th - 1) + reach + 1;
+    if ((Th + 2) * nhy >= ((i64)1 << 22)) continue;              // float-reciprocal index splits
+    if (ngx + px + reach + sx >= ((i64)1 << 22) || batch * c_in > 65535) return false;
+    if ((reach - sx + 1) * ngy >= ((i64)1 << 22)) return false;
+    if (c_in * std::max(Rp, sx * Th) * ngy >= ((i64)1 << 22) || std::max(Rp, sx * Th) > K * 64) continue;
+    // chunk buffer: three 32-position blocks when streaming, else one chunk of 64 or
+    // (when the planes are small) 128 positions
+    int nt = 2;
+    if (!pl.pipe && (force_nt == 4 || (force_nt == 0 && 4 * (K * 128 + units * Rp * Wp) * pl.jobs <= 40 * 1024)))
+      nt = 4;
+    const i64 job_words = ((K * (pl.pipe ? 96 : nt * 32) + units * Rp * Wp) + 3) & ~(i64)3;
+    const size_t lds = 4 * (size_t)job_words * pl.jobs;
+    if (lds > 160 * 1024 - 512) continue;
+    pl.nt = nt; pl.Th = (int)Th; pl.H = (int)H; pl.strips = (int)((H + Th - 1) / Th);
+    pl.Rp = (int)Rp; pl.Wp = (int)Wp; pl.lds_bytes = lds;
+    pl.nshared = (int)std::max<i64>(0, reach - sx + 1);
+    pl.ws_bytes = pl.strips > 1 && pl.nshared > 0
+                      ? 4 * (size_t)batch * c_in * (pl.strips - 1) * pl.nshared * 2 * ngy : 0;
+    if ((i64)pl.batch * pl.strips >= ((i64)1 << 31)) return false;
+    if ((i64)batch * c_in * pl.strips * pl.nshared * 2 * ngy >= ((i64)1 << 40)) return false;
+    return true;
   }
   return false;
 }
 
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
-                        float *grad_input, hipStream_t stream) {
+                        float *grad_input, float *workspace, hipStream_t stream) {
+  // the pipelined fold needs batches that cannot collide and no padded matrix rows
+  const bool pipe = pl.pipe && pl.nt == 2;
 #define MELLIN_IGRAD_CASE(KS, NT_)                                                       \
   if (pl.ksteps == KS && pl.nt == NT_)                                                   \
-    return launch_instance<KS, NT_>(pl, weight, grad_out, grad_input, stream);
+    return pipe ? launch_instance<KS, NT_, (NT_ == 2)>(pl, weight, grad_out, grad_input, workspace, stream) \
+                : launch_instance<KS, NT_, false>(pl, weight, grad_out, grad_input, workspace, stream);
   MELLIN_IGRAD_CASE(16, 2) MELLIN_IGRAD_CASE(16, 4)
   MELLIN_IGRAD_CASE(32, 2) MELLIN_IGRAD_CASE(32, 4)
   MELLIN_IGRAD_CASE(64, 2) MELLIN_IGRAD_CASE(64, 4)

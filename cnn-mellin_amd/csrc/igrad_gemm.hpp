@@ -16,23 +16,28 @@ struct IgradPlan {
   int sx, dx, px, sy, dy, py;
   // blocking
   int mtn;                         // 32-tap tiles per input channel
-  int units;                       // c_in * mtn: wavefronts per workgroup
+  int units;                       // c_in * mtn: wavefronts per job
+  int jobs;                        // (image, strip) jobs that share a workgroup
   int ksteps;                      // (c_out rounded up) / 2: template instance
   int nt;                          // 32-position tiles per chunk: template instance
-  int T, strips;                   // grad_input rows per workgroup; workgroups per image
+  int H;                           // grad_out rows that have a tap inside grad_input
+  int Th, strips;                  // grad_out rows per workgroup; workgroups per image
+  int nshared;                     // grad_input rows fed by both strips at a boundary
   int Rp, Wp;                      // accumulator plane: rows and row length (words)
+  int pipe;                        // streaming variant (fold overlapped with the multiplies)
   int batched_fold;                // taps with congruent matrix rows never share a word: fold them in batches
-  size_t lds_bytes;
+  size_t lds_bytes, ws_bytes;      // ws: partial rows at the strip boundaries
 };
 
-// force_nt / force_T (0 = automatic) pin the chunk width and the strip height.
+// force_nt / force_Th (0 = automatic) pin the chunk width and the strip height;
+// force_pipe = 0 rules the streaming variant out.
 // False when the layer does not suit the kernel (Mellin x axis, ux or uy != 1,
 // too many channels, planes that do not fit in LDS, sizes beyond 32-bit indexing).
 bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                      i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
-                     i64 ux, i64 uy, IgradPlan &pl, int force_nt = 0, int force_T = 0);
+                     i64 ux, i64 uy, IgradPlan &pl, int force_nt = 0, int force_Th = 0, int force_pipe = -1);
 
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
-                        float *grad_input, hipStream_t stream);
+                        float *grad_input, float *workspace, hipStream_t stream);
 
 }  // namespace mellin

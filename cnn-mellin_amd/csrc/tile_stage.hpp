@@ -32,17 +32,33 @@ __device__ __forceinline__ void load_to_lds(const float *base, unsigned byte_off
                :: "s"(lds_addr), "v"(byte_offset), "s"(sbase) : "memory");
 }
 
+// LDS byte address of a pointer into shared memory (what m0 must hold).
+__device__ __forceinline__ unsigned lds_address(const float *p) {
+  return (unsigned)(size_t)(lds_float_ptr)p;
+}
+
 // Sixteen bytes per active lane: lane l reads the four dwords at `base` +
-// `byte_offset` (any 4-byte alignment) and they land at `row` + 16 * l (`row`
-// wave-uniform and 16-byte aligned).
-__device__ __forceinline__ void load16_to_lds(const float *base, unsigned byte_offset, float *row) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_float_ptr)row);
+// `byte_offset` (any 4-byte alignment) and they land at LDS byte address
+// `lds_addr` + 16 * l (`lds_addr` wave-uniform and 16-byte aligned).
+__device__ __forceinline__ void load16_to_lds_at(const float *base, unsigned byte_offset, unsigned lds_addr) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   const unsigned long long b = (unsigned long long)base;
   const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
   const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
   const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(lds_addr), "v"(byte_offset), "s"(sbase) : "memory");
+               :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
+}
+
+// load_to_lds with the destination given as an LDS byte address.
+__device__ __forceinline__ void load_to_lds_at(const float *base, unsigned byte_offset, unsigned lds_addr) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  const unsigned long long b = (unsigned long long)base;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
 }
 
 __device__ __forceinline__ void wait_all_memory() {
