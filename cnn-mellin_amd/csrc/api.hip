@@ -16,6 +16,7 @@ namespace {
 thread_local char g_error[512] = "";
 thread_local const char *g_variant = "";
 thread_local int g_forced = 0;   // 0 automatic, 1 generic, 2 automatic without the fused input gradient
+                                 // and without the row-wise weight gradient
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -283,11 +284,11 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
   if (sizeof(T) == 4 && g_forced != 1 && batch * ng * nh != 0) {
     WgradPlan wp;
     if (make_wgrad_plan(forward_problem(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy,
-                                        sx, sy, dx, dy, px, py, ux, uy), wp)) {
+                                        sx, sy, dx, dy, px, py, ux, uy), wp, g_forced != 2)) {
       if (!workspace || workspace_bytes < wp.ws_bytes)
         return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
                     wp.ws_bytes, workspace_bytes);
-      g_variant = "mfma";
+      g_variant = wp.rows_mode ? "mfma-rows" : "mfma";
       return check_hip(launch_wgrad(wp, (const float *)grad_out, (const float *)input,
                                     (float *)grad_weight, (float *)workspace,
                                     (hipStream_t)stream), fn);
@@ -394,7 +395,7 @@ size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
   WgradPlan wp;
-  if (!make_wgrad_plan(forward_problem(kind_x, CORR2D_ARGS), wp)) return 0;
+  if (!make_wgrad_plan(forward_problem(kind_x, CORR2D_ARGS), wp, g_forced != 2)) return 0;
   return wp.ws_bytes;
 }
 int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,

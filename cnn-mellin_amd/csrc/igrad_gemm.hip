@@ -80,9 +80,13 @@ __global__ __launch_bounds__((KSTEPS * NT <= 128 ? 768 : 512)) void igrad_kernel
   // group of pl.units wavefronts each with its own slice of LDS: same strip,
   // consecutive images, hence the same trip counts and barriers.  That makes the
   // wavefront count a multiple of four (all four SIMDs of a CU equally loaded).
-  const int job = (int)(threadIdx.x >> 6) / pl.units;
-  const int tid = threadIdx.x - job * pl.units * 64, nthreads = pl.units * 64;
-  const int lane = tid & 63, wave = tid >> 6;
+  // (wave-uniform quantities are marked as such: what derives from them is then
+  // computed on the scalar unit)
+  const int wave_in_group = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int job = wave_in_group / pl.units;
+  const int wave = wave_in_group - job * pl.units;
+  const int lane = threadIdx.x & 63;
+  const int tid = wave * 64 + lane, nthreads = pl.units * 64;
   const int half = lane >> 5, l32 = lane & 31;
   const int image_group = blockIdx.x / pl.strips, strip = blockIdx.x - image_group * pl.strips;
   const int n_want = image_group * pl.jobs + job;

@@ -64,7 +64,9 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
 
   MELLIN_PROBE_DECL
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  // the wave index is wave-uniform: say so, and everything derived from it (row
+  // loops, base addresses) is computed on the scalar unit
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, l32 = lane & 31;
   const int m0 = blockIdx.y * M_T;
   const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
@@ -73,7 +75,8 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   // ---- filter block: Ws[m][k], k = cl * nf + t, row stride WSS (odd) --------------
   // one direct load per (m, 64 taps): lane k fetches F[m0 + m, c0 + cl, t], coalesced
   // along the taps; taps past the chunk and channels past M are zero
-  auto issue_filter = [&](int c0, int cc, float *Ws) {
+  const unsigned lds_base = lds_address(lds);
+  auto issue_filter = [&](int c0, int cc, int ws_word) {        // ws_word: where the block starts in lds[]
     const int KC = cc * pl.nf;
     const FastDiv by_nf(pl.nf);
     const int m_live = max(0, min(M_T, pl.M - m0));       // channels of this block that exist
@@ -84,10 +87,10 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
       const unsigned voff = (unsigned)(((i64)(c0 + cl) * pl.f_c + t) * 4);   // < 4 GB: checked by the plan
       if (k < KC) {
         for (int m = wave; m < m_live; m += kWaves)
-          load_to_lds(F + (i64)(m0 + m) * pl.f_m, voff, Ws + m * pl.WSS + kb);
-        for (int m = m_live + wave; m < M_T; m += kWaves) Ws[m * pl.WSS + k] = 0.f;
+          load_to_lds_at(F + (i64)(m0 + m) * pl.f_m, voff, lds_base + 4u * (unsigned)(ws_word + m * pl.WSS + kb));
+        for (int m = m_live + wave; m < M_T; m += kWaves) lds[ws_word + m * pl.WSS + k] = 0.f;
       } else if (k < pl.KCp) {
-        for (int m = wave; m < M_T; m += kWaves) Ws[m * pl.WSS + k] = 0.f;
+        for (int m = wave; m < M_T; m += kWaves) lds[ws_word + m * pl.WSS + k] = 0.f;
       }
     }
   };
@@ -101,8 +104,9 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
     const int ti = st / chunks, ch = st - ti * chunks;
     const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
     const int c0 = ch * pl.CC, cc = min(pl.CC, pl.C - c0);
-    issue_signal(pl, tg, G, c0, cc, Gs0 + (st & 1) * g_words, mellin_x, lane, wave);
-    if (!single_chunk) issue_filter(c0, cc, Ws0 + (st & 1) * w_words);
+    issue_signal(pl, tg, G, c0, cc, Gs0 + (st & 1) * g_words, lds_base + 4u * (unsigned)((st & 1) * g_words),
+                 mellin_x, lane, wave);
+    if (!single_chunk) issue_filter(c0, cc, 2 * g_words + (st & 1) * w_words);
   };
 
   {
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   }
   MELLIN_STAMP(0);
   if (my_stages > 0) {
-    if (single_chunk) issue_filter(0, pl.C, Ws0);
+    if (single_chunk) issue_filter(0, pl.C, 2 * g_words);
     issue_stage(0);
   }
   MELLIN_STAMP(1);

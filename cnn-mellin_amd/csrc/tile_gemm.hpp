@@ -49,10 +49,15 @@ struct WgradPlan {
   int CCj;                         // input channels a column block can touch
   int GSS;                         // row stride of the staged grad_out tile (words)
   int S;                           // position shares = persistent workgroups per output block
+  int rows_mode;                   // 1: the row-wise kernel (one output row per wavefront)
+  int nbuf;                        // row-wise kernel: LDS buffers per operand (1 or 2)
   size_t lds_bytes, ws_bytes;
 };
 
-bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp);
+// allow_rows = false rules the row-wise kernel out (for comparisons)
+// rows_mt / rows_nbuf: channel tiles per workgroup and buffers of the row-wise kernel
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool allow_rows = true, int rows_mt = 1,
+                     int rows_nbuf = 2);
 
 hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float *input,
                         float *grad_weight, float *workspace, hipStream_t stream);

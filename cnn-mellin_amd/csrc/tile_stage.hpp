@@ -15,23 +15,6 @@ constexpr int kThreads = kWaves * 64;
 
 typedef __attribute__((address_space(3))) float *lds_float_ptr;
 
-// One dword per active lane straight from global memory to LDS: lane l reads
-// the dword at `base` + `byte_offset` (base wave-uniform, offset per lane) and
-// it lands at `row` + 4 * l (`row` wave-uniform).  Completion is counted by
-// vmcnt.  Written as inline assembly on purpose: the compiler then does not
-// order later LDS reads after these loads, which is what lets the loads of the
-// next stage stay in flight during the matrix loop; every consumer waits
-// explicitly (wait_all_memory + barrier).  m0 carries the LDS base.
-__device__ __forceinline__ void load_to_lds(const float *base, unsigned byte_offset, float *row) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_float_ptr)row);
-  const unsigned long long b = (unsigned long long)base;
-  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
-  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
-  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-               :: "s"(lds_addr), "v"(byte_offset), "s"(sbase) : "memory");
-}
-
 // LDS byte address of a pointer into shared memory (what m0 must hold).
 __device__ __forceinline__ unsigned lds_address(const float *p) {
   return (unsigned)(size_t)(lds_float_ptr)p;
@@ -50,7 +33,14 @@ __device__ __forceinline__ void load16_to_lds_at(const float *base, unsigned byt
                :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
 }
 
-// load_to_lds with the destination given as an LDS byte address.
+// One dword per active lane straight from global memory to LDS: lane l reads
+// the dword at `base` + `byte_offset` (base wave-uniform, offset per lane) and
+// it lands at LDS byte address `lds_addr` + 4 * l (`lds_addr` wave-uniform).
+// Completion is counted by vmcnt.  Written as inline assembly on purpose: the
+// compiler then does not order later LDS reads after these loads, which is
+// what lets the loads of the next stage stay in flight during the matrix
+// loop; every consumer waits explicitly (wait_all_memory + barrier).  m0
+// carries the LDS base.  Destinations are passed as addresses, not pointers.
 __device__ __forceinline__ void load_to_lds_at(const float *base, unsigned byte_offset, unsigned lds_addr) {
   const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   const unsigned long long b = (unsigned long long)base;
@@ -130,7 +120,8 @@ __device__ __forceinline__ TileGeom tile_geometry(const TilePlan &pl, int tile_i
 // columns; columns or rows without a source are written as zeros.
 __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom &tg,
                                              const float *__restrict__ G, int c0, int cc,
-                                             float *Gs, bool mellin_x, int lane, int wave) {
+                                             float *Gs, unsigned gs_addr, bool mellin_x, int lane,
+                                             int wave) {
   const int total_rows = cc * tg.R_tile;
   const float *Gimg = G + (i64)tg.n * pl.g_n + (i64)c0 * pl.g_c;
   const int g_c = (int)pl.g_c;                         // fits: c_in * ngx * ngy < 2^31
@@ -175,7 +166,7 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
           const int s_src = __builtin_amdgcn_readlane(src_off, j);
           if (s_src >= 0) {
             const int s_dst = __builtin_amdgcn_readlane(dst_off, j);
-            load_to_lds(Gimg + s_src, voff, Gs + s_dst + cb);
+            load_to_lds_at(Gimg + s_src, voff, gs_addr + 4u * (unsigned)(s_dst + cb));
           }
         }
       }

@@ -43,9 +43,12 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
   float *Xs0 = lds;                                  // [2][CCj][R][RS]
   float *As0 = Xs0 + 2 * x_words;                    // [2][M_T][GSS]
   int *posoff0 = (int *)(As0 + 2 * a_words);         // [2][P]
+  const unsigned lds_base = lds_address(lds);
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  // the wave index is wave-uniform: say so, and everything derived from it (row
+  // loops, base addresses) is computed on the scalar unit
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, l32 = lane & 31;
   const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
 
@@ -77,7 +80,8 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
   auto issue_stage = [&](int ti) {
     const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
     const int b = ti & 1;
-    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, mellin_x, lane, wave);
+    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words), mellin_x,
+                 lane, wave);
     // grad_out rows: P consecutive positions per output channel, zeros past the tile
     const float *An = A + (i64)tg.n * wp.a_n + tg.q0;
     float *As = As0 + b * a_words;
@@ -86,7 +90,8 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
       const int p = pb + lane;
       if (p < tg.count) {
         for (int m = wave; m < m_live; m += kWaves)
-          load_to_lds(An + (i64)(m0 + m) * wp.a_m, (unsigned)p * 4u, As + m * wp.GSS + pb);
+          load_to_lds_at(An + (i64)(m0 + m) * wp.a_m, (unsigned)p * 4u,
+                         lds_base + 4u * (unsigned)(2 * x_words + b * a_words + m * wp.GSS + pb));
         for (int m = max(m_live, 0) + wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
       } else {
         for (int m = wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
@@ -205,6 +210,223 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
   }
 }
 
+// Row-wise variant for layers whose outputs are walked a whole row at a time
+// (unit y stride, rows of at least 16 outputs that fit one tile).  A unit of work
+// is four consecutive output rows of one image, one row per wavefront.  Within
+// a row every operand address is affine in the column: position oy of output
+// row ox reads grad_out word  row_base + oy  and, for column j = (c, fx, fy),
+// input word  col_offset[j] + virtual_row(ox) * RS + oy - by_min,  so the loop
+// over the row needs no index arithmetic at all: LDS reads with immediate
+// offsets and matrix instructions only.  (On this chip the fp32 matrix
+// instructions run on the same ALUs as ordinary vector instructions: every
+// vector instruction saved in the loop is matrix throughput gained.)
+// grad_out rows arrive by 16-byte direct loads (the four rows of a unit are
+// contiguous per channel); the input rows are staged as in the forward kernel.
+template <int MT, int JT>
+__global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
+    WgradPlan wp, const float *__restrict__ A, const float *__restrict__ G,
+    float *__restrict__ ws) {
+  extern __shared__ __align__(16) float lds[];
+  const TilePlan &pl = wp.t;
+  constexpr int M_T = MT * 32, J_T = JT * 32, RB = kWaves;
+  const int x_words = (wp.CCj * pl.R * pl.RS + 3) & ~3;
+  const int a_words = M_T * wp.GSS;
+  float *Xs0 = lds;                                  // [nbuf][CCj][R][RS]
+  float *As0 = Xs0 + wp.nbuf * x_words;              // [nbuf][M_T][GSS]
+
+  const int tid = threadIdx.x;
+  // the wave index is wave-uniform: say so, and everything derived from it (row
+  // loops, base addresses) is computed on the scalar unit
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, l32 = lane & 31;
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+
+  const int mg = blockIdx.y / wp.j_groups, jg = blockIdx.y - mg * wp.j_groups;
+  const int m0 = mg * M_T, j0 = jg * J_T;
+  const int c_lo = j0 / pl.nf;
+  const int j_last = min(wp.J, j0 + J_T) - 1;
+  const int ccj = j_last / pl.nf - c_lo + 1;
+  const int m_live = max(0, min(M_T, pl.M - m0));
+
+  int col_off[JT];
+  {
+    const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
+#pragma unroll
+    for (int t = 0; t < JT; ++t) {
+      const int j = min(j0 + t * 32 + l32, wp.J - 1);   // columns past J are computed but never stored
+      int c, tt, fx, fy;
+      by_nf.divmod(j, c, tt);
+      by_nfy.divmod(tt, fx, fy);
+      col_off[t] = (c - c_lo) * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+    }
+  }
+  // grad_out rows of channels past M are never loaded: zeros, once
+  if (m_live < M_T) {
+    const int dead = (M_T - m_live) * wp.GSS;
+    for (int i = tid; i < dead; i += kThreads) {
+      As0[m_live * wp.GSS + i] = 0.f;
+      if (wp.nbuf == 2) As0[a_words + m_live * wp.GSS + i] = 0.f;
+    }
+  }
+
+  const int units_per_image = (pl.nox_eff + RB - 1) / RB;
+  const int total_units = pl.batch * units_per_image;
+  const int my_units = (int)blockIdx.x < total_units
+                           ? (total_units - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+  const unsigned lds_base = lds_address(lds);
+  const unsigned as_addr = lds_base + 4u * (unsigned)(wp.nbuf * x_words);
+
+  auto unit_geometry = [&](int unit) {
+    TileGeom g;
+    g.n = unit / units_per_image;
+    g.ox_lo = (unit - g.n * units_per_image) * RB;
+    const int rows = min(RB, pl.nox_eff - g.ox_lo);
+    g.oy_lo = 0;
+    g.q0 = g.ox_lo * pl.noy;
+    g.count = rows * pl.noy;
+    g.R_tile = mellin_x ? rows * pl.nfx : pl.ax * (rows - 1) + pl.bx_span + 1;
+    g.vx_min = pl.ax * g.ox_lo + pl.cx + pl.bx_min;
+    g.vy_min = pl.cy + pl.by_min;
+    g.RSL = pl.ay * (pl.noy - 1) + pl.by_span + 1;
+    return g;
+  };
+  auto issue_stage = [&](int ui) {
+    const TileGeom tg = unit_geometry(blockIdx.x + ui * gridDim.x);
+    const int b = wp.nbuf == 2 ? (ui & 1) : 0;
+    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words), mellin_x,
+                 lane, wave);
+    // grad_out: the unit's rows are one run of `count` words per channel
+    const float *An = A + (i64)tg.n * wp.a_n;
+    const int count4 = tg.count & ~3;
+    for (int m = wave; m < m_live; m += kWaves) {
+      const float *src = An + (i64)(m0 + m) * wp.a_m;
+      const unsigned dst = as_addr + 4u * (unsigned)(b * a_words + m * wp.GSS);
+      for (int w0 = 0; w0 < count4; w0 += 256) {
+        const int idx = w0 + 4 * lane;
+        if (idx < count4) load16_to_lds_at(src, (unsigned)(tg.q0 + idx) * 4u, dst + 4u * (unsigned)w0);
+      }
+      if (lane < tg.count - count4)
+        load_to_lds_at(src, (unsigned)(tg.q0 + count4 + lane) * 4u, dst + 4u * (unsigned)count4);
+    }
+  };
+
+  floatx16 acc[MT][JT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
+
+  const int pairs = pl.noy >> 1;
+  auto multiply_unit = [&](int ui) {
+    const int unit = blockIdx.x + ui * gridDim.x;
+    const int ox_lo = (unit % units_per_image) * RB;
+    if (ox_lo + wave < pl.nox_eff) {                     // this wavefront's row exists
+      const int b = wp.nbuf == 2 ? (ui & 1) : 0;
+      const float *Xs = Xs0 + b * x_words;
+      const float *As = As0 + b * a_words;
+      int ao = l32 * wp.GSS + wave * pl.noy + half;
+      int bo[JT];
+#pragma unroll
+      for (int t = 0; t < JT; ++t)
+        bo[t] = col_off[t] + (pl.Ax * wave + pl.Cx0) * pl.RS - pl.by_min + half;
+      int s = 0;
+      for (; s + 8 <= pairs; s += 8) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float a[MT], b[JT];
+#pragma unroll
+          for (int i = 0; i < MT; ++i) a[i] = As[ao + i * 32 * wp.GSS + 2 * k];
+#pragma unroll
+          for (int t = 0; t < JT; ++t) b[t] = Xs[bo[t] + 2 * k];
+#pragma unroll
+          for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int t = 0; t < JT; ++t)
+              acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+        }
+        ao += 16;
+#pragma unroll
+        for (int t = 0; t < JT; ++t) bo[t] += 16;
+      }
+      for (; s < pairs; ++s) {
+        float a[MT], b[JT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a[i] = As[ao + i * 32 * wp.GSS];
+#pragma unroll
+        for (int t = 0; t < JT; ++t) b[t] = Xs[bo[t]];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int t = 0; t < JT; ++t)
+            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+        ao += 2;
+#pragma unroll
+        for (int t = 0; t < JT; ++t) bo[t] += 2;
+      }
+      if (pl.noy & 1) {
+        // the row's last position stands alone: the other half-wave multiplies zeros
+        float a[MT], b[JT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) a[i] = half ? 0.f : As[ao + i * 32 * wp.GSS];
+#pragma unroll
+        for (int t = 0; t < JT; ++t) b[t] = half ? 0.f : Xs[bo[t]];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int t = 0; t < JT; ++t)
+            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+      }
+    }
+  };
+  __syncthreads();
+  if (wp.nbuf == 2) {
+    // two buffers: the loads of the next unit fly during the multiplies of this one
+    if (my_units > 0) issue_stage(0);
+    for (int ui = 0; ui < my_units; ++ui) {
+      wait_all_memory();
+      __syncthreads();
+      if (ui + 1 < my_units) issue_stage(ui + 1);
+      multiply_unit(ui);
+    }
+  } else {
+    // one buffer and more workgroups per CU: they cover each other's loads
+    for (int ui = 0; ui < my_units; ++ui) {
+      issue_stage(ui);
+      wait_all_memory();
+      __syncthreads();
+      multiply_unit(ui);
+      __syncthreads();
+    }
+  }
+
+  // ---- sum the four wavefronts in wave order, then write the partial block ------
+  __syncthreads();
+  float *red = lds;                                   // [M_T][J_T]
+  for (int w = 0; w < kWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < JT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float *dst = red + m * J_T + t * 32 + l32;
+            if (w == 0) *dst = acc[i][t][r];
+            else *dst += acc[i][t][r];
+          }
+    }
+    __syncthreads();
+  }
+  float *out = ws + (i64)blockIdx.x * wp.M_pad * wp.J_pad + (i64)m0 * wp.J_pad + j0;
+  for (int e = tid; e < M_T * J_T; e += kThreads) {
+    const int m = e / J_T, jj = e - m * J_T;
+    out[(i64)m * wp.J_pad + jj] = red[e];
+  }
+}
+
 // W[m, j] = sum over the S partial blocks, in index order.  A block of 256
 // threads handles 16 outputs: 16 threads per output add every 16th partial,
 // then thread 0 of each output adds the 16 sums in order.
@@ -254,11 +476,28 @@ hipError_t launch_variant(const WgradPlan &wp, size_t lds_bytes, dim3 grid, cons
   return hipGetLastError();
 }
 
+template <int MT, int JT>
+hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const float *g, float *ws,
+                       hipStream_t stream) {
+  auto kern = wgrad_rows_kernel<MT, JT>;
+  if (wp.lds_bytes > 64 * 1024) {
+    static thread_local size_t granted = 0;
+    if (granted < wp.lds_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)wp.lds_bytes);
+      if (e != hipSuccess) return e;
+      granted = wp.lds_bytes;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 // Plan the weight gradient of the layer whose FORWARD problem is `fwd`
 // (filter = weight, signal = input, output = grad_out, write mode).
-bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp) {
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf) {
   size_t lds_fwd;
   int mt, nt;
   // 128 positions per tile: the staged grad_out tile (channels x positions, two
@@ -277,6 +516,43 @@ bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp) {
   wp.a_m = pl.Q;
   // the forward plan fixed the position tiling (nt) and the row geometry
   wp.nt = nt;
+  wp.rows_mode = 0;
+  if (!pl.segment && pl.ay == 1 && pl.noy >= 16 && pl.nox_eff >= 1 && g_allow_rows) {
+    // row-wise variant: units of kWaves output rows
+    const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+    const int rb = std::min<int>(kWaves, pl.nox);
+    const i64 Rr = mellin_x ? (i64)rb * pl.nfx : (i64)pl.ax * (rb - 1) + pl.bx_span + 1;
+    int pitch = (kWaves * pl.noy + 3) & ~3;
+    if (((pitch >> 2) & 1) == 0) pitch += 4;              // 4 x odd: channels spread over the banks
+    const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
+    const size_t xw = ((size_t)ccj * Rr * pl.RS + 3) & ~(size_t)3;
+    // all channels in one workgroup (two 32-row tiles) when they fit: the input is then staged once
+    int mt_rows = (pl.M > 32 && rows_opt_mt == 2) ? 2 : 1;
+    const int nbuf = rows_opt_nbuf;
+    size_t bytes = 4 * std::max(nbuf * (xw + (size_t)mt_rows * 32 * pitch), (size_t)mt_rows * 32 * J_T);
+    if (mt_rows == 2 && bytes > 150 * 1024) {
+      mt_rows = 1;
+      bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), (size_t)32 * J_T);
+    }
+    if (Rr <= 8192 && bytes <= (mt_rows == 2 ? 150 : 78) * 1024) {
+      wp.nbuf = nbuf;
+      wp.rows_mode = 1;
+      pl.R = (int)Rr;
+      wp.GSS = pitch;
+      wp.CCj = ccj;
+      wp.lds_bytes = bytes;
+      wp.mt = mt_rows;
+      wp.m_groups = (pl.M + mt_rows * 32 - 1) / (mt_rows * 32);
+      wp.M_pad = wp.m_groups * mt_rows * 32;
+      const int blocks_y_rows = wp.m_groups * wp.j_groups;
+      const i64 units = (i64)pl.batch * ((pl.nox_eff + kWaves - 1) / kWaves);
+      int per_cu = std::max(1, std::min((int)((160 * 1024) / (bytes + 512)), nbuf == 2 ? 4 : 6));
+      i64 S = std::max<i64>(1, (256 * per_cu) / blocks_y_rows);
+      wp.S = (int)std::min<i64>(S, units);
+      wp.ws_bytes = (size_t)wp.S * wp.M_pad * wp.J_pad * sizeof(float);
+      return true;
+    }
+  }
   const int P = kWaves * nt * 32;
   wp.GSS = P + 1;
   wp.CCj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
@@ -299,6 +575,13 @@ hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float 
                         float *grad_weight, float *workspace, hipStream_t stream) {
   dim3 grid((unsigned)wp.S, (unsigned)(wp.m_groups * wp.j_groups));
   hipError_t e = hipErrorInvalidValue;
+  if (wp.rows_mode) {
+#define MELLIN_ROWS_CASE(MT_, JT_)                                                         \
+  if (wp.mt == MT_ && wp.jt == JT_) e = launch_rows<MT_, JT_>(wp, grid, grad_out, input, workspace, stream);
+    MELLIN_ROWS_CASE(1, 1) MELLIN_ROWS_CASE(1, 2) MELLIN_ROWS_CASE(1, 3)
+    MELLIN_ROWS_CASE(2, 1) MELLIN_ROWS_CASE(2, 2) MELLIN_ROWS_CASE(2, 3)
+#undef MELLIN_ROWS_CASE
+  } else {
 #define MELLIN_WGRAD_CASE(MT_, JT_, NT_)                                                   \
   if (wp.mt == MT_ && wp.jt == JT_ && wp.nt == NT_)                                          \
     e = launch_variant<MT_, JT_, NT_>(wp, wp.lds_bytes, grid, grad_out, input, workspace, stream);
@@ -306,6 +589,7 @@ hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float 
   MELLIN_WGRAD_CASE(1, 2, 1)
   MELLIN_WGRAD_CASE(1, 1, 1)
 #undef MELLIN_WGRAD_CASE
+  }
   if (e != hipSuccess) return e;
   const int outputs = wp.t.M * wp.J;
   hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((outputs + 15) / 16)), dim3(256), 0, stream,
