@@ -361,6 +361,12 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   if (pr.c_in * pr.f_c + nf >= lim || pr.f_c < 0 || pr.f_m < 0) return false;   // 32-bit byte offsets into the filter
   pl.R = (int)R;
   pl.RS = (int)RSL | 1;                                            // odd stride spreads LDS banks
+  // Linear axes without up-sampling or left padding, tiles spanning whole rows
+  // that use every signal column: a virtual row is a signal row.  Give it the
+  // signal's pitch, and a tile's rows are one contiguous run per channel.
+  pl.contig = !mellin_x && !pl.segment && pl.ux == 1 && pl.uy == 1 && pl.cy + pl.by_min == 0 &&
+              RSL <= pl.ngy && pl.ngy <= RSL + 8;
+  if (pl.contig) pl.RS = pl.ngy;
 
 
   // channels per chunk from the LDS budget: two signal buffers, and two

@@ -24,6 +24,7 @@ struct TilePlan {
   // tiling
   int segment, chunks_per_row, tiles_per_image, total_tiles;
   int R, RS;                       // virtual rows per channel and their stride (words)
+  int contig;                      // virtual rows coincide with the signal's rows (same pitch): block copies
   int CP, CP_log2;                 // staged columns rounded up to a power of two
   int CC;                          // channels staged per chunk
   int KCp;                         // CC * nf rounded up to even

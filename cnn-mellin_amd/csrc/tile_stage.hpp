@@ -125,6 +125,26 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
   const int total_rows = cc * tg.R_tile;
   const float *Gimg = G + (i64)tg.n * pl.g_n + (i64)c0 * pl.g_c;
   const int g_c = (int)pl.g_c;                         // fits: c_in * ngx * ngy < 2^31
+  if (pl.contig && tg.vx_min >= 0 && tg.vx_min + tg.R_tile <= pl.ngx) {
+    // the virtual rows ARE the signal rows vx_min ... of each channel, with the
+    // signal's own row pitch: one run of R_tile * ngy words per channel, moved
+    // 16 bytes per lane (1 KB per instruction), the pieces dealt out to the waves
+    const int count = tg.R_tile * pl.ngy, count4 = count & ~3;
+    const int pieces = (count4 + 255) >> 8;
+    const float *src0 = Gimg + tg.vx_min * pl.ngy;
+    for (int i = wave; i < cc * pieces; i += kWaves) {
+      const int cl = i / pieces, w0 = (i - cl * pieces) << 8;
+      const int idx = w0 + 4 * lane;
+      if (idx < count4)
+        load16_to_lds_at(src0 + (i64)cl * g_c, (unsigned)idx * 4u, gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + w0));
+    }
+    if (count4 < count)
+      for (int cl = wave; cl < cc; cl += kWaves)
+        if (lane < count - count4)
+          load_to_lds_at(src0 + (i64)cl * g_c, (unsigned)(count4 + lane) * 4u,
+                         gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + count4));
+    return;
+  }
   const FastDiv by_rows(tg.R_tile), by_nfx(pl.nfx);
   for (int base = 0; base < total_rows; base += 64 * kWaves) {
     // per-lane: row base + 4 * lane + wave
