@@ -31,6 +31,10 @@ int check_hip(hipError_t e, const char *what) {
   return fail(MELLIN_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
 }
 
+// The tap-product input gradient keeps c_in * taps values per grad_out element in
+// the workspace; past this size the two-pass variant is used instead.
+const size_t kMaxTapProductBytes = (size_t)1 << 30;
+
 bool mellin_kind(int k) { return k == AX_MCORR || k == AX_MCONV; }
 
 // Parameter domain of one axis.  s, d, u divide or scale indices and must be
@@ -236,6 +240,25 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
                                     (float *)grad_input, (float *)workspace, (hipStream_t)stream), fn);
     }
   }
+  if (sizeof(T) == 4 && g_forced == 0 && c_out * nf * nh != 0) {
+    // tap products through the workspace, then a gather (any x axis kind)
+    TapProductPlan zp;
+    if (make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, zp) && zp.ws_bytes <= kMaxTapProductBytes) {
+      if (!workspace || workspace_bytes < zp.ws_bytes)
+        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
+                    zp.ws_bytes, workspace_bytes);
+      g_variant = "mfma-taps+fold";
+      hipError_t e = launch_tap_product(zp, (const float *)weight, (const float *)grad_out,
+                                        (float *)workspace, (hipStream_t)stream);
+      if (e == hipSuccess) {
+        const Axis fx = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
+        const Axis fy = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
+        e = launch_fold_xy(fx, fy, batch * c_in, zp.nf_pad, (const float *)workspace,
+                           (float *)grad_input, (hipStream_t)stream);
+      }
+      return check_hip(e, fn);
+    }
+  }
   if (sizeof(T) == 4 && g_forced != 1 && c_out * nf * nh != 0) {
     TwoPassInput tp;
     if (plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy,
@@ -371,6 +394,10 @@ size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
   if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
   IgradPlan ip;
   if (g_forced == 0 && make_igrad_plan(kind_x, CORR2D_ARGS, ip)) return ip.ws_bytes;
+  TapProductPlan zp;
+  if (g_forced == 0 && make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, zp) &&
+      zp.ws_bytes <= kMaxTapProductBytes)
+    return zp.ws_bytes;
   TwoPassInput tp;
   if (!plan_two_pass_input(kind_x, CORR2D_ARGS, tp)) return 0;
   return tp.ws_bytes;

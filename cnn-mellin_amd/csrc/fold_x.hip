@@ -1,5 +1,6 @@
-// Second half of the two-pass input gradient used when the layer has few input
-// channels.  The first pass (the matrix-core gather-GEMM, run with one output
+// Gathers that finish the input gradient of layers with few input channels.
+//
+// fold_x: second half of the two-pass input gradient.  The first pass (the matrix-core gather-GEMM, run with one output
 // channel per (input channel, filter row) pair) leaves
 //
 //   Y[n, ci * nfx + fx, hx, gy] = sum_{co, fy} weight[co, ci, fx, fy] *
@@ -40,7 +41,189 @@ __global__ __launch_bounds__(256) void fold_x_kernel(Axis x, i64 batch_cin, i64 
   }
 }
 
+// Signal index chosen by (h, f) on one axis, or -1, in 32-bit arithmetic with a
+// float-reciprocal division.  Exact while numerators stay below 2^22 (the
+// launcher checks); p1 = p + 1.
+__device__ __forceinline__ int tap32(int kind, int h, int f, int ng, int s, int d, int p, int u) {
+  int num, den, off = 0;
+  switch (kind) {
+    case AX_MCORR: num = (h + s) * (f + d); den = p + 1; off = u; break;
+    case AX_MCONV: num = (p + 1) * (h + s); den = f + d; off = u; break;
+    case AX_LCORR: num = s * h + d * f - p; den = u; break;
+    default:       num = s * h - d * f + p; den = u; break;
+  }
+  if (num < 0) return -1;                               // linear kinds only; a negative index is no tap
+  int q = (int)((float)num * (1.0f / (float)den));
+  int r = num - q * den;
+  if (r < 0) { --q; r += den; }
+  else if (r >= den) { ++q; r -= den; }
+  if (r != 0) return -1;
+  const int g = q - off;
+  return (g >= 0 && g < ng) ? g : -1;
+}
+
+// Gather that finishes the tap-product input gradient:
+//
+//   grad_input[n, ci, gx, gy] = sum_{fx, fy} Z[n, ci, fx * nfy + fy, hx(gx, fx), hy(gy, fy)]
+//
+// over the taps that exist, in ascending (fx, fy): a fixed order, no atomics.
+// Z has nf_pad tap rows per (n, ci).  One thread per output, coalesced along gy.
+// SMALL: every index product fits the 32-bit path above.
+template <bool SMALL>
+__global__ __launch_bounds__(256) void fold_xy_kernel(Axis x, Axis y, i64 batch_cin, int nf_pad,
+                                                      const float *__restrict__ Z,
+                                                      float *__restrict__ gi) {
+  // x, y: convolution-kind axes with nf = filter extent, ng = grad_out extent, nh = grad_input extent
+  const i64 ngx = x.nh, ngy = y.nh, nhx = x.ng, nhy = y.ng;
+  const i64 total = batch_cin * ngx * ngy;
+  const i64 nh = nhx * nhy;
+  const i64 step = (i64)gridDim.x * blockDim.x;
+  for (i64 i = (i64)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+    i64 gy, gx, nc;                                     // nc = n * c_in + ci
+    if (SMALL) {
+      const unsigned ui = (unsigned)i, r = ui / (unsigned)ngy;
+      gy = ui - r * (unsigned)ngy;
+      nc = r / (unsigned)ngx;
+      gx = r - (unsigned)nc * (unsigned)ngx;
+    } else {
+      gy = i % ngy;
+      const i64 r = i / ngy;
+      gx = r % ngx;
+      nc = r / ngx;
+    }
+    const float *Znc = Z + nc * nf_pad * nh;
+    float acc = 0.f;
+    if (gx < x.nh_eff && gy < y.nh_eff) {
+      // the column's y taps are the same for every filter row: work them out once
+      // (as offsets into a tap row of Z, -1 = no tap) when the filter is narrow enough
+      constexpr int kHoist = 8;
+      int yoff[kHoist];
+      const int nfy = (int)y.nf;
+      const bool hoisted = nfy <= kHoist;
+      if (hoisted) {
+#pragma unroll
+        for (int fy = 0; fy < kHoist; ++fy) {
+          i64 hy = -1;
+          if (fy < nfy)
+            hy = SMALL ? (i64)tap32(y.kind, (int)gy, fy, (int)nhy, (int)y.s, (int)y.d, (int)y.p, (int)y.u)
+                       : tap_index(y.kind, gy, fy, nhy, y.s, y.d, y.p, y.u);
+          yoff[fy] = hy < 0 ? -1 : (int)hy;
+        }
+      }
+      for (int fx = 0; fx < (int)x.nf; ++fx) {
+        const i64 hx = SMALL ? (i64)tap32(x.kind, (int)gx, fx, (int)nhx, (int)x.s, (int)x.d, (int)x.p, (int)x.u)
+                             : tap_index(x.kind, gx, fx, nhx, x.s, x.d, x.p, x.u);
+        if (hx < 0) continue;
+        const float *Zf = Znc + (i64)fx * y.nf * nh + hx * nhy;
+        if (hoisted) {
+#pragma unroll
+          for (int fy = 0; fy < kHoist; ++fy)
+            if (fy < nfy && yoff[fy] >= 0) acc += Zf[(i64)fy * nh + yoff[fy]];
+        } else {
+          for (int fy = 0; fy < nfy; ++fy) {
+            const i64 hy = SMALL ? (i64)tap32(y.kind, (int)gy, fy, (int)nhy, (int)y.s, (int)y.d, (int)y.p, (int)y.u)
+                                 : tap_index(y.kind, gy, fy, nhy, y.s, y.d, y.p, y.u);
+            if (hy >= 0) acc += Zf[(i64)fy * nh + hy];
+          }
+        }
+      }
+    }
+    gi[i] = acc;
+  }
+}
+
+// The same gather, one wavefront per 8 consecutive grad_input rows of one
+// (image, channel), lanes along gy.  The y taps of a column do not depend on
+// the row, so a lane works them out once; the x taps of a row do not depend on
+// the column, so lane fx works out tap fx and the wavefront reads them back as
+// scalars.  For filters of at most 64 x 8 taps and indices on the 32-bit path.
+__global__ __launch_bounds__(256) void fold_xy_rows_kernel(Axis x, Axis y, int batch_cin, int nf_pad,
+                                                           const float *__restrict__ Z,
+                                                           float *__restrict__ gi) {
+  const int ngx = (int)x.nh, ngy = (int)y.nh, nhx = (int)x.ng, nhy = (int)y.ng;
+  const int nfx = (int)x.nf, nfy = (int)y.nf;
+  const i64 nh = (i64)nhx * nhy;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int blocks_per_nc = (ngx + 31) >> 5;
+  const int nc = blockIdx.x / blocks_per_nc;
+  const int gx0 = (blockIdx.x - nc * blocks_per_nc) * 32 + wave * 8;
+  const float *Znc = Z + (i64)nc * nf_pad * nh;
+  float *out = gi + (i64)nc * ngx * ngy;
+  for (int gy0 = 0; gy0 < ngy; gy0 += 64) {
+    const int gy = gy0 + lane;
+    const bool live = gy < ngy;
+    // word of this column's tap fy inside a (channel, filter row, grad_out row) block
+    // of Z: fy * nh + hy, or -1
+    int yoff[8];
+#pragma unroll
+    for (int fy = 0; fy < 8; ++fy) {
+      const int hy = (live && gy < (int)y.nh_eff && fy < nfy)
+                         ? tap32(y.kind, gy, fy, nhy, (int)y.s, (int)y.d, (int)y.p, (int)y.u) : -1;
+      yoff[fy] = hy < 0 ? -1 : fy * (int)nh + hy;
+    }
+    for (int r = 0; r < 8; ++r) {
+      const int gx = gx0 + r;
+      if (gx >= ngx) break;
+      const int hx_lane = (lane < nfx && gx < (int)x.nh_eff)
+                              ? tap32(x.kind, gx, lane, nhx, (int)x.s, (int)x.d, (int)x.p, (int)x.u) : -1;
+      float acc = 0.f;
+      // eight filter rows at a time: every load is issued before the first sum, so a
+      // row costs one memory round trip rather than one per tap; the sums keep
+      // their (fx, fy) order.  Row bases are scalars, lane offsets 32-bit.
+      for (int fxc = 0; fxc < nfx; fxc += 8) {
+        float v[8][8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int fx = fxc + j;
+          const int hx = fx < nfx ? __builtin_amdgcn_readlane(hx_lane, fx & 63) : -1;
+          if (hx >= 0) {
+            const unsigned row = (unsigned)(fx * nfy) * (unsigned)nh + (unsigned)(hx * nhy);
+#pragma unroll
+            for (int fy = 0; fy < 8; ++fy) v[j][fy] = yoff[fy] >= 0 ? Znc[row + (unsigned)yoff[fy]] : 0.f;
+          } else {
+#pragma unroll
+            for (int fy = 0; fy < 8; ++fy) v[j][fy] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int fy = 0; fy < 8; ++fy) acc += v[j][fy];
+      }
+      if (live) out[(i64)gx * ngy + gy] = acc;
+    }
+  }
+}
+
 }  // namespace
+
+hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
+                          float *grad_input, hipStream_t stream) {
+  const i64 total = batch_cin * x.nh * y.nh;
+  if (total == 0) return hipSuccess;
+  i64 blocks = (total + 255) / 256;
+  if (blocks > (1 << 20)) blocks = 1 << 20;
+  // the 32-bit path: every numerator of the tap relations and the flat index below 2^22 / 2^32
+  const auto small_axis = [](const Axis &a) {
+    const i64 lim = (i64)1 << 22;
+    return (a.nh + a.s) * (a.nf + a.d) < lim && (a.p + 1) * (a.nh + a.s) < lim &&
+           a.s * a.nh + a.d * a.nf + (a.p < 0 ? -a.p : a.p) < lim && a.u < lim && a.p + 1 < lim && a.nf + a.d < lim;
+  };
+  const bool small = small_axis(x) && small_axis(y) && total < ((i64)1 << 32);
+  const i64 row_blocks = batch_cin * ((x.nh + 31) / 32);
+  if (small && x.nf <= 64 && y.nf <= 8 && row_blocks < ((i64)1 << 31) && batch_cin < ((i64)1 << 24) &&
+      (i64)nf_pad * x.ng * y.ng < ((i64)1 << 30))
+    hipLaunchKernelGGL(fold_xy_rows_kernel, dim3((unsigned)row_blocks), dim3(256), 0, stream, x, y,
+                       (int)batch_cin, nf_pad, Z, grad_input);
+  else if (small)
+    hipLaunchKernelGGL(fold_xy_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, x, y, batch_cin,
+                       nf_pad, Z, grad_input);
+  else
+    hipLaunchKernelGGL(fold_xy_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, x, y, batch_cin,
+                       nf_pad, Z, grad_input);
+  return hipGetLastError();
+}
 
 hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
                          float *grad_input, hipStream_t stream) {

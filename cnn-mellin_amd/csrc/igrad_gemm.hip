@@ -442,7 +442,170 @@ hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go,
   return hipGetLastError();
 }
 
+// Tap products for the gather-fold input gradient (any x axis kind):
+//   Z[n, ci, m, q] = sum_co w[co, ci, m] * grad_out[n, co, q]
+// Same operands, staging and work split over wavefronts as above; the
+// accumulators are stored instead of folded.  A workgroup takes pl.cpw chunks
+// of 64 positions of pl.jobs consecutive images.
+template <int KSTEPS>
+__global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan pl,
+                                                          const float *__restrict__ W,
+                                                          const float *__restrict__ GO,
+                                                          float *__restrict__ Z) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int K = 2 * KSTEPS, P = 64, NT = 2, KH = K / 2;
+  const int wave_in_group = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int job = wave_in_group / pl.units;
+  const int wave = wave_in_group - job * pl.units;
+  const int lane = threadIdx.x & 63;
+  const int tid = wave * 64 + lane, nthreads = pl.units * 64;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int groups_x = (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
+  const int image_group = blockIdx.x / groups_x, chunk_group = blockIdx.x - image_group * groups_x;
+  const int n_want = image_group * pl.jobs + job;
+  const bool active = n_want < pl.batch;
+  const int n = active ? n_want : pl.batch - 1;
+  const int c_first = chunk_group * pl.cpw;
+  const int nchunks = min(pl.cpw, pl.chunks_per_image - c_first);
+  float *Bs = lds + job * K * P;
+  const unsigned bs_addr = lds_address(lds) + 4u * (unsigned)(job * K * P);
+
+  // channels past c_out and positions past the image are never loaded: keep them finite
+  if ((c_first + nchunks) * P > pl.nh) {
+    for (int i = tid; i < K * P; i += nthreads) Bs[i] = 0.f;
+  } else {
+    for (int i = pl.c_out * P + tid; i < K * P; i += nthreads) Bs[i] = 0.f;
+  }
+  const int ci = wave / pl.mtn, mt = wave - ci * pl.mtn;
+  float areg[KSTEPS];
+  {
+    const int m = mt * 32 + l32;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int k = 2 * s + half;
+      areg[s] = (k < pl.c_out && m < pl.nf) ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : 0.f;
+    }
+  }
+  const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
+  const int row_in = lane >> 4, seg = lane & 15;          // 16 lanes x 16 bytes per channel row
+  auto issue = [&](int c, int k_lo) {                     // channels [k_lo, k_lo + KH) of chunk c
+    const int q0 = c * P;
+    const int k_hi = min(k_lo + KH, pl.c_out);
+    if (q0 + P <= pl.nh) {
+      for (int k0 = k_lo + wave * 4; k0 < k_hi; k0 += pl.units * 4) {
+        const int k = k0 + row_in;
+        const unsigned voff = (unsigned)(row_in * pl.nh + q0 + 4 * (seg ^ ((k & 1) << 3))) * 4u;
+        if (k < k_hi) load16_to_lds_at(GOn + (i64)k0 * pl.nh, voff, bs_addr + 4u * (unsigned)(k0 * P));
+      }
+    } else {
+      for (int k = k_lo + wave; k < k_hi; k += pl.units) {
+        const int q = q0 + (lane ^ ((k & 1) << 5));
+        if (q < pl.nh) load_to_lds_at(GOn + (i64)k * pl.nh, (unsigned)q * 4u, bs_addr + 4u * (unsigned)(k * P));
+      }
+    }
+  };
+  int bo[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) bo[t] = half * P + ((t ^ half) << 5) + l32;
+  // rows of Z this lane stores: tap m(r) of input channel ci
+  float *Zrow = Z + ((i64)(n * pl.c_in + ci) * pl.nf_pad + mt * 32 + half * 4) * pl.nh;
+  const int m_base = mt * 32 + half * 4;
+
+  __syncthreads();
+  issue(c_first, 0);
+  issue(c_first, KH);
+  for (int c = 0; c < nchunks; ++c) {
+    wait_all_memory();
+    __syncthreads();
+    floatx16 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KSTEPS / 2; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
+    __syncthreads();                                   // the first half is free
+    if (c + 1 < nchunks) issue(c_first + c + 1, 0);
+#pragma unroll
+    for (int s = KSTEPS / 2; s < KSTEPS; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
+    __syncthreads();                                   // the second half is free
+    if (c + 1 < nchunks) issue(c_first + c + 1, KH);
+    if (active) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int q = (c_first + c) * P + t * 32 + l32;
+        if (q < pl.nh) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int dm = (r >> 2) * 8 + (r & 3);
+            if (m_base + dm < pl.nf) Zrow[(i64)dm * pl.nh + q] = acc[t][r];
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int KSTEPS>
+hipError_t launch_tap_product_instance(const TapProductPlan &pl, const float *w, const float *go,
+                                       float *z, hipStream_t stream) {
+  auto kern = tap_product_kernel<KSTEPS>;
+  if (pl.lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)pl.lds_bytes);
+    if (e != hipSuccess) return e;
+  }
+  const int groups_x = (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
+  const int image_groups = (pl.batch + pl.jobs - 1) / pl.jobs;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(image_groups * groups_x)), dim3(64 * pl.units * pl.jobs),
+                     pl.lds_bytes, stream, pl, w, go, z);
+  return hipGetLastError();
+}
+
 }  // namespace
+
+bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 nhx, i64 nhy,
+                           TapProductPlan &pl) {
+  const i64 nf = nfx * nfy, nh = nhx * nhy;
+  if (batch < 1 || c_in < 1 || c_out < 1 || nf < 1 || nh < 1) return false;
+  const i64 lim = (i64)1 << 28;
+  if (nh >= lim || c_out * c_in * nf >= lim || batch * c_in >= lim) return false;
+  const i64 mtn = (nf + 31) / 32, units = c_in * mtn;
+  // few input channels, and taps that fill their 32-row tiles reasonably
+  if (c_in >= 16 || units > 8 || mtn * 32 * 2 > nf * 3 || c_out > 128) return false;
+  pl.batch = (int)batch; pl.c_in = (int)c_in; pl.c_out = (int)c_out;
+  pl.nf = (int)nf; pl.nh = (int)nh;
+  pl.mtn = (int)mtn; pl.units = (int)units; pl.nf_pad = (int)mtn * 32;
+  pl.ksteps = c_out <= 32 ? 16 : c_out <= 64 ? 32 : 64;
+  const int max_waves = pl.ksteps == 64 ? 8 : 12;
+  if (units > max_waves) return false;
+  pl.jobs = 1;
+  for (int j = 1; j <= 4; ++j)
+    if ((j * units) % 4 == 0 && j * units <= max_waves && j <= batch) { pl.jobs = j; break; }
+  pl.chunks_per_image = (int)((nh + 63) / 64);
+  // chunks per workgroup: about two workgroups per CU in all, at least two chunks each
+  const i64 image_groups = (batch + pl.jobs - 1) / pl.jobs;
+  i64 cpw = (image_groups * pl.chunks_per_image + 511) / 512;
+  pl.cpw = (int)std::max<i64>(2, std::min<i64>(cpw, pl.chunks_per_image));
+  pl.lds_bytes = 4 * (size_t)(2 * pl.ksteps * 64) * pl.jobs;
+  pl.ws_bytes = 4 * (size_t)batch * c_in * pl.nf_pad * nh;
+  if (image_groups * ((pl.chunks_per_image + pl.cpw - 1) / pl.cpw) >= ((i64)1 << 31)) return false;
+  return true;
+}
+
+hipError_t launch_tap_product(const TapProductPlan &pl, const float *weight, const float *grad_out,
+                              float *z, hipStream_t stream) {
+  if (pl.ksteps == 16) return launch_tap_product_instance<16>(pl, weight, grad_out, z, stream);
+  if (pl.ksteps == 32) return launch_tap_product_instance<32>(pl, weight, grad_out, z, stream);
+  if (pl.ksteps == 64) return launch_tap_product_instance<64>(pl, weight, grad_out, z, stream);
+  return hipErrorInvalidValue;
+}
 
 bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                      i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,

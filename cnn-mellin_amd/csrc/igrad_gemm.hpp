@@ -40,4 +40,22 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
                         float *grad_input, float *workspace, hipStream_t stream);
 
+// Tap products of the input gradient for layers with few input channels, any x
+// axis kind: Z[n, ci, m, hx, hy] = sum_co w[co, ci, m] * grad_out[n, co, hx, hy]
+// for every tap m = fx * nfy + fy (rows padded to a multiple of 32 per input
+// channel; padded rows are not written).  A gather (fold_x.hip) finishes.
+struct TapProductPlan {
+  int batch, c_in, c_out, nf, nh;
+  int mtn, units, jobs, ksteps;
+  int chunks_per_image, cpw;         // 64-position chunks; chunks per workgroup
+  int nf_pad;                        // mtn * 32
+  size_t lds_bytes, ws_bytes;        // ws: Z
+};
+
+bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 nhx, i64 nhy,
+                           TapProductPlan &pl);
+
+hipError_t launch_tap_product(const TapProductPlan &pl, const float *weight, const float *grad_out,
+                              float *z, hipStream_t stream);
+
 }  // namespace mellin

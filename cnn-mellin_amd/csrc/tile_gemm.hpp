@@ -52,13 +52,15 @@ struct WgradPlan {
   int S;                           // position shares = persistent workgroups per output block
   int rows_mode;                   // 1: the row-wise kernel (one output row per wavefront)
   int nbuf;                        // row-wise kernel: LDS buffers per operand (1 or 2)
+  int rpw;                         // row-wise kernel: output rows per wavefront and unit
   size_t lds_bytes, ws_bytes;
 };
 
 // allow_rows = false rules the row-wise kernel out (for comparisons)
-// rows_mt / rows_nbuf: channel tiles per workgroup and buffers of the row-wise kernel
-bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool allow_rows = true, int rows_mt = 1,
-                     int rows_nbuf = 2);
+// rows_mt / rows_nbuf / rows_rpw pin the row-wise kernel's channel tiles per
+// workgroup, buffers, and output rows per wavefront and unit (0 = automatic)
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool allow_rows = true, int rows_mt = 0,
+                     int rows_nbuf = 0, int rows_rpw = 0);
 
 hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float *input,
                         float *grad_weight, float *workspace, hipStream_t stream);

@@ -228,7 +228,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     float *__restrict__ ws) {
   extern __shared__ __align__(16) float lds[];
   const TilePlan &pl = wp.t;
-  constexpr int M_T = MT * 32, J_T = JT * 32, RB = kWaves;
+  constexpr int M_T = MT * 32, J_T = JT * 32;
+  const int RB = kWaves * wp.rpw;                    // output rows per unit
   const int x_words = (wp.CCj * pl.R * pl.RS + 3) & ~3;
   const int a_words = M_T * wp.GSS;
   float *Xs0 = lds;                                  // [nbuf][CCj][R][RS]
@@ -322,15 +323,15 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
   auto multiply_unit = [&](int ui) {
     const int unit = blockIdx.x + ui * gridDim.x;
     const int ox_lo = (unit % units_per_image) * RB;
-    if (ox_lo + wave < pl.nox_eff) {                     // this wavefront's row exists
+    for (int row = wave; row < RB && ox_lo + row < pl.nox_eff; row += kWaves) {   // this wavefront's rows
       const int b = wp.nbuf == 2 ? (ui & 1) : 0;
       const float *Xs = Xs0 + b * x_words;
       const float *As = As0 + b * a_words;
-      int ao = l32 * wp.GSS + wave * pl.noy + half;
+      int ao = l32 * wp.GSS + row * pl.noy + half;
       int bo[JT];
 #pragma unroll
       for (int t = 0; t < JT; ++t)
-        bo[t] = col_off[t] + (pl.Ax * wave + pl.Cx0) * pl.RS - pl.by_min + half;
+        bo[t] = col_off[t] + (pl.Ax * row + pl.Cx0) * pl.RS - pl.by_min + half;
       int s = 0;
       for (; s + 8 <= pairs; s += 8) {
 #pragma unroll
@@ -497,7 +498,8 @@ hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const flo
 
 // Plan the weight gradient of the layer whose FORWARD problem is `fwd`
 // (filter = weight, signal = input, output = grad_out, write mode).
-bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf) {
+bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf,
+                     int rows_opt_rpw) {
   size_t lds_fwd;
   int mt, nt;
   // 128 positions per tile: the staged grad_out tile (channels x positions, two
@@ -518,34 +520,41 @@ bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int r
   wp.nt = nt;
   wp.rows_mode = 0;
   if (!pl.segment && pl.ay == 1 && pl.noy >= 16 && pl.nox_eff >= 1 && g_allow_rows) {
-    // row-wise variant: units of kWaves output rows
+    // Row-wise variant: units of kWaves * rpw output rows.  Preferred shape: two
+    // rows per wavefront and a single buffer (several workgroups per CU cover each
+    // other's loads); then one row per wavefront with two buffers, then with one.
     const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
-    const int rb = std::min<int>(kWaves, pl.nox);
-    const i64 Rr = mellin_x ? (i64)rb * pl.nfx : (i64)pl.ax * (rb - 1) + pl.bx_span + 1;
-    int pitch = (kWaves * pl.noy + 3) & ~3;
-    if (((pitch >> 2) & 1) == 0) pitch += 4;              // 4 x odd: channels spread over the banks
     const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
-    const size_t xw = ((size_t)ccj * Rr * pl.RS + 3) & ~(size_t)3;
-    // all channels in one workgroup (two 32-row tiles) when they fit: the input is then staged once
-    int mt_rows = (pl.M > 32 && rows_opt_mt == 2) ? 2 : 1;
-    const int nbuf = rows_opt_nbuf;
-    size_t bytes = 4 * std::max(nbuf * (xw + (size_t)mt_rows * 32 * pitch), (size_t)mt_rows * 32 * J_T);
-    if (mt_rows == 2 && bytes > 150 * 1024) {
-      mt_rows = 1;
-      bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), (size_t)32 * J_T);
-    }
-    if (Rr <= 8192 && bytes <= (mt_rows == 2 ? 150 : 78) * 1024) {
-      wp.nbuf = nbuf;
+    const int shapes[3][2] = {{2, 1}, {1, 2}, {1, 1}};   // {rows per wavefront, buffers}
+    for (const auto &shape : shapes) {
+      const int rpw = rows_opt_rpw > 0 ? rows_opt_rpw : shape[0];
+      const int nbuf = rows_opt_nbuf > 0 ? rows_opt_nbuf : shape[1];
+      const int rb = kWaves * rpw;
+      const i64 Rr = mellin_x ? (i64)rb * pl.nfx : (i64)pl.ax * (rb - 1) + pl.bx_span + 1;
+      int pitch = (rb * pl.noy + 3) & ~3;
+      if (((pitch >> 2) & 1) == 0) pitch += 4;            // 4 x odd: channels spread over the banks
+      const size_t xw = ((size_t)ccj * Rr * pl.RS + 3) & ~(size_t)3;
+      // all channels in one workgroup (two 32-row tiles) only on request: fewer, fatter
+      // workgroups have measured slower
+      int mt_rows = (pl.M > 32 && rows_opt_mt == 2) ? 2 : 1;
+      size_t bytes = 4 * std::max(nbuf * (xw + (size_t)mt_rows * 32 * pitch), (size_t)mt_rows * 32 * J_T);
+      if (mt_rows == 2 && bytes > 150 * 1024) {
+        mt_rows = 1;
+        bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), (size_t)32 * J_T);
+      }
+      if (Rr > 8192 || pitch * 32 * 4 >= 65536 || bytes > (mt_rows == 2 ? 150 : 78) * 1024) continue;
       wp.rows_mode = 1;
       pl.R = (int)Rr;
       wp.GSS = pitch;
       wp.CCj = ccj;
       wp.lds_bytes = bytes;
+      wp.nbuf = nbuf;
+      wp.rpw = rpw;
       wp.mt = mt_rows;
       wp.m_groups = (pl.M + mt_rows * 32 - 1) / (mt_rows * 32);
       wp.M_pad = wp.m_groups * mt_rows * 32;
       const int blocks_y_rows = wp.m_groups * wp.j_groups;
-      const i64 units = (i64)pl.batch * ((pl.nox_eff + kWaves - 1) / kWaves);
+      const i64 units = (i64)pl.batch * ((pl.nox_eff + rb - 1) / rb);
       int per_cu = std::max(1, std::min((int)((160 * 1024) / (bytes + 512)), nbuf == 2 ? 4 : 6));
       i64 S = std::max<i64>(1, (256 * per_cu) / blocks_y_rows);
       wp.S = (int)std::min<i64>(S, units);

@@ -103,3 +103,35 @@ def test_fused_is_run_to_run_deterministic():
     for _ in range(3):
         again, _ = _grad_input(hip.AX_LCORR, w, go, (4, 3, 128, 41), (1, 1), (1, 1), (0, 0), (1, 1), None)
         assert torch.equal(first, again)
+
+
+MELLIN_CASES = [
+    # (kind, n, c_in, c_out, nf, ng, s, d, p, u, r)
+    ("mcorr", 2, 3, 64, (8, 4), (96, 41), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),     # the benchmark layer, shortened
+    ("mcorr", 3, 1, 7, (5, 5), (40, 29), (1, 1), (2, 1), (1, 1), (2, 1), (0, 0)),      # s, d, p, u on the Mellin axis
+    ("mcorr", 2, 2, 100, (6, 4), (33, 20), (2, 2), (1, 2), (0, 3), (1, 1), (3, 1)),    # rows past the support, y stride
+    ("lcorr", 2, 4, 33, (4, 7), (30, 25), (1, 1), (2, 1), (3, 2), (2, 3), (0, 0)),     # linear x with up-sampling: no fused kernel
+    ("mcorr", 1, 3, 16, (7, 8), (50, 30), (1, 1), (1, 1), (2, 0), (1, 2), (0, 0)),     # two tap tiles per channel
+]
+
+
+@pytest.mark.parametrize("case", MELLIN_CASES, ids=[str(i) for i in range(len(MELLIN_CASES))])
+def test_tap_product_and_two_pass_match_checker(case):
+    kind, n, c_in, c_out, nf, ng, s, d, p, u, r = case
+    kind_x = hip.AX_MCORR if kind == "mcorr" else hip.AX_LCORR
+    fwd = oracle.mcorrlcorr if kind == "mcorr" else oracle.lcorrlcorr
+    bwd = oracle.mcorrlcorr_backward if kind == "mcorr" else oracle.lcorrlcorr_backward
+    rng = np.random.default_rng(500 + MELLIN_CASES.index(case))
+    x = np.zeros((n, c_in) + ng, dtype=np.float32)
+    w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+    nh = fwd(x, w, None, s, d, p, u, r).shape[2:]
+    assert min(nh) > 0
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    exp, _, _ = bwd(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64), s, d, p, u)
+    fan_in = c_out * nf[0] * nf[1]
+    got, v1 = _grad_input(kind_x, w, go, (n, c_in) + ng, s, d, p, u, None)
+    assert v1 == "mfma-taps+fold", v1
+    assert_close(got, exp, fan_in, "taps %s" % (case,))
+    other, v2 = _grad_input(kind_x, w, go, (n, c_in) + ng, s, d, p, u, "two-pass")
+    assert v2 != "mfma-taps+fold", v2
+    assert_close(other, exp, fan_in, "%s %s" % (v2, case))
