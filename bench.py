@@ -10,8 +10,11 @@ s = d = u = 1, p = 0, fp32, inputs resident in HBM before the clock starts.
 Prints one JSON line.  `value` is algorithmic GB/s (each operand read once,
 each result written once) over the whole step; `frames_per_s` counts the
 32 x 512 input frames once per step.  `roofline` describes the pass that takes
-the longest, timed with HIP events on the launch stream; `cpu_baseline` times
-the CPU checker on a bounded slice of the same batch on the host cores.
+the longest, timed with HIP events on the launch stream: against the fp32
+matrix peak when its arithmetic intensity (algorithmic FLOP per algorithmic
+byte) is above the machine's ridge point, against the HBM peak otherwise, with
+the other figure alongside.  `cpu_baseline` times the CPU checker on the same
+batch on the host cores.
 """
 import argparse
 import json
@@ -26,6 +29,21 @@ for _p in (ROOT, os.path.join(ROOT, "cnn-mellin_amd")):
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3     # MI355X fp32 matrix (MFMA) = packed vector fp32, published
+
+# HBM bytes per launch of each pass at this workload, measured with
+#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 3 --warmup 1 --no-cpu
+#   rocprofv3 --pmc WRITE_SIZE -- python3 bench.py --steps 3 --warmup 1 --no-cpu
+# (KiB per dispatch, summed over the kernels of the pass) and scaled by what the same
+# counters read for a plain 256 MiB device copy (--copy-calibration): FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0.  The summary is kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "mconv2d.forward": 35.3e6, "mconv2d.grad_input": 90.9e6, "mconv2d.grad_weight": 51.6e6,
+    "lconv2d.forward": 217.1e6, "lconv2d.grad_input": 190.2e6, "lconv2d.grad_weight": 218.4e6,
+}
+MEASURED_TRAFFIC_VARIANTS = {
+    "mconv2d.forward": "mfma", "mconv2d.grad_input": "mfma-taps+fold", "mconv2d.grad_weight": "mfma-rows",
+    "lconv2d.forward": "mfma", "lconv2d.grad_input": "mfma-fused", "lconv2d.grad_weight": "mfma-rows",
+}
 
 CFG = dict(batch=32, c_in=3, c_out=64, ngx=512, ngy=41, nfx=8, nfy=4,
            s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1))
@@ -124,7 +142,7 @@ def time_pass(fn, reps, torch):
     return start.elapsed_time(stop) * 1e3 / reps
 
 
-def cpu_baseline(layers, slice_n, reps=3):
+def cpu_baseline(layers, slice_n, reps=25):
     """The CPU checker (restatement of the reference's OpenMP kernels) on the first
     `slice_n` utterances of the same batch: forward + both gradients of both layers."""
     import numpy as np
@@ -148,8 +166,9 @@ def cpu_baseline(layers, slice_n, reps=3):
                  for L in layers)
     return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": min(threads, cores),
             "kind": "port",
-            "sample": "same step on utterances 0..%d of 32 (%.0f MB algorithmic), median of %d, %.2f s each; "
-                      "%.0f frames/s" % (slice_n - 1, nbytes / 1e6, reps, med, slice_n * CFG["ngx"] / med),
+            "sample": "same step on utterances 0..%d of 32 (%.0f MB algorithmic), median of %d repetitions "
+                      "(%.1f s of CPU work in all), %.2f s each; %.0f frames/s"
+                      % (slice_n - 1, nbytes / 1e6, reps, sum(times), med, slice_n * CFG["ngx"] / med),
             "frames_per_s": round(slice_n * CFG["ngx"] / med, 1)}
 
 
@@ -219,6 +238,21 @@ def main():
     dom_us = per_pass[dom]
     achieved_gbs = domL.bytes_per_pass / dom_us / 1e3
     dom_tflops = 2 * domL.macs_per_pass / dom_us / 1e6
+    # which roof: arithmetic intensity against the ridge point of the two peaks
+    intensity = 2 * domL.macs_per_pass / domL.bytes_per_pass
+    ridge = FP32_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS
+    traffic = MEASURED_TRAFFIC_BYTES.get(dom) if variants[dom] == MEASURED_TRAFFIC_VARIANTS.get(dom) else None
+    if intensity > ridge:
+        roof = {"bound": "mfma", "achieved": round(dom_tflops, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(dom_tflops / FP32_PEAK_TFLOPS, 4)}
+    else:
+        roof = {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved_gbs / HBM_PEAK_GBS, 4)}
+    roof.update({"traffic": traffic, "kernel": dom, "variant": variants[dom], "avg_us": round(dom_us, 2),
+                 "flop_per_byte": round(intensity, 1), "ridge_flop_per_byte": round(ridge, 1),
+                 "algorithmic_bytes": domL.bytes_per_pass, "algorithmic_flops": 2 * domL.macs_per_pass,
+                 "hbm_GBps": round(achieved_gbs, 1), "hbm_frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
+                 "fp32_TFLOPs": round(dom_tflops, 2), "fp32_frac": round(dom_tflops / FP32_PEAK_TFLOPS, 4)})
 
     line = {
         "metric": "mconv2d+lconv2d fwd+bwd GB/s and frames/sec on 1 MI355X; % HBM roofline",
@@ -236,15 +270,16 @@ def main():
         "frames_per_s": round(frames / (elapsed / args.steps), 1),
         "pct_hbm_roofline": round(100.0 * step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS, 2),
         "tflops": round(step_flops / (elapsed / args.steps) / 1e12, 2),
-        "roofline": {"bound": "hbm", "kernel": dom, "variant": variants[dom],
-                     "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "avg_us": round(dom_us, 2),
-                     "fp32_tflops": round(dom_tflops, 2),
-                     "fp32_frac": round(dom_tflops / FP32_PEAK_TFLOPS, 4)},
+        "roofline": roof,
         "per_pass_us": {k: round(v, 2) for k, v in per_pass.items()},
         "per_pass_variant": variants,
     }
+    line["per_pass_roofline"] = {
+        k: {"hbm_frac": round((layers[0] if k.startswith("mconv2d") else layers[1]).bytes_per_pass / v / 1e3
+                              / HBM_PEAK_GBS, 4),
+            "fp32_frac": round(2 * (layers[0] if k.startswith("mconv2d") else layers[1]).macs_per_pass / v / 1e6
+                               / FP32_PEAK_TFLOPS, 4)}
+        for k, v in per_pass.items()}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(layers, args.cpu_slice)
     print(json.dumps(line))
