@@ -119,11 +119,13 @@ MELLIN_DECL_2D(mellin_lconvlconv_f64, double);
  * y axis (nfy = ngy = nhy = 1, sy = dy = uy = 1, py = 0).
  *
  * The backward passes may need scratch memory (partial sums of the weight
- * gradient; the intermediate of the two-pass input gradient used for layers
- * with few input channels): ask mellin_corr2d_backward_*_workspace() for the
- * byte count (0 = none) and pass a device buffer of at least that size
- * (256-byte aligned); its contents on entry do not matter and are garbage on
- * exit.
+ * gradient; for layers with few input channels the partial rows, the tap
+ * products or the first-pass result of the input gradient): ask
+ * mellin_corr2d_backward_*_workspace() for the byte count (0 = none) and pass
+ * a device buffer of at least that size (256-byte aligned); its contents on
+ * entry do not matter and are garbage on exit.  The count depends on the
+ * variant in force on the calling thread (mellin_set_variant): query and call
+ * under the same setting.
  * ------------------------------------------------------------------------ */
 #define MELLIN_CORR2D_DIMS                                                     \
   int64_t batch, int64_t c_in, int64_t c_out, int64_t nfx, int64_t nfy,        \
@@ -160,12 +162,18 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       size_t workspace_bytes, void *stream);
 
 /* Name of the kernel variant the most recent operator-level call on this
- * thread dispatched to (for tests and profiling), e.g. "generic". */
+ * thread dispatched to (for tests and profiling): "generic", "mfma" (tiled
+ * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"
+ * (one-kernel input gradient, linear x axis, few input channels),
+ * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
+ * (two-pass input gradient). */
 const char *mellin_last_variant(void);
 
 /* Force a variant for subsequent operator-level calls on this thread:
- * NULL or "" = automatic choice; "generic" = the one-thread-per-output
- * kernels.  Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
+ * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
+ * kernels; "two-pass" = automatic choice without the specialised gradient
+ * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows"), i.e. the tiled ones.
+ * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);
 
 #ifdef __cplusplus
