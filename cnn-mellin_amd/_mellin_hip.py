@@ -33,6 +33,8 @@ _SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
 _ACC1D = [_ptr, _ptr] + [_i64] * 10 + [_int] * 3 + [_ptr, _ptr]
 _ACC2D = [_ptr, _ptr] + [_i64] * 17 + [_int] * 3 + [_ptr, _ptr]
 _DIMS = [_i64] * 17
+_SND = [_ptr] + [_i64] * 9 + [_int] * 2 + [_ptr, _ptr]
+_SPEC = [_ptr] + [_i64] * 16 + [_int] * 2 + [_ptr, _ptr]
 SYMBOLS = {
     "mellin_version": (_int, []),
     "mellin_last_error": (ctypes.c_char_p, []),
@@ -46,6 +48,10 @@ for _t in ("f32", "f64"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC1D)
     for _n in ("mcorrlcorr", "mconvlconv", "lcorrlcorr", "lconvlconv"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC2D)
+    for _n in ("snd2col", "col2snd"):
+        SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _SND)
+    for _n in ("spec2col", "col2spec"):
+        SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _SPEC)
     SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_backward_input_" + _t] = (
         _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
@@ -122,6 +128,21 @@ def accumulate(name, f, g, h, c_out, c_in, batch, nf, ng, nh, s, d, p, u, tf, tg
                       int(tf), int(tg), int(th), _dp(h), _stream(dev))
     _check(code)
     return h
+
+
+def col_op(name, src, dst, c_in, batch, nf, ng, ngg, s, d, p, u, tg, tgg):
+    """snd2col / col2snd (ints) or spec2col / col2spec (pairs): `src` -> `dst`, both dense."""
+    dev = require_device(src, dst)
+    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(dst.dtype)))
+    with torch.cuda.device(dev):
+        if isinstance(nf, int):
+            code = fn(_dp(src), c_in, batch, nf, ng, ngg, s, d, p, u, int(tg), int(tgg), _dp(dst),
+                      _stream(dev))
+        else:
+            code = fn(_dp(src), c_in, batch, nf[0], nf[1], ng[0], ng[1], ngg[0], ngg[1], s[0], s[1],
+                      d[0], d[1], p[0], p[1], u[0], u[1], int(tg), int(tgg), _dp(dst), _stream(dev))
+    _check(code)
+    return dst
 
 
 def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):

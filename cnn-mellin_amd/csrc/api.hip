@@ -327,7 +327,55 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
                                                (hipStream_t)stream), fn);
 }
 
+// Column ops (mconv.h:1247-1380): x Mellin correlation, y linear correlation.
+template <typename T>
+int col_op(const char *fn, bool to_col, const T *src, i64 c_in, i64 batch, i64 nfx, i64 nfy,
+           i64 ngx, i64 ngy, i64 nggx, i64 nggy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
+           i64 ux, i64 uy, int transposed_g, int transposed_gg, T *dst, void *stream) {
+  int rc = check_channels(fn, 0, c_in, batch);
+  if (!rc) rc = check_axis(fn, "x", AX_MCORR, nfx, ngx, nggx, sx, dx, px, ux);
+  if (!rc) rc = check_axis(fn, "y", AX_LCORR, nfy, ngy, nggy, sy, dy, py, uy);
+  if (rc) return rc;
+  const i64 n_g = batch * c_in * ngx * ngy, n_gg = batch * c_in * nfx * nfy * nggx * nggy;
+  if ((to_col ? n_gg : n_g) == 0) return MELLIN_OK;
+  if (!dst || ((to_col ? n_g : n_gg) != 0 && !src))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e;
+  if (to_col) {
+    const Axis x = make_axis(AX_MCORR, nfx, ngx, nggx, sx, dx, px, ux);
+    const Axis y = make_axis(AX_LCORR, nfy, ngy, nggy, sy, dy, py, uy);
+    e = launch_spec2col<T>(x, y, c_in, batch, transposed_g, transposed_gg, src, dst, (hipStream_t)stream);
+  } else {
+    // inverse relations: the convolution kinds with s and u exchanged (mconv.h:1294-1298, :1362-1372)
+    const Axis x = make_axis(AX_MCONV, nfx, nggx, ngx, ux, dx, px, sx);
+    const Axis y = make_axis(AX_LCONV, nfy, nggy, ngy, uy, dy, py, sy);
+    e = launch_col2spec<T>(x, y, c_in, batch, transposed_g, transposed_gg, src, dst, (hipStream_t)stream);
+  }
+  return check_hip(e, fn);
+}
+
 }  // namespace
+
+#define DEFINE_SND(NAME, T, SRC, DST, TO_COL)                                   \
+  MELLIN_DECL_SND(NAME, T, SRC, DST) {                                          \
+    return col_op<T>(#NAME, TO_COL, SRC, c_in, batch, nf, 1, ng, 1, ngg, 1, s,  \
+                     1, d, 1, p, 0, u, 1, transposed_g, transposed_gg, DST,    \
+                     stream);                                                  \
+  }
+#define DEFINE_SPEC(NAME, T, SRC, DST, TO_COL)                                  \
+  MELLIN_DECL_SPEC(NAME, T, SRC, DST) {                                         \
+    return col_op<T>(#NAME, TO_COL, SRC, c_in, batch, nfx, nfy, ngx, ngy, nggx, \
+                     nggy, sx, sy, dx, dy, px, py, ux, uy, transposed_g,       \
+                     transposed_gg, DST, stream);                              \
+  }
+DEFINE_SND(mellin_snd2col_f32, float, g, gg, true)
+DEFINE_SND(mellin_snd2col_f64, double, g, gg, true)
+DEFINE_SND(mellin_col2snd_f32, float, gg, g, false)
+DEFINE_SND(mellin_col2snd_f64, double, gg, g, false)
+DEFINE_SPEC(mellin_spec2col_f32, float, g, gg, true)
+DEFINE_SPEC(mellin_spec2col_f64, double, g, gg, true)
+DEFINE_SPEC(mellin_col2spec_f32, float, gg, g, false)
+DEFINE_SPEC(mellin_col2spec_f64, double, gg, g, false)
 
 #define CORR2D_ARGS                                                            \
   batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \

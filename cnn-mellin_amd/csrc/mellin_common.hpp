@@ -90,6 +90,13 @@ hipError_t launch_sepreduce_generic(const SepReduce &pr, const T *a, const T *g,
 hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
                          float *grad_input, hipStream_t stream);
 
+template <typename T>
+hipError_t launch_spec2col(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
+                           int transposed_gg, const T *g, T *gg, hipStream_t stream);
+template <typename T>
+hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
+                           int transposed_gg, const T *gg, T *g, hipStream_t stream);
+
 hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
                           float *grad_input, hipStream_t stream);
 

@@ -310,12 +310,80 @@ def _raw_mcorrlcorr(input, weight, bias=None, s=(1, 1), d=(1, 1), p=(0, 0), u=(1
     return _raw_op("mcorrlcorr", (AX_MCORR, AX_LCORR), input, weight, bias, s, d, p, u, r)
 
 
+# ---------------------------------------------------------------------------
+# column ops (Snd2ColOp / Spec2ColOp, ext/torch.cpp:310-389; adapters
+# ext/torch_cuda.cu:179-291): the gather behind the reference's "mm" path
+# ---------------------------------------------------------------------------
+def _check_col_args(c: str, dim: int, input: torch.Tensor):
+    """CheckAndInferArgumentsCol (ext/torch.cpp:57-85): returns (batch, c_in)."""
+    _check_dim(c, input, "input", 1, dim)
+    return input.size(0), input.size(1)
+
+
+class _ToColFunction(torch.autograd.Function):
+    """gg = x2col(input); backward is col2x (the adjoint gather)."""
+
+    @staticmethod
+    def forward(ctx, input, nf, s, d, p, u, r, name):
+        dim = len(nf)
+        batch, c_in = _check_col_args(name, dim + 2, input)
+        ng = tuple(input.shape[2:])
+        kinds = (_hip.AX_MCORR, _hip.AX_LCORR)[:dim]
+        ngg = tuple(_VALID_SIZE[k](nf[i], ng[i], s[i], d[i], p[i], u[i]) + r[i]
+                    for i, k in enumerate(kinds))
+        g, tg = _dense_or_transposed(input)
+        gg = input.new_empty((batch, c_in) + tuple(nf) + ngg)
+        ctx.args = (nf, ng, ngg, s, d, p, u, dim)
+        if gg.numel():
+            if dim == 1:
+                _hip.col_op("snd2col", g, gg, c_in, batch, nf[0], ng[0], ngg[0], s[0], d[0], p[0], u[0],
+                            tg, False)
+            else:
+                _hip.col_op("spec2col", g, gg, c_in, batch, nf, ng, ngg, s, d, p, u, tg, False)
+        return gg
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        nf, ng, ngg, s, d, p, u, dim = ctx.args
+        grad_input = _from_col(grad_out, ng, s, d, p, u, dim)
+        return (grad_input,) + (None,) * 7
+
+
+def _from_col(cols, ng, s, d, p, u, dim):
+    """col2snd / col2spec (ext/torch_cuda.cu:208-235, :267-291)."""
+    name = "col2snd" if dim == 1 else "col2spec"
+    batch, c_in = _check_col_args(name, 2 + 2 * dim, cols)
+    nf = tuple(cols.shape[2:2 + dim])
+    ngg = tuple(cols.shape[2 + dim:])
+    gg, tgg = _dense_or_transposed(cols)
+    g = cols.new_empty((batch, c_in) + tuple(ng))
+    if g.numel():
+        if dim == 1:
+            _hip.col_op(name, gg, g, c_in, batch, nf[0], ng[0], ngg[0], s[0], d[0], p[0], u[0], False, tgg)
+        else:
+            _hip.col_op(name, gg, g, c_in, batch, nf, tuple(ng), ngg, s, d, p, u, False, tgg)
+    return g
+
+
 def _ext_snd2col(input, kernel_width, s=1, d=1, p=0, u=1, r=0):
-    raise NotImplementedError("snd2col is not built yet in this package")
+    """``torch.ops.mellin.snd2col`` (ext/torch.cpp:473): (N, C, T) -> (N, C, K, T_out)."""
+    return _ToColFunction.apply(input, (kernel_width,), (s,), (d,), (p,), (u,), (r,), "snd2col")
+
+
+def _ext_col2snd(input, snd_width, s=1, d=1, p=0, u=1):
+    """``torch.ops.mellin.col2snd`` (ext/torch.cpp:474): the adjoint of snd2col, no autograd."""
+    return _from_col(input, (snd_width,), (s,), (d,), (p,), (u,), 1)
 
 
 def _ext_spec2col(input, kernel_size, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1), r=(0, 0)):
-    raise NotImplementedError("spec2col is not built yet in this package")
+    """``torch.ops.mellin.spec2col`` (ext/torch.cpp:475): (N, C, T, F) -> (N, C, Kx, Ky, T_out, F_out)."""
+    return _ToColFunction.apply(input, tuple(kernel_size), tuple(s), tuple(d), tuple(p), tuple(u),
+                                tuple(r), "spec2col")
+
+
+def _ext_col2spec(input, spec_size, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1)):
+    """``torch.ops.mellin.col2spec`` (ext/torch.cpp:476): the adjoint of spec2col, no autograd."""
+    return _from_col(input, tuple(spec_size), tuple(s), tuple(d), tuple(p), tuple(u), 2)
 
 
 # ---------------------------------------------------------------------------

@@ -161,6 +161,43 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       double *grad_weight, void *workspace,
                                       size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------------------------------
+ * 3. Column ops: the gather behind the reference's matrix-multiply path and
+ *    its adjoint.
+ *
+ * Same argument meaning and order as the reference's host launchers
+ *   Snd2Col   mconv.h:262-269   / Snd2ColCuda     Col2Snd   mconv.h:301-308   / Col2SndCuda
+ *   Spec2Col  mconv.h:360-368   / Spec2ColCuda    Col2Spec  mconv.h:417-425   / Col2SpecCuda
+ * which ext/torch_cuda.cu:179-291 binds, plus the trailing stream:
+ *   g    signal, (batch, c_in, ngx[, ngy]) or (c_in, batch, ...) if transposed_g
+ *   gg   columns, (batch, c_in, nfx[, nfy], nggx[, nggy]) or (c_in, batch, ...)
+ *        if transposed_gg
+ * x2col WRITES every element of gg:
+ *   gg[n, c, fx, fy, x, y] = g[n, c, (x + sx)(fx + dx)/(px + 1) - ux, (sy y + dy fy - py)/uy]
+ * or 0 where that tap does not exist (Mellin relation on x, linear on y).
+ * col2x WRITES every element of g with the sum of the gg elements whose tap it
+ * is (the adjoint; the gradient of x2col), in a fixed order.
+ * ------------------------------------------------------------------------ */
+#define MELLIN_DECL_SND(NAME, T, SRC, DST)                                      \
+  int NAME(const T *SRC, int64_t c_in, int64_t batch, int64_t nf, int64_t ng,  \
+           int64_t ngg, int64_t s, int64_t d, int64_t p, int64_t u,            \
+           int transposed_g, int transposed_gg, T *DST, void *stream)
+#define MELLIN_DECL_SPEC(NAME, T, SRC, DST)                                     \
+  int NAME(const T *SRC, int64_t c_in, int64_t batch, int64_t nfx, int64_t nfy, \
+           int64_t ngx, int64_t ngy, int64_t nggx, int64_t nggy, int64_t sx,   \
+           int64_t sy, int64_t dx, int64_t dy, int64_t px, int64_t py,         \
+           int64_t ux, int64_t uy, int transposed_g, int transposed_gg,        \
+           T *DST, void *stream)
+
+MELLIN_DECL_SND(mellin_snd2col_f32, float, g, gg);
+MELLIN_DECL_SND(mellin_snd2col_f64, double, g, gg);
+MELLIN_DECL_SND(mellin_col2snd_f32, float, gg, g);
+MELLIN_DECL_SND(mellin_col2snd_f64, double, gg, g);
+MELLIN_DECL_SPEC(mellin_spec2col_f32, float, g, gg);
+MELLIN_DECL_SPEC(mellin_spec2col_f64, double, g, gg);
+MELLIN_DECL_SPEC(mellin_col2spec_f32, float, gg, g);
+MELLIN_DECL_SPEC(mellin_col2spec_f64, double, gg, g);
+
 /* Name of the kernel variant the most recent operator-level call on this
  * thread dispatched to (for tests and profiling): "generic", "mfma" (tiled
  * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"

@@ -89,7 +89,7 @@ def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "mellin_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
     names = set(re.findall(r"\b(mellin_[a-z0-9_]+)\s*\(", text))
-    names |= set(re.findall(r"MELLIN_DECL_[12]D\((mellin_[a-z0-9_]+)\s*,", text))
+    names |= set(re.findall(r"MELLIN_DECL_(?:1D|2D|SND|SPEC)\((mellin_[a-z0-9_]+)\s*,", text))
     return sorted(names)
 
 
