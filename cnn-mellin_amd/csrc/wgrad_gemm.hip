@@ -519,13 +519,16 @@ bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int r
   // the forward plan fixed the position tiling (nt) and the row geometry
   wp.nt = nt;
   wp.rows_mode = 0;
-  if (!pl.segment && pl.ay == 1 && pl.noy >= 16 && pl.nox_eff >= 1 && g_allow_rows) {
-    // Row-wise variant: units of kWaves * rpw output rows.  Preferred shape: two
-    // rows per wavefront and a single buffer (several workgroups per CU cover each
-    // other's loads); then one row per wavefront with two buffers, then with one.
+  if (!pl.segment && pl.ay == 1 && pl.noy >= 4 && pl.nox_eff >= 1 && g_allow_rows) {
+    // Row-wise variant: units of kWaves * rpw output rows, about 300 positions per
+    // unit (two rows of 38 per wavefront, sixteen rows of 5).  Preferred shape: a
+    // single buffer (several workgroups per CU cover each other's loads); then half
+    // the rows with two buffers, then with one.
     const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
     const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
-    const int shapes[3][2] = {{2, 1}, {1, 2}, {1, 1}};   // {rows per wavefront, buffers}
+    const int rpw_auto = std::max(2, std::min(16, (76 + pl.noy - 1) / pl.noy));
+    const int shapes[4][2] = {{rpw_auto, 1}, {std::max(1, rpw_auto / 2), 2}, {std::max(1, rpw_auto / 2), 1},
+                              {1, 1}};   // {rows per wavefront, buffers}
     for (const auto &shape : shapes) {
       const int rpw = rows_opt_rpw > 0 ? rows_opt_rpw : shape[0];
       const int nbuf = rows_opt_nbuf > 0 ? rows_opt_nbuf : shape[1];

@@ -1,0 +1,140 @@
+"""The model-style convolution stack (conv_stack.ConvStack) end to end on the GPU.
+
+* geometry: layer output sizes follow the reference's rule (models.py:292-327:
+  every layer's output is input // factor, whatever the kernel);
+* parity: forward output and every gradient of a reduced stack against the same
+  stack evaluated with the CPU checker in float64 (checker ops wrapped in
+  torch.autograd.Function, ReLU / max-pool by torch on the CPU);
+* the full-size 10-layer stack (3 -> 256 channels, 4x4 kernels, batch 32,
+  780 x 41) runs forward + backward, is finite and run-to-run identical.
+
+Tolerance: the stack compounds ten layers, so outputs and gradients are held to
+rtol 1e-4 of the largest magnitude of the tensor compared (per-layer tolerance
+is checked by the operator tests).
+"""
+import numpy as np
+import pytest
+import torch
+
+import mconv
+from conv_stack import ConvStack, ConvStackParams, layer_plan
+from _gpu import to_gpu, to_np
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+class _CheckerCorr(torch.autograd.Function):
+    """A correlation layer evaluated by the CPU checker (float64 numpy)."""
+
+    @staticmethod
+    def forward(ctx, x, w, b, kind, s, d, p, r):
+        fwd = oracle.mcorrlcorr if kind == "mcorrlcorr" else oracle.lcorrlcorr
+        ctx.save_for_backward(x, w)
+        ctx.args = (kind, s, d, p)
+        return torch.from_numpy(fwd(x.numpy(), w.numpy(), b.numpy(), s, d, p, 1, r))
+
+    @staticmethod
+    def backward(ctx, go):
+        x, w = ctx.saved_tensors
+        kind, s, d, p = ctx.args
+        bwd = oracle.mcorrlcorr_backward if kind == "mcorrlcorr" else oracle.lcorrlcorr_backward
+        gi, gw, gb = bwd(x.numpy(), w.numpy(), np.ascontiguousarray(go.numpy()), s, d, p, 1)
+        return (torch.from_numpy(np.ascontiguousarray(gi)), torch.from_numpy(np.ascontiguousarray(gw)),
+                torch.from_numpy(np.ascontiguousarray(gb)), None, None, None, None, None)
+
+
+def _checker_stack(stack, x64, params64):
+    h = x64
+    for lay, (w, b) in zip(stack.plan, params64):
+        h = torch.relu(_CheckerCorr.apply(h, w, b, lay["kind"], lay["s"], lay["d"], lay["p"], lay["r"]))
+        if lay["pool"]:
+            h = torch.nn.functional.max_pool2d(h, (1, 2))
+    return h
+
+
+def _close(got, exp, what):
+    exp = exp.numpy() if isinstance(exp, torch.Tensor) else exp
+    got = to_np(got).astype(np.float64)
+    scale = max(float(np.abs(exp).max()), 1e-30)
+    np.testing.assert_allclose(got, exp, rtol=0, atol=1e-4 * scale, err_msg=what)
+
+
+@pytest.mark.parametrize("mellin", [True, False], ids=["mellin", "linear"])
+def test_layer_sizes_follow_the_reference_rule(mellin):
+    p = ConvStackParams(layers=6, mellin=mellin, kernel_time=5, kernel_freq=3, initial_channels=4,
+                        factor_schedule=2, channel_factor=2, time_factor=2, freq_factor=2, in_channels=1)
+    x, y = 96, 41
+    plan = layer_plan(p, x, y)
+    for no, lay in enumerate(plan, 1):
+        on = no % 2 == 0
+        if mellin:
+            x, y = (max(x // 2, 1), max(y // 2, 1)) if on else (x, y)
+        else:
+            px, py = lay["p"]
+            x = (x + 2 * px - 5) // lay["s"][0] + 1
+            y = (y + 2 * py - 3) // lay["s"][1] + 1
+        assert lay["out_size"] == (x, y), (no, lay)
+        assert lay["out_channels"] == 4 * 2 ** (no // 2)
+    stack = ConvStack(96, 41, p).cuda()
+    out = stack(torch.randn(2, 1, 96, 41, device="cuda"))
+    assert tuple(out.shape) == (2, stack.out_channels) + stack.out_size
+
+
+@pytest.mark.parametrize("mellin", [True, False], ids=["mellin", "linear"])
+def test_reduced_stack_matches_checker(mellin):
+    p = ConvStackParams(layers=5, mellin=mellin, kernel_time=4, kernel_freq=4, initial_channels=6,
+                        factor_schedule=3, channel_factor=2, time_factor=2 if not mellin else 1,
+                        freq_factor=1, in_channels=3, freq_pool_after=(3,), seed=4)
+    stack = ConvStack(40, 21, p).cuda()
+    gen = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 3, 40, 21, generator=gen)
+    xg = x.cuda().requires_grad_(True)
+    out = stack(xg)
+    go = torch.randn(out.shape, generator=gen)
+    out.backward(go.cuda())
+
+    x64 = x.double().requires_grad_(True)
+    params64 = [(c.weight.detach().cpu().double().requires_grad_(True),
+                 c.bias.detach().cpu().double().requires_grad_(True)) for c in stack.convs]
+    exp = _checker_stack(stack, x64, params64)
+    assert tuple(out.shape) == tuple(exp.shape)
+    exp.backward(go.double())
+    _close(out, exp.detach(), "stack output")
+    _close(xg.grad, x64.grad, "grad_input")
+    for no, (conv, (w, b)) in enumerate(zip(stack.convs, params64), 1):
+        _close(conv.weight.grad, w.grad, "grad_weight layer %d" % no)
+        _close(conv.bias.grad, b.grad, "grad_bias layer %d" % no)
+
+
+def test_full_size_stack_runs_and_is_deterministic():
+    """BASELINE config 5: ten layers, 3 -> 256 channels, 4 x 4 kernels, ReLU, frequency
+    max-pool 2 after layers 3, 6 and 9, batch 32, up to 780 frames x 41 bins, seed 4."""
+    p = ConvStackParams(layers=10, mellin=True, kernel_time=4, kernel_freq=4, initial_channels=32,
+                        factor_schedule=3, channel_factor=2, time_factor=1, freq_factor=1, in_channels=3,
+                        freq_pool_after=(3, 6, 9), seed=4)
+    stack = ConvStack(780, 41, p).cuda()
+    assert [lay["out_channels"] for lay in stack.plan] == [32, 32, 64, 64, 64, 128, 128, 128, 256, 256]
+    assert stack.out_size == (780, 5)
+    gen = torch.Generator().manual_seed(4)
+    lens = torch.randint(100, 781, (32,), generator=gen)
+    x = torch.randn(32, 3, 780, 41, generator=gen)
+    x = x * (torch.arange(780)[None, :] < lens[:, None])[:, None, :, None]     # zero past each length
+    results = []
+    for _ in range(2):
+        for q in stack.parameters():
+            q.grad = None
+        xg = x.cuda().requires_grad_(True)
+        out = stack(xg)
+        assert tuple(out.shape) == (32, 256, 780, 5)
+        loss = out.square().mean()
+        loss.backward()
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(xg.grad).all())
+        results.append((out.detach().clone(), xg.grad.clone(),
+                        [q.grad.clone() for q in stack.parameters()]))
+    assert torch.equal(results[0][0], results[1][0])
+    assert torch.equal(results[0][1], results[1][1])
+    for a, b in zip(results[0][2], results[1][2]):
+        assert bool(torch.isfinite(a).all())
+        assert torch.equal(a, b)
