@@ -498,8 +498,19 @@ hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const flo
 
 // Plan the weight gradient of the layer whose FORWARD problem is `fwd`
 // (filter = weight, signal = input, output = grad_out, write mode).
+static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt,
+                               int rows_opt_nbuf, int rows_opt_rpw, int jt_max);
+
 bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf,
                      int rows_opt_rpw) {
+  // narrower column blocks touch fewer input channels and so need less LDS
+  for (int jt_max = 3; jt_max >= 1; --jt_max)
+    if (make_wgrad_plan_jt(fwd, wp, g_allow_rows, rows_opt_mt, rows_opt_nbuf, rows_opt_rpw, jt_max)) return true;
+  return false;
+}
+
+static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt,
+                               int rows_opt_nbuf, int rows_opt_rpw, int jt_max) {
   size_t lds_fwd;
   int mt, nt;
   // 128 positions per tile: the staged grad_out tile (channels x positions, two
@@ -508,7 +519,7 @@ bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int r
   TilePlan &pl = wp.t;
   wp.J = pl.C * pl.nf;
   wp.mt = 1;
-  wp.jt = wp.J > 64 ? 3 : (wp.J > 32 ? 2 : 1);
+  wp.jt = std::min(jt_max, wp.J > 64 ? 3 : (wp.J > 32 ? 2 : 1));
   const int M_T = wp.mt * 32, J_T = wp.jt * 32;
   wp.m_groups = (pl.M + M_T - 1) / M_T;
   wp.j_groups = (wp.J + J_T - 1) / J_T;
