@@ -577,8 +577,9 @@ bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64
   const i64 lim = (i64)1 << 28;
   if (nh >= lim || c_out * c_in * nf >= lim || batch * c_in >= lim) return false;
   const i64 mtn = (nf + 31) / 32, units = c_in * mtn;
-  // few input channels, and taps that fill their 32-row tiles reasonably
-  if (c_in >= 16 || units > 8 || mtn * 32 * 2 > nf * 3 || c_out > 128) return false;
+  // few input channels, and taps that fill at least a quarter of their 32-row tiles
+  // (even a half-empty tile beats the gather form, whose tiles hold c_in rows)
+  if (c_in >= 16 || units > 8 || mtn * 32 > nf * 4 || c_out > 128) return false;
   pl.batch = (int)batch; pl.c_in = (int)c_in; pl.c_out = (int)c_out;
   pl.nf = (int)nf; pl.nh = (int)nh;
   pl.mtn = (int)mtn; pl.units = (int)units; pl.nf_pad = (int)mtn * 32;
@@ -617,10 +618,11 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
   const i64 lim = (i64)1 << 28;
   if (nh >= lim || ng >= lim || c_out * c_in * nf >= lim) return false;
   if (sx >= 4096 || sy >= 4096 || dx >= 4096 || dy >= 4096 || px >= lim || py >= lim) return false;
-  // few input channels, and taps that fill their 32-row tiles reasonably
+  // few input channels, and taps that fill at least a quarter of their 32-row tiles
+  // (even a half-empty tile beats the gather form, whose tiles hold c_in rows)
   const i64 mtn = (nf + 31) / 32;
   const i64 units = c_in * mtn;
-  if (c_in >= 16 || units > 8 || mtn * 32 * 2 > nf * 3) return false;
+  if (c_in >= 16 || units > 8 || mtn * 32 > nf * 4) return false;
   if (c_out > 128) return false;
   pl.batch = (int)batch; pl.c_in = (int)c_in; pl.c_out = (int)c_out;
   pl.nfx = (int)nfx; pl.nfy = (int)nfy; pl.nf = (int)nf;
