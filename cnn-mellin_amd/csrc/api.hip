@@ -15,7 +15,7 @@ namespace {
 
 thread_local char g_error[512] = "";
 thread_local const char *g_variant = "";
-thread_local int g_forced = 0;   // 0 automatic, 1 generic, 2 automatic without the fused input gradient
+thread_local int g_forced = 0;   // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
                                  // and without the row-wise weight gradient
 
 int fail(int code, const char *fmt, ...) {

@@ -32,6 +32,7 @@
 // MT * NT accumulator tiles (16 registers each).  Stores write 128-byte runs
 // of one output row.
 #include <algorithm>
+#include <type_traits>
 
 #include "mellin_common.hpp"
 #include "tile_gemm.hpp"
@@ -47,17 +48,27 @@ namespace {
 #endif
 
 template <int MT, int NT, bool ACC>
-__global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
-    TilePlan pl, const float *__restrict__ F, const float *__restrict__ G,
+__global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
+    TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H) {
+  // The plan is read where it lies, in the kernel-argument segment (it is the
+  // first argument), through a pointer the compiler must treat as new in every
+  // iteration of the stage loop: fields are then re-read by scalar loads where
+  // they are used instead of all being held in scalar registers for the whole
+  // kernel, which had the register allocator spill hundreds of them to vector
+  // lanes around the stores and the staging code.
+  typedef const __attribute__((address_space(4))) TilePlan ConstPlan;
+  ConstPlan *const plan_base = (ConstPlan *)__builtin_amdgcn_kernarg_segment_ptr();
+  ConstPlan *plp = plan_base;
+#define pl (*plp)
   extern __shared__ float lds[];
   constexpr int M_T = MT * 32;
   constexpr int P = kWaves * NT * 32;
-  constexpr int GS = 4;                              // tap pairs per operand group
   const int g_words = pl.CC * pl.R * pl.RS;          // one signal buffer
   const int w_words = M_T * pl.WSS;                  // one filter buffer
-  float *Gs0 = lds;                                  // [2][CC][R][RS]
-  float *Ws0 = Gs0 + 2 * g_words;                    // [1 or 2][M_T][WSS]
+  float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
+  const int ws_word0 = pl.sbuf * g_words;
+  float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS]
   const bool single_chunk = pl.CC >= pl.C;
   int *tapoff = (int *)(Ws0 + (single_chunk ? 1 : 2) * w_words);   // [KCp]
   float *Bs = (float *)(tapoff + pl.KCp);            // [M_T] bias (zeros when accumulating)
@@ -73,13 +84,30 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   const int chunks = (pl.C + pl.CC - 1) / pl.CC;
 
   // ---- filter block: Ws[m][k], k = cl * nf + t, row stride WSS (odd) --------------
-  // one direct load per (m, 64 taps): lane k fetches F[m0 + m, c0 + cl, t], coalesced
-  // along the taps; taps past the chunk and channels past M are zero
+  // direct loads, coalesced along the taps; taps past the chunk and channels past M
+  // are zero
   const unsigned lds_base = lds_address(lds);
   auto issue_filter = [&](int c0, int cc, int ws_word) {        // ws_word: where the block starts in lds[]
     const int KC = cc * pl.nf;
-    const FastDiv by_nf(pl.nf);
     const int m_live = max(0, min(M_T, pl.M - m0));       // channels of this block that exist
+    const int KC4 = KC & ~3;
+    if (pl.f_c == pl.nf && ((KC4 + 255) >> 8) + (KC4 < KC) < ((pl.KCp + 63) >> 6)) {
+      // the taps of consecutive channels are one run of KC words per output channel:
+      // 16 bytes per lane, then the last KC % 4 words singly (taken when that is
+      // fewer instructions than 64 single words at a time)
+      for (int m = wave; m < m_live; m += kWaves) {
+        const float *row = F + (i64)(m0 + m) * pl.f_m + (i64)c0 * pl.f_c;
+        const unsigned dst = lds_base + 4u * (unsigned)(ws_word + m * pl.WSS);
+        for (int kb = 0; kb < KC4; kb += 256)
+          if (kb + 4 * lane < KC4) load16_to_lds_at(row, (unsigned)(kb + 4 * lane) * 4u, dst + 4u * (unsigned)kb);
+        if (lane < KC - KC4) load_to_lds_at(row, (unsigned)(KC4 + lane) * 4u, dst + 4u * (unsigned)KC4);
+        if (lane < pl.KCp - KC) lds[ws_word + m * pl.WSS + KC + lane] = 0.f;     // KCp - KC <= 1
+      }
+      for (int m = m_live + wave; m < M_T; m += kWaves)
+        for (int k = lane; k < pl.KCp; k += 64) lds[ws_word + m * pl.WSS + k] = 0.f;
+      return;
+    }
+    const FastDiv by_nf(pl.nf);
     for (int kb = 0; kb < pl.KCp; kb += 64) {
       const int k = kb + lane;
       int cl, t;
@@ -100,13 +128,12 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   const int my_tiles = (int)blockIdx.x < pl.total_tiles
                            ? (pl.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
   const int my_stages = my_tiles * chunks;
-  auto issue_stage = [&](int st) {
-    const int ti = st / chunks, ch = st - ti * chunks;
+  auto issue_stage = [&](int st, int ti, int ch) {           // st = ti * chunks + ch
     const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
     const int c0 = ch * pl.CC, cc = min(pl.CC, pl.C - c0);
-    issue_signal(pl, tg, G, c0, cc, Gs0 + (st & 1) * g_words, lds_base + 4u * (unsigned)((st & 1) * g_words),
-                 mellin_x, lane, wave);
-    if (!single_chunk) issue_filter(c0, cc, 2 * g_words + (st & 1) * w_words);
+    const int sb = (st & 1) * (pl.sbuf - 1) * g_words;    // sbuf == 1: a workgroup has one stage only
+    issue_signal(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave);
+    if (!single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words);
   };
 
   {
@@ -122,8 +149,8 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   }
   MELLIN_STAMP(0);
   if (my_stages > 0) {
-    if (single_chunk) issue_filter(0, pl.C, 2 * g_words);
-    issue_stage(0);
+    if (single_chunk) issue_filter(0, pl.C, ws_word0);
+    issue_stage(0, 0, 0);
   }
   MELLIN_STAMP(1);
 
@@ -132,13 +159,17 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
   int lane_base[NT], lane_q[NT];
   TileGeom tg;
 
-  // ---- epilogue: 32 consecutive lanes write 32 consecutive positions of one
-  // channel.  It runs one stage late (after the next stage's loads are issued,
-  // before its multiplies) so that the stores drain behind the next matrix
-  // loop instead of holding up the wait for those loads.
-  auto epilogue = [&]() {
-    float *Hq = H + (i64)tg.n * pl.h_n + (i64)(m0 + half * 4) * pl.h_m;
-    const int m_left = pl.M - m0 - half * 4;              // channels from this lane's first row on
+  // ---- stores: 32 consecutive lanes write 32 consecutive positions of one
+  // channel; each lane walks one pointer down the channels in steps of whole
+  // channel strides, so the only scalars the stores need are four byte strides.
+  const i64 hm1 = pl.h_m * 4, hm2 = 2 * hm1, hm3 = 3 * hm1, hm8 = 8 * hm1;
+  const bool full_m = m0 + M_T <= pl.M;
+  const int m_left = pl.M - m0 - half * 4;              // channels from this lane's first row on
+  // They run one stage late, after the next stage's loads are issued and before
+  // its multiplies, so that they drain behind the next matrix loop.
+  auto write_tile = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    char *Himg = (char *)(H + (i64)tg.n * pl.h_n + (i64)m0 * pl.h_m);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int local = (wave * NT + t) * 32 + l32;
@@ -149,30 +180,48 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
         live = live && ox < pl.nox_eff && oy < pl.noy_eff;
       }
       if (!live) continue;
-      float *Ht = Hq + lane_q[t];
+      char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * 4;
 #pragma unroll
       for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int mo = i * 32 + (r >> 2) * 8 + (r & 3);
-          if (mo < m_left) {
-            float *dst = Ht + (i64)mo * pl.h_m;
-            if (ACC) *dst += acc[i][t][r];
-            else *dst = acc[i][t][r];
-          }
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int mo = i * 32 + g4 * 8;
+          auto put = [&](char *at, int row, float v) {
+            if (FULL || row < m_left) {
+              float *dst = (float *)at;
+              if (ACC) *dst += v;
+              else *dst = v;
+            }
+          };
+          put(o, mo, acc[i][t][4 * g4]);
+          put(o + hm1, mo + 1, acc[i][t][4 * g4 + 1]);
+          put(o + hm2, mo + 2, acc[i][t][4 * g4 + 2]);
+          put(o + hm3, mo + 3, acc[i][t][4 * g4 + 3]);
+          o += hm8;                                        // next group of four channels: 8 further on
         }
     }
   };
-
-  for (int st = 0; st < my_stages; ++st) {
-    const int ti = st / chunks, ch = st - ti * chunks;
+  auto epilogue = [&]() {
+    if (full_m) write_tile(std::true_type());
+    else write_tile(std::false_type());
+  };
+  for (int st = 0, ti = 0, ch = 0; st < my_stages; ++st, ti += (ch + 1 == chunks), ch = (ch + 1 == chunks) ? 0 : ch + 1) {
+    {
+      unsigned zero;                                      // a zero the compiler cannot see through
+      asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
+      plp = (ConstPlan *)((const __attribute__((address_space(4))) char *)plan_base + zero);
+    }
     // every wave's loads for this stage have landed, and every wave is done
     // reading the buffer the next stage will fill
     wait_all_memory();
     MELLIN_STAMP(2);
     __syncthreads();
     MELLIN_STAMP(3);
-    if (st + 1 < my_stages) { MELLIN_STAMP(7); issue_stage(st + 1); MELLIN_STAMP(8); }
+    if (st + 1 < my_stages) {
+      MELLIN_STAMP(7);
+      issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
+      MELLIN_STAMP(8);
+    }
     MELLIN_STAMP(4);
 
     if (ch == 0) {
@@ -190,6 +239,8 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
         lane_q[t] = q;
         lane_base[t] = (pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min;
       }
+    }
+    if (ch == 0) {
       // accumulators start from the bias of the channel each register holds
 #pragma unroll
       for (int a = 0; a < MT; ++a)
@@ -203,68 +254,17 @@ __global__ __launch_bounds__(kThreads, 2) void tile_gemm_kernel(
           }
         }
     }
-
-    // ---- matrix-core loop over tap pairs: operands of the next group of GS
-    // pairs are fetched from LDS while the current group multiplies
+    // ---- matrix-core loop over the tap pairs of this chunk
     {
       const int cc = min(pl.CC, pl.C - ch * pl.CC);
-      const int KC = cc * pl.nf;
-      const int steps = (KC + 1) >> 1;
-      const float *Gs = Gs0 + (st & 1) * g_words;
-      const float *wa = Ws0 + (single_chunk ? 0 : (st & 1) * w_words) + l32 * pl.WSS + half;
-      const int *tp = tapoff + half;
-      const int wrow = 32 * pl.WSS;                        // next 32 channels
-      const int full = (KC & 1) ? steps - 1 : steps;       // steps whose two taps both exist
-      const int groups = full / GS;
-      float a0[GS][MT], b0[GS][NT], a1[GS][MT], b1[GS][NT];
-      auto fetch = [&](int g, float (&a)[GS][MT], float (&b)[GS][NT]) {
-        int off[GS];
-#pragma unroll
-        for (int j = 0; j < GS; ++j) off[j] = tp[2 * (g * GS + j)];
-#pragma unroll
-        for (int j = 0; j < GS; ++j) {
-#pragma unroll
-          for (int i = 0; i < MT; ++i) a[j][i] = wa[2 * (g * GS + j) + i * wrow];
-#pragma unroll
-          for (int t = 0; t < NT; ++t) b[j][t] = Gs[lane_base[t] + off[j]];
-        }
-      };
-      auto multiply = [&](float (&a)[GS][MT], float (&b)[GS][NT]) {
-#pragma unroll
-        for (int j = 0; j < GS; ++j)
-#pragma unroll
-          for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][i], b[j][t], acc[i][t], 0, 0, 0);
-      };
-      int g = 0;
-      if (groups > 0) fetch(0, a0, b0);
-      for (; g + 1 < groups; g += 2) {
-        fetch(g + 1, a1, b1);
-        multiply(a0, b0);
-        if (g + 2 < groups) fetch(g + 2, a0, b0);
-        multiply(a1, b1);
-      }
-      if (g < groups) multiply(a0, b0);
-      for (int s = groups * GS; s < steps; ++s) {
-        const int off = tp[2 * s];
-        float a[MT], b[NT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i) a[i] = wa[2 * s + i * wrow];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) b[t] = (s >= full && half) ? 0.f : Gs[lane_base[t] + off];
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
-      }
+      multiply_taps<MT, NT>(acc, Ws0 + (single_chunk ? 0 : (st & 1) * w_words) + l32 * pl.WSS + half, 32 * pl.WSS,
+                            tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
     MELLIN_STAMP(6);
   }
   if (my_stages > 0) epilogue();
   MELLIN_STAMP(9);
+#undef pl
 }
 
 template <int MT, int NT, bool ACC>
@@ -286,6 +286,14 @@ hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const
 }
 
 }  // namespace
+
+// Workgroups of the forward kernel that a CU holds at once: bounded by LDS and
+// by the registers of the instance (NT == 2 needs more than 128).
+static int workgroups_per_cu(size_t lds_bytes, int mt, int nt) {
+  const int by_lds = (int)((160 * 1024) / (lds_bytes + 512));
+  (void)mt;
+  return std::max(1, std::min(by_lds, nt == 2 ? 3 : 4));
+}
 
 // Fill `pl` for the problem `pr`; returns false when the tiled kernel does not
 // apply (sizes beyond 32-bit indexing or a single channel not fitting in LDS).
@@ -330,6 +338,8 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.chunks_per_row = (pl.noy + P - 1) / P;
   pl.tiles_per_image = pl.segment ? pl.nox * pl.chunks_per_row : (pl.Q + P - 1) / P;
   pl.total_tiles = pl.batch * pl.tiles_per_image;
+  auto magic = [](int d) { return d <= 1 ? 0xFFFFFFFFu : (unsigned)(0x100000000ull / (unsigned)d); };
+  pl.mg_tpi = magic(pl.tiles_per_image); pl.mg_cpr = magic(pl.chunks_per_row); pl.mg_noy = magic(pl.noy);
   const int RT = pl.segment ? 1 : std::min(pl.nox, (P - 1 + pl.noy - 1) / pl.noy + 1);
   const int oy_span = pl.segment ? P : pl.noy;
   const i64 RSL = (i64)pl.ay * (oy_span - 1) + pl.by_span + 1;
@@ -390,19 +400,32 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   const bool single = pl.CC >= pl.C;
   *lds_bytes = 4 * (2 * (size_t)pl.CC * pl.R * pl.RS + (single ? 1 : 2) * (size_t)M_T * pl.WSS +
                     pl.KCp + M_T);
-  return *lds_bytes <= 76 * 1024;
+  if (*lds_bytes > 76 * 1024) return false;
+  // A launch small enough that every tile gets a workgroup of its own once the
+  // second signal buffer is dropped (more workgroups fit per CU) runs as one
+  // wave of single-stage workgroups: nothing to prefetch, and no second round
+  // in which most of the chip idles.
+  pl.sbuf = 2;
+  if (single) {
+    const size_t one = *lds_bytes - 4 * (size_t)pl.CC * pl.R * pl.RS;
+    const i64 slots2 = 256 * (i64)workgroups_per_cu(*lds_bytes, *mt, *nt);
+    const i64 slots1 = 256 * (i64)workgroups_per_cu(one, *mt, *nt);
+    const i64 wgs = (i64)pl.total_tiles * m_tiles;
+    if (wgs > slots2 && wgs <= slots1) { pl.sbuf = 1; *lds_bytes = one; }
+  }
+  return true;
 }
 
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
                             float *h, hipStream_t stream) {
   const int M_T = mt * 32;
-  // persistent workgroups: as many as fit at once (by LDS, two per CU at most) on the 256 CUs
+  // persistent workgroups: as many as fit at once on the 256 CUs
   const int m_tiles = (pl.M + M_T - 1) / M_T;
-  int per_cu = (int)((160 * 1024) / (lds_bytes + 512));
-  per_cu = std::max(1, std::min(per_cu, nt == 2 ? 3 : 4));
+  const int per_cu = workgroups_per_cu(lds_bytes, mt, nt);
   int gx = std::max(1, (256 * per_cu) / m_tiles);
   gx = std::min(gx, pl.total_tiles);
+  if (pl.sbuf == 1 && gx < pl.total_tiles) return hipErrorInvalidValue;   // one buffer: one stage per workgroup
   dim3 grid((unsigned)gx, (unsigned)m_tiles);
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_)                                                                \

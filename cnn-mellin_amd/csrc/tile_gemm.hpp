@@ -23,7 +23,9 @@ struct TilePlan {
   int ay, by, cy, uy, by_min, by_span;
   // tiling
   int segment, chunks_per_row, tiles_per_image, total_tiles;
+  unsigned mg_tpi, mg_cpr, mg_noy;  // floor(2^32 / d) for tiles_per_image, chunks_per_row, noy (see udiv)
   int R, RS;                       // virtual rows per channel and their stride (words)
+  int sbuf;                        // signal buffers in LDS: 2, or 1 when no workgroup has a second stage
   int contig;                      // virtual rows coincide with the signal's rows (same pitch): block copies
   int CP, CP_log2;                 // staged columns rounded up to a power of two
   int CC;                          // channels staged per chunk

@@ -22,7 +22,7 @@ __device__ __forceinline__ unsigned lds_address(const float *p) {
 
 // Sixteen bytes per active lane: lane l reads the four dwords at `base` +
 // `byte_offset` (any 4-byte alignment) and they land at LDS byte address
-// `lds_addr` + 16 * l (`lds_addr` wave-uniform and 16-byte aligned).
+// `lds_addr` + 16 * l (`lds_addr` wave-uniform; 4-byte alignment is enough).
 __device__ __forceinline__ void load16_to_lds_at(const float *base, unsigned byte_offset, unsigned lds_addr) {
   const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   const unsigned long long b = (unsigned long long)base;
@@ -80,19 +80,30 @@ struct FastDiv {
   }
 };
 
+// x / d for 0 <= x < 2^31 and d >= 1 with m = floor(2^32 / d) (0xFFFFFFFF for d = 1):
+// the product's high word is the quotient or one less.  On wave-uniform values this
+// is a handful of scalar instructions; a plain integer division goes through the
+// vector unit's reciprocal, and vector instructions queue behind the matrix ones.
+__device__ __forceinline__ int udiv(int x, int d, unsigned m) {
+  unsigned q = __umulhi((unsigned)x, m);
+  if ((unsigned)x - q * (unsigned)d >= (unsigned)d) ++q;
+  return (int)q;
+}
+
 // Uniform description of one position tile.
 struct TileGeom {
   int n, q0, count, ox_lo, oy_lo, R_tile, RSL, vx_min, vy_min;
 };
 
-template <int P>
-__device__ __forceinline__ TileGeom tile_geometry(const TilePlan &pl, int tile_id, bool mellin_x) {
+// (PL: TilePlan in whatever address space the caller holds it)
+template <int P, class PL>
+__device__ __forceinline__ TileGeom tile_geometry(const PL &pl, int tile_id, bool mellin_x) {
   TileGeom g;
-  g.n = tile_id / pl.tiles_per_image;
+  g.n = udiv(tile_id, pl.tiles_per_image, pl.mg_tpi);
   const int tile = tile_id - g.n * pl.tiles_per_image;
   int ox_hi, oy_hi;
   if (pl.segment) {
-    g.ox_lo = ox_hi = tile / pl.chunks_per_row;
+    g.ox_lo = ox_hi = udiv(tile, pl.chunks_per_row, pl.mg_cpr);
     g.oy_lo = (tile - g.ox_lo * pl.chunks_per_row) * P;
     g.count = min(P, pl.noy - g.oy_lo);
     oy_hi = g.oy_lo + g.count - 1;
@@ -100,8 +111,8 @@ __device__ __forceinline__ TileGeom tile_geometry(const TilePlan &pl, int tile_i
   } else {
     g.q0 = tile * P;
     g.count = min(P, pl.Q - g.q0);
-    g.ox_lo = g.q0 / pl.noy;
-    ox_hi = (g.q0 + g.count - 1) / pl.noy;
+    g.ox_lo = udiv(g.q0, pl.noy, pl.mg_noy);
+    ox_hi = udiv(g.q0 + g.count - 1, pl.noy, pl.mg_noy);
     g.oy_lo = 0;
     oy_hi = pl.noy - 1;
   }
@@ -115,10 +126,11 @@ __device__ __forceinline__ TileGeom tile_geometry(const TilePlan &pl, int tile_i
 
 
 // ---- signal rows of one (tile, channel range) --------------------------------
-// wave w owns virtual rows w, w + 4, ...; 64 lanes first work out the source of
-// 64 such rows, then one direct load per row is issued with the lanes on
-// columns; columns or rows without a source are written as zeros.
-__device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom &tg,
+// wave w of the NW that stage together owns virtual rows w, w + NW, ...; 64 lanes
+// first work out the source of 64 such rows, then direct loads are issued per row
+// with the lanes on columns; columns or rows without a source are written as zeros.
+template <int NW = kWaves, class PL>
+__device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
                                              const float *__restrict__ G, int c0, int cc,
                                              float *Gs, unsigned gs_addr, bool mellin_x, int lane,
                                              int wave) {
@@ -132,14 +144,15 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
     const int count = tg.R_tile * pl.ngy, count4 = count & ~3;
     const int pieces = (count4 + 255) >> 8;
     const float *src0 = Gimg + tg.vx_min * pl.ngy;
-    for (int i = wave; i < cc * pieces; i += kWaves) {
-      const int cl = i / pieces, w0 = (i - cl * pieces) << 8;
-      const int idx = w0 + 4 * lane;
+    for (int cl = 0, pc = wave; ; pc += NW) {              // piece pc of channel cl; pieces go round the waves
+      while (pc >= pieces) { pc -= pieces; ++cl; }
+      if (cl >= cc) break;
+      const int w0 = pc << 8, idx = w0 + 4 * lane;
       if (idx < count4)
         load16_to_lds_at(src0 + (i64)cl * g_c, (unsigned)idx * 4u, gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + w0));
     }
     if (count4 < count)
-      for (int cl = wave; cl < cc; cl += kWaves)
+      for (int cl = wave; cl < cc; cl += NW)
         if (lane < count - count4)
           load_to_lds_at(src0 + (i64)cl * g_c, (unsigned)(count4 + lane) * 4u,
                          gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + count4));
@@ -158,7 +171,7 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
     }
     const int words = cc * pl.R;
     const FastDiv by_R(pl.R), by_nfx1(pl.nfx);
-    for (int w0 = wave * 64; w0 < words; w0 += 64 * kWaves) {
+    for (int w0 = wave * 64; w0 < words; w0 += 64 * NW) {
       const int wd = w0 + lane;
       int src = -1;
       if (wd < words && gy >= 0) {
@@ -186,9 +199,9 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
     return;
   }
   const FastDiv by_rows(tg.R_tile), by_nfx(pl.nfx);
-  for (int base = 0; base < total_rows; base += 64 * kWaves) {
+  for (int base = 0; base < total_rows; base += 64 * NW) {
     // per-lane: row base + 4 * lane + wave
-    const int rr = base + kWaves * lane + wave;
+    const int rr = base + NW * lane + wave;
     int src_off = -1, dst_off = 0;
     if (rr < total_rows) {
       int cl, r;
@@ -208,7 +221,7 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
       if (gx >= 0) src_off = cl * g_c + gx * pl.ngy;
       dst_off = (cl * pl.R + r) * pl.RS;
     }
-    const int mine = min(64, (total_rows - base - wave + kWaves - 1) / kWaves);
+    const int mine = min(64, (total_rows - base - wave + NW - 1) / NW);
     for (int cb = 0; cb < tg.RSL; cb += 64) {
       const int col = cb + lane;
       const int vy = tg.vy_min + col;
@@ -239,6 +252,66 @@ __device__ __forceinline__ void issue_signal(const TilePlan &pl, const TileGeom 
         }
       }
     }
+  }
+}
+
+// ---- matrix-core loop over the tap pairs of one staged chunk ---------------------
+// acc[i][t] += sum_k A[i * 32 + row][k] * B[k][t * 32 + col] on v_mfma_f32_32x32x2_f32:
+// lane (l32, half) supplies A[l32][2 s + half] = wa[2 s + i * wrow] and
+// B[2 s + half][l32] = Gs[lane_base[t] + tp[2 s]] for tap pair s.  Operands of the
+// next group of GS pairs are fetched from LDS while the current group multiplies.
+// KC taps (a last odd tap is paired with a zero).
+template <int MT, int NT>
+__device__ __forceinline__ void multiply_taps(floatx16 (&acc)[MT][NT], const float *wa, int wrow,
+                                              const int *tp, const float *Gs, const int (&lane_base)[NT],
+                                              int KC, int half) {
+  constexpr int GS = 4;                              // tap pairs per operand group
+  const int steps = (KC + 1) >> 1;
+  const int full = (KC & 1) ? steps - 1 : steps;       // steps whose two taps both exist
+  const int groups = full / GS;
+  float a0[GS][MT], b0[GS][NT], a1[GS][MT], b1[GS][NT];
+  auto fetch = [&](int g, float (&a)[GS][MT], float (&b)[GS][NT]) {
+    int off[GS];
+#pragma unroll
+    for (int j = 0; j < GS; ++j) off[j] = tp[2 * (g * GS + j)];
+#pragma unroll
+    for (int j = 0; j < GS; ++j) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) a[j][i] = wa[2 * (g * GS + j) + i * wrow];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) b[j][t] = Gs[lane_base[t] + off[j]];
+    }
+  };
+  auto multiply = [&](float (&a)[GS][MT], float (&b)[GS][NT]) {
+#pragma unroll
+    for (int j = 0; j < GS; ++j)
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][i], b[j][t], acc[i][t], 0, 0, 0);
+  };
+  int g = 0;
+  if (groups > 0) fetch(0, a0, b0);
+  for (; g + 1 < groups; g += 2) {
+    fetch(g + 1, a1, b1);
+    multiply(a0, b0);
+    if (g + 2 < groups) fetch(g + 2, a0, b0);
+    multiply(a1, b1);
+  }
+  if (g < groups) multiply(a0, b0);
+  for (int s = groups * GS; s < steps; ++s) {
+    const int off = tp[2 * s];
+    float a[MT], b[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a[i] = wa[2 * s + i * wrow];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) b[t] = (s >= full && half) ? 0.f : Gs[lane_base[t] + off];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
   }
 }
 
