@@ -42,7 +42,10 @@ SYMBOLS = {
     "mellin_set_variant": (_int, [ctypes.c_char_p]),
     "mellin_corr2d_backward_weight_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
+    "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
 }
+_dbl = ctypes.c_double
+PW_LOG, PW_LIFT = 1, 2
 for _t in ("f32", "f64"):
     for _n in ("mcorr1d", "mconv1d"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _ACC1D)
@@ -52,6 +55,9 @@ for _t in ("f32", "f64"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _SND)
     for _n in ("spec2col", "col2spec"):
         SYMBOLS["mellin_%s_%s" % (_n, _t)] = (_int, _SPEC)
+    SYMBOLS["mellin_log_lift_forward_" + _t] = (_int, [_ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr])
+    SYMBOLS["mellin_log_lift_backward_" + _t] = (
+        _int, [_ptr, _ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
     SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_backward_input_" + _t] = (
         _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
@@ -143,6 +149,27 @@ def col_op(name, src, dst, c_in, batch, nf, ng, ngg, s, d, p, u, tg, tgg):
                       d[0], d[1], p[0], p[1], u[0], u[1], int(tg), int(tgg), _dp(dst), _stream(dev))
     _check(code)
     return dst
+
+
+def log_lift_forward(x, eps, tau, flags, outer, t, inner, y):
+    """y = the selected pointwise function of x, both dense and viewed as (outer, t, inner)."""
+    dev = require_device(x, y)
+    fn = getattr(lib, "mellin_log_lift_forward_" + suffix(y.dtype))
+    with torch.cuda.device(dev):
+        _check(fn(_dp(x), float(eps), float(tau), flags, outer, t, inner, _dp(y), _stream(dev)))
+    return y
+
+
+def log_lift_backward(x, grad_y, eps, tau, flags, outer, t, inner, grad_x, grad_params):
+    """grad_x and grad_params = (d/d eps, d/d tau); allocates the scratch the library asks for."""
+    dev = require_device(x, grad_y, grad_x, grad_params)
+    fn = getattr(lib, "mellin_log_lift_backward_" + suffix(grad_x.dtype))
+    need = lib.mellin_log_lift_backward_workspace(grad_x.element_size(), outer, t, inner)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(fn(_dp(x), _dp(grad_y), float(eps), float(tau), flags, outer, t, inner, _dp(grad_x),
+                  _ptr(grad_params.data_ptr()), _ptr(ws.data_ptr()), need, _stream(dev)))
+    return grad_x, grad_params
 
 
 def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):

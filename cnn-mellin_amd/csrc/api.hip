@@ -377,6 +377,51 @@ DEFINE_SPEC(mellin_spec2col_f64, double, g, gg, true)
 DEFINE_SPEC(mellin_col2spec_f32, float, gg, g, false)
 DEFINE_SPEC(mellin_col2spec_f64, double, gg, g, false)
 
+// ---- section 4: pointwise layers ----------------------------------------------
+int check_log_lift(const char *fn, double eps, int flags, i64 outer, i64 t, i64 inner) {
+  if (!(flags & (MELLIN_PW_LOG | MELLIN_PW_LIFT)) || (flags & ~(MELLIN_PW_LOG | MELLIN_PW_LIFT)))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: flags must be MELLIN_PW_LOG, MELLIN_PW_LIFT or both (got %d)", fn, flags);
+  if (outer < 0 || t < 0 || inner < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: negative size (outer=%lld t=%lld inner=%lld)", fn, (long long)outer,
+                (long long)t, (long long)inner);
+  if ((flags & MELLIN_PW_LOG) && !(eps > 0))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: eps must be positive (got %g)", fn, eps);
+  if (t * inner >= ((i64)1 << 40) || outer >= ((i64)1 << 40))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: sizes beyond the supported range", fn);
+  return MELLIN_OK;
+}
+
+template <typename T>
+int log_lift_forward(const char *fn, const T *x, double eps, double tau, int flags, i64 outer, i64 t, i64 inner,
+                     T *y, void *stream) {
+  int rc;
+  if ((rc = check_log_lift(fn, eps, flags, outer, t, inner))) return rc;
+  if (outer * t * inner == 0) return MELLIN_OK;
+  if (!x || !y) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e = launch_log_lift_forward<T>(x, (T)eps, (T)tau, flags & MELLIN_PW_LOG, flags & MELLIN_PW_LIFT,
+                                            outer, t, inner, y, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
+template <typename T>
+int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, double tau, int flags, i64 outer,
+                      i64 t, i64 inner, T *gx, T *grad_params, void *workspace, size_t workspace_bytes,
+                      void *stream) {
+  int rc;
+  if ((rc = check_log_lift(fn, eps, flags, outer, t, inner))) return rc;
+  if (!grad_params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  const size_t need = log_lift_workspace_bytes(outer, t, inner, sizeof(T));
+  if (need && (!x || !gy || !gx)) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  if (need && (!workspace || workspace_bytes < need))
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, need, workspace_bytes);
+  hipError_t e = launch_log_lift_backward<T>(x, gy, (T)eps, (T)tau, flags & MELLIN_PW_LOG, flags & MELLIN_PW_LIFT,
+                                             outer, t, inner, gx, grad_params, (T *)workspace,
+                                             (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
 #define CORR2D_ARGS                                                            \
   batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
   ux, uy
@@ -388,6 +433,30 @@ int mellin_version(void) { return 100; }
 const char *mellin_last_error(void) { return g_error; }
 
 const char *mellin_last_variant(void) { return g_variant; }
+
+int mellin_log_lift_forward_f32(const float *x, double eps, double tau, int flags, int64_t outer, int64_t t,
+                                int64_t inner, float *y, void *stream) {
+  return log_lift_forward<float>("mellin_log_lift_forward_f32", x, eps, tau, flags, outer, t, inner, y, stream);
+}
+int mellin_log_lift_forward_f64(const double *x, double eps, double tau, int flags, int64_t outer, int64_t t,
+                                int64_t inner, double *y, void *stream) {
+  return log_lift_forward<double>("mellin_log_lift_forward_f64", x, eps, tau, flags, outer, t, inner, y, stream);
+}
+size_t mellin_log_lift_backward_workspace(int elem_bytes, int64_t outer, int64_t t, int64_t inner) {
+  return log_lift_workspace_bytes(outer, t, inner, (size_t)elem_bytes);
+}
+int mellin_log_lift_backward_f32(const float *x, const float *grad_y, double eps, double tau, int flags,
+                                 int64_t outer, int64_t t, int64_t inner, float *grad_x, float *grad_params,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+  return log_lift_backward<float>("mellin_log_lift_backward_f32", x, grad_y, eps, tau, flags, outer, t, inner,
+                                  grad_x, grad_params, workspace, workspace_bytes, stream);
+}
+int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double eps, double tau, int flags,
+                                 int64_t outer, int64_t t, int64_t inner, double *grad_x, double *grad_params,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+  return log_lift_backward<double>("mellin_log_lift_backward_f64", x, grad_y, eps, tau, flags, outer, t, inner,
+                                   grad_x, grad_params, workspace, workspace_bytes, stream);
+}
 
 int mellin_set_variant(const char *name) {
   if (!name || !*name) { g_forced = 0; return MELLIN_OK; }

@@ -100,4 +100,14 @@ hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, in
 hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
                           float *grad_input, hipStream_t stream);
 
+// pointwise.hip: log compression and dilation lift over x viewed as (outer, t, inner)
+size_t log_lift_workspace_bytes(i64 outer, i64 t, i64 inner, size_t elem);
+template <typename T>
+hipError_t launch_log_lift_forward(const T *x, T eps, T tau, bool with_log, bool with_lift, i64 outer, i64 t,
+                                   i64 inner, T *y, hipStream_t stream);
+template <typename T>
+hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool with_log, bool with_lift,
+                                    i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
+                                    hipStream_t stream);
+
 }  // namespace mellin

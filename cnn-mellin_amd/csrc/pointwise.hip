@@ -1,0 +1,180 @@
+// The two pointwise layers that sit in front of the first convolution of the
+// reference's acoustic model (models.py:414-417), fused into one pass each way:
+//
+//   log compression   y = log(eps + |x|)                 (layers.py:79-101)
+//   dilation lift     y[.., t, ..] = (t + 1)^tau * x     (layers.py:8-21)
+//   both              y = (t + 1)^tau * log(eps + |x|)
+//
+// x is dense, viewed as (outer, T, inner) with the lifted axis in the middle.
+// PyTorch runs the pair as six elementwise launches forward (abs, add, log,
+// arange/pow, mul, reshape copy) and more backward; here the forward reads x and
+// writes y once, and the backward reads x and grad_y once, writes grad_x once and
+// leaves the two parameter gradients as per-block partial sums that a second
+// small kernel adds up in index order (bit-reproducible, no float atomics).
+//
+// A thread owns one (t, inner) column of the (T, inner) plane and walks down the
+// outer axis: the power (t + 1)^tau, the only expensive function, is evaluated
+// once per thread, and consecutive threads touch consecutive words.
+#include "mellin_common.hpp"
+
+namespace mellin {
+
+namespace {
+
+constexpr int kPwThreads = 256;
+
+template <typename T> __device__ __forceinline__ T sign_of(T v) { return v > T(0) ? T(1) : (v < T(0) ? T(-1) : T(0)); }
+
+template <typename T, bool LOG, bool LIFT>
+__global__ __launch_bounds__(kPwThreads) void log_lift_forward_kernel(
+    const T *__restrict__ x, T eps, T tau, i64 outer, i64 plane, i64 inner, i64 rows_per_block,
+    T *__restrict__ y) {
+  const i64 col = (i64)blockIdx.x * kPwThreads + threadIdx.x;      // t * inner + i
+  if (col >= plane) return;
+  T p = T(1);
+  if (LIFT) p = pow((T)(col / inner + 1), tau);
+  const i64 n0 = (i64)blockIdx.y * rows_per_block, n1 = min(outer, n0 + rows_per_block);
+  for (i64 n = n0; n < n1; ++n) {
+    const T v = x[n * plane + col];
+    const T l = LOG ? log(eps + fabs(v)) : v;
+    y[n * plane + col] = LIFT ? p * l : l;
+  }
+}
+
+// grad_x, and partial sums of d/d eps and d/d tau per block (two values per block)
+template <typename T, bool LOG, bool LIFT>
+__global__ __launch_bounds__(kPwThreads) void log_lift_backward_kernel(
+    const T *__restrict__ x, const T *__restrict__ gy, T eps, T tau, i64 outer, i64 plane, i64 inner,
+    i64 rows_per_block, T *__restrict__ gx, T *__restrict__ partial) {
+  __shared__ T red[2][kPwThreads / 64];
+  const i64 col = (i64)blockIdx.x * kPwThreads + threadIdx.x;
+  T s_eps = T(0), s_tau = T(0);
+  if (col < plane) {
+    T p = T(1), lnt = T(0);
+    if (LIFT) {
+      const T t1 = (T)(col / inner + 1);
+      p = pow(t1, tau);
+      lnt = log(t1);
+    }
+    const i64 n0 = (i64)blockIdx.y * rows_per_block, n1 = min(outer, n0 + rows_per_block);
+    for (i64 n = n0; n < n1; ++n) {
+      const T v = x[n * plane + col], g = gy[n * plane + col];
+      const T gp = g * p;                                  // gradient reaching the logarithm
+      if (LOG) {
+        const T a = eps + fabs(v);
+        const T inv = gp / a;
+        gx[n * plane + col] = inv * sign_of(v);
+        s_eps += inv;
+        if (LIFT) s_tau += gp * lnt * log(a);
+      } else {
+        gx[n * plane + col] = gp;
+        s_tau += gp * lnt * v;
+      }
+    }
+  }
+  // wave sums by shuffles (fixed tree), then the block's wavefronts in order
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    s_eps += __shfl_down(s_eps, o);
+    s_tau += __shfl_down(s_tau, o);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { red[0][wave] = s_eps; red[1][wave] = s_tau; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    T a = T(0), b = T(0);
+    for (int w = 0; w < kPwThreads / 64; ++w) { a += red[0][w]; b += red[1][w]; }
+    const i64 blk = (i64)blockIdx.y * gridDim.x + blockIdx.x;
+    partial[2 * blk] = a;
+    partial[2 * blk + 1] = b;
+  }
+}
+
+// grad_params[0 .. 1] = sums of the partials, in index order (one wavefront:
+// lane l adds partials l, l + 64, ..., then a fixed shuffle tree)
+template <typename T>
+__global__ __launch_bounds__(64) void log_lift_reduce_kernel(const T *__restrict__ partial, i64 blocks,
+                                                             T *__restrict__ grad_params) {
+  T a = T(0), b = T(0);
+  for (i64 i = threadIdx.x; i < blocks; i += 64) { a += partial[2 * i]; b += partial[2 * i + 1]; }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    a += __shfl_down(a, o);
+    b += __shfl_down(b, o);
+  }
+  if (threadIdx.x == 0) { grad_params[0] = a; grad_params[1] = b; }
+}
+
+// Blocks along the outer axis: enough workgroups to fill the chip several times
+// over, but rows_per_block >= 4 so that the power is amortised.
+void shape_grid(i64 outer, i64 plane, dim3 &grid, i64 &rows_per_block) {
+  const i64 gx = (plane + kPwThreads - 1) / kPwThreads;
+  i64 gy = std::max<i64>(1, std::min<i64>((4096 + gx - 1) / gx, (outer + 3) / 4));
+  gy = std::min<i64>(gy, 65535);
+  rows_per_block = (outer + gy - 1) / gy;
+  gy = (outer + rows_per_block - 1) / rows_per_block;
+  grid = dim3((unsigned)gx, (unsigned)gy);
+}
+
+}  // namespace
+
+size_t log_lift_workspace_bytes(i64 outer, i64 t, i64 inner, size_t elem) {
+  if (outer <= 0 || t <= 0 || inner <= 0) return 0;
+  dim3 grid;
+  i64 rpb;
+  shape_grid(outer, t * inner, grid, rpb);
+  return (size_t)grid.x * grid.y * 2 * elem;
+}
+
+template <typename T>
+hipError_t launch_log_lift_forward(const T *x, T eps, T tau, bool with_log, bool with_lift, i64 outer, i64 t,
+                                   i64 inner, T *y, hipStream_t stream) {
+  if (outer <= 0 || t <= 0 || inner <= 0) return hipSuccess;
+  dim3 grid;
+  i64 rpb;
+  shape_grid(outer, t * inner, grid, rpb);
+#define MELLIN_PW_FWD(L_, F_)                                                                    \
+  hipLaunchKernelGGL((log_lift_forward_kernel<T, L_, F_>), grid, dim3(kPwThreads), 0, stream, x, \
+                     eps, tau, outer, t * inner, inner, rpb, y)
+  if (with_log && with_lift) MELLIN_PW_FWD(true, true);
+  else if (with_log) MELLIN_PW_FWD(true, false);
+  else MELLIN_PW_FWD(false, true);
+#undef MELLIN_PW_FWD
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool with_log, bool with_lift,
+                                    i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
+                                    hipStream_t stream) {
+  if (outer <= 0 || t <= 0 || inner <= 0) {
+    hipLaunchKernelGGL((log_lift_reduce_kernel<T>), dim3(1), dim3(64), 0, stream, workspace, (i64)0, grad_params);
+    return hipGetLastError();
+  }
+  dim3 grid;
+  i64 rpb;
+  shape_grid(outer, t * inner, grid, rpb);
+#define MELLIN_PW_BWD(L_, F_)                                                                     \
+  hipLaunchKernelGGL((log_lift_backward_kernel<T, L_, F_>), grid, dim3(kPwThreads), 0, stream, x, \
+                     gy, eps, tau, outer, t * inner, inner, rpb, gx, workspace)
+  if (with_log && with_lift) MELLIN_PW_BWD(true, true);
+  else if (with_log) MELLIN_PW_BWD(true, false);
+  else MELLIN_PW_BWD(false, true);
+#undef MELLIN_PW_BWD
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((log_lift_reduce_kernel<T>), dim3(1), dim3(64), 0, stream, workspace,
+                     (i64)grid.x * grid.y, grad_params);
+  return hipGetLastError();
+}
+
+template hipError_t launch_log_lift_forward<float>(const float *, float, float, bool, bool, i64, i64, i64,
+                                                   float *, hipStream_t);
+template hipError_t launch_log_lift_forward<double>(const double *, double, double, bool, bool, i64, i64, i64,
+                                                    double *, hipStream_t);
+template hipError_t launch_log_lift_backward<float>(const float *, const float *, float, float, bool, bool, i64,
+                                                    i64, i64, float *, float *, float *, hipStream_t);
+template hipError_t launch_log_lift_backward<double>(const double *, const double *, double, double, bool, bool,
+                                                     i64, i64, i64, double *, double *, double *, hipStream_t);
+
+}  // namespace mellin

@@ -198,6 +198,46 @@ MELLIN_DECL_SPEC(mellin_spec2col_f64, double, g, gg);
 MELLIN_DECL_SPEC(mellin_col2spec_f32, float, gg, g);
 MELLIN_DECL_SPEC(mellin_col2spec_f64, double, gg, g);
 
+/* ------------------------------------------------------------------------
+ * 4. The pointwise layers in front of the first convolution
+ *    (models.py:414-417): LogCompression.forward, layers.py:100-101, and
+ *    dilation_lift, layers.py:8-21, one pass each way.
+ *
+ * x, y, grad_y, grad_x are dense and viewed as (outer, t, inner), the lifted
+ * axis in the middle (outer = product of the sizes before it, inner = of those
+ * after it).  flags selects the function:
+ *   MELLIN_PW_LOG                    y = log(eps + |x|)
+ *   MELLIN_PW_LIFT                   y[o, k, i] = (k + 1)^tau * x[o, k, i]
+ *   MELLIN_PW_LOG | MELLIN_PW_LIFT   y[o, k, i] = (k + 1)^tau * log(eps + |x[o, k, i]|)
+ * eps (> 0 with MELLIN_PW_LOG) and tau are the VALUES, not the reference
+ * modules' log_eps / log_tau parameters.  backward WRITES grad_x and
+ * grad_params[0] = sum grad_y * dy/d eps, grad_params[1] = sum grad_y * dy/d tau
+ * (0 for a function that is not selected; |x| has derivative 0 at 0, as in
+ * PyTorch); the sums run in a fixed order.  It needs
+ * mellin_log_lift_backward_workspace() bytes of scratch (256-byte aligned).
+ * ------------------------------------------------------------------------ */
+#define MELLIN_PW_LOG 1
+#define MELLIN_PW_LIFT 2
+
+int mellin_log_lift_forward_f32(const float *x, double eps, double tau, int flags,
+                                int64_t outer, int64_t t, int64_t inner,
+                                float *y, void *stream);
+int mellin_log_lift_forward_f64(const double *x, double eps, double tau, int flags,
+                                int64_t outer, int64_t t, int64_t inner,
+                                double *y, void *stream);
+size_t mellin_log_lift_backward_workspace(int elem_bytes, int64_t outer,
+                                          int64_t t, int64_t inner);
+int mellin_log_lift_backward_f32(const float *x, const float *grad_y, double eps,
+                                 double tau, int flags, int64_t outer, int64_t t,
+                                 int64_t inner, float *grad_x, float *grad_params,
+                                 void *workspace, size_t workspace_bytes,
+                                 void *stream);
+int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double eps,
+                                 double tau, int flags, int64_t outer, int64_t t,
+                                 int64_t inner, double *grad_x, double *grad_params,
+                                 void *workspace, size_t workspace_bytes,
+                                 void *stream);
+
 /* Name of the kernel variant the most recent operator-level call on this
  * thread dispatched to (for tests and profiling): "generic", "mfma" (tiled
  * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"

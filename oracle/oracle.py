@@ -384,3 +384,41 @@ def col2spec(input, spec_size, s=1, d=1, p=0, u=1, impl="port"):
         _col_call("col2spec", gg, g, c_in, batch, (nfx, nfy), ng, (nggx, nggy),
                   s, d, p, u, False, tgg, impl)
     return g
+
+
+# ---- the pointwise layers in front of the convolutions (numpy, float64) ----------
+def log_lift(x, eps=None, tau=None, dim=2):
+    """``[t ** tau *] [log(eps + |x|)]`` with ``t = 1 .. T`` along `dim`.
+
+    Follows the reference's ``LogCompression.forward`` (layers.py:100-101:
+    ``(input.abs() + eps).log()``) and ``dilation_lift`` (layers.py:8-21: the input
+    times ``arange(1, T + 1) ** tau`` broadcast along `dim`); a function that is
+    not selected (``eps`` or ``tau`` None) is skipped."""
+    y = np.asarray(x, dtype=np.float64)
+    if eps is not None:
+        y = np.log(np.abs(y) + float(eps))
+    if tau is not None:
+        shape = [1] * y.ndim
+        shape[dim] = y.shape[dim]
+        y = y * (np.arange(1, y.shape[dim] + 1, dtype=np.float64) ** float(tau)).reshape(shape)
+    return y
+
+
+def log_lift_backward(x, grad_y, eps=None, tau=None, dim=2):
+    """(grad_x, d/d eps, d/d tau) of `log_lift` by the chain rule; |x| has
+    derivative 0 at 0, as in PyTorch's ``abs``."""
+    x = np.asarray(x, dtype=np.float64)
+    g = np.asarray(grad_y, dtype=np.float64)
+    p = np.ones_like(x)
+    lnt = np.zeros_like(x)
+    if tau is not None:
+        shape = [1] * x.ndim
+        shape[dim] = x.shape[dim]
+        t = np.arange(1, x.shape[dim] + 1, dtype=np.float64).reshape(shape)
+        p = p * t ** float(tau)
+        lnt = lnt + np.log(t)
+    gp = g * p
+    if eps is not None:
+        a = np.abs(x) + float(eps)
+        return gp / a * np.sign(x), float((gp / a).sum()), float((gp * lnt * np.log(a)).sum())
+    return gp, 0.0, float((gp * lnt * x).sum())
