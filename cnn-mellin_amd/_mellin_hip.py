@@ -27,7 +27,7 @@ if not os.path.isfile(LIB_PATH):
 
 lib = ctypes.CDLL(LIB_PATH)
 
-_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16"}
 
 # name -> (restype, argtypes); every symbol include/mellin_hip.h declares
 _ACC1D = [_ptr, _ptr] + [_i64] * 10 + [_int] * 3 + [_ptr, _ptr]
@@ -44,6 +44,11 @@ SYMBOLS = {
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
 }
+for _n in ("forward", "backward_input", "backward_weight"):
+    SYMBOLS["mellin_corr2d_%s_f16_workspace" % _n] = (_size_t, [_int] + _DIMS)
+SYMBOLS["mellin_corr2d_forward_f16"] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
+SYMBOLS["mellin_corr2d_backward_input_f16"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
+SYMBOLS["mellin_corr2d_backward_weight_f16"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 _dbl = ctypes.c_double
 PW_LOG, PW_LIFT = 1, 2
 for _t in ("f32", "f64"):
@@ -87,12 +92,14 @@ def _check(code):
         raise RuntimeError("libmellin_hip: %s (code %d)" % (last_error(), code))
 
 
-def suffix(dtype):
+def suffix(dtype, half_ok=True):
+    if dtype == torch.float16 and not half_ok:
+        raise RuntimeError("this entry point takes float32 or float64 tensors, got %s" % dtype)
     try:
         return _SUFFIX[dtype]
     except KeyError:
         raise RuntimeError(
-            "libmellin_hip computes in float32 or float64, got %s" % dtype) from None
+            "libmellin_hip takes float16, float32 or float64 tensors, got %s" % dtype) from None
 
 
 def require_device(*tensors):
@@ -123,7 +130,7 @@ def _dp(t):
 def accumulate(name, f, g, h, c_out, c_in, batch, nf, ng, nh, s, d, p, u, tf, tg, th):
     """Call one of the accumulate-into-h kernels; sizes/params are ints (1-D) or pairs (2-D)."""
     dev = require_device(f, g, h)
-    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(h.dtype)))
+    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(h.dtype, half_ok=False)))
     with torch.cuda.device(dev):
         if isinstance(nf, int):
             code = fn(_dp(f), _dp(g), c_out, c_in, batch, nf, ng, nh, s, d, p, u,
@@ -139,7 +146,7 @@ def accumulate(name, f, g, h, c_out, c_in, batch, nf, ng, nh, s, d, p, u, tf, tg
 def col_op(name, src, dst, c_in, batch, nf, ng, ngg, s, d, p, u, tg, tgg):
     """snd2col / col2snd (ints) or spec2col / col2spec (pairs): `src` -> `dst`, both dense."""
     dev = require_device(src, dst)
-    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(dst.dtype)))
+    fn = getattr(lib, "mellin_%s_%s" % (name, suffix(dst.dtype, half_ok=False)))
     with torch.cuda.device(dev):
         if isinstance(nf, int):
             code = fn(_dp(src), c_in, batch, nf, ng, ngg, s, d, p, u, int(tg), int(tgg), _dp(dst),
@@ -154,7 +161,7 @@ def col_op(name, src, dst, c_in, batch, nf, ng, ngg, s, d, p, u, tg, tgg):
 def log_lift_forward(x, eps, tau, flags, outer, t, inner, y):
     """y = the selected pointwise function of x, both dense and viewed as (outer, t, inner)."""
     dev = require_device(x, y)
-    fn = getattr(lib, "mellin_log_lift_forward_" + suffix(y.dtype))
+    fn = getattr(lib, "mellin_log_lift_forward_" + suffix(y.dtype, half_ok=False))
     with torch.cuda.device(dev):
         _check(fn(_dp(x), float(eps), float(tau), flags, outer, t, inner, _dp(y), _stream(dev)))
     return y
@@ -163,7 +170,7 @@ def log_lift_forward(x, eps, tau, flags, outer, t, inner, y):
 def log_lift_backward(x, grad_y, eps, tau, flags, outer, t, inner, grad_x, grad_params):
     """grad_x and grad_params = (d/d eps, d/d tau); allocates the scratch the library asks for."""
     dev = require_device(x, grad_y, grad_x, grad_params)
-    fn = getattr(lib, "mellin_log_lift_backward_" + suffix(grad_x.dtype))
+    fn = getattr(lib, "mellin_log_lift_backward_" + suffix(grad_x.dtype, half_ok=False))
     need = lib.mellin_log_lift_backward_workspace(grad_x.element_size(), outer, t, inner)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -177,18 +184,34 @@ def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):
             s[0], s[1], d[0], d[1], p[0], p[1], u[0], u[1])
 
 
+def _same_dtype(*tensors):
+    dts = {t.dtype for t in tensors if t is not None}
+    if len(dts) > 1:
+        raise RuntimeError("operands must share one dtype, got %s" % sorted(str(d) for d in dts))
+
+
 def corr2d_forward(kind_x, input, weight, bias, out, dims):
     dev = require_device(input, weight, bias, out)
-    fn = getattr(lib, "mellin_corr2d_forward_" + suffix(out.dtype))
+    _same_dtype(input, weight, bias, out)
     with torch.cuda.device(dev):
-        _check(fn(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))
+        if out.dtype == torch.float16:
+            need = lib.mellin_corr2d_forward_f16_workspace(kind_x, *dims)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+            _check(lib.mellin_corr2d_forward_f16(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out),
+                                                 _ptr(ws.data_ptr()), need, _stream(dev)))
+        else:
+            fn = getattr(lib, "mellin_corr2d_forward_" + suffix(out.dtype))
+            _check(fn(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))
     return out
 
 
 def _workspace(kind_x, which, out, dims, workspace, workspace_bytes):
     if workspace is None:
-        query = getattr(lib, "mellin_corr2d_backward_%s_workspace" % which)
-        workspace_bytes = query(kind_x, out.element_size(), *dims)
+        if out.dtype == torch.float16:
+            workspace_bytes = getattr(lib, "mellin_corr2d_backward_%s_f16_workspace" % which)(kind_x, *dims)
+        else:
+            query = getattr(lib, "mellin_corr2d_backward_%s_workspace" % which)
+            workspace_bytes = query(kind_x, out.element_size(), *dims)
         workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=out.device)
                      if workspace_bytes else None)
     return workspace, workspace_bytes
@@ -201,6 +224,7 @@ def corr2d_backward_input(kind_x, weight, grad_out, grad_input, dims, workspace=
     dev = require_device(weight, grad_out, grad_input)
     workspace, workspace_bytes = _workspace(kind_x, "input", grad_input, dims, workspace,
                                             workspace_bytes)
+    _same_dtype(weight, grad_out, grad_input)
     fn = getattr(lib, "mellin_corr2d_backward_input_" + suffix(grad_input.dtype))
     with torch.cuda.device(dev):
         _check(fn(kind_x, _dp(weight), _dp(grad_out), *dims, _dp(grad_input),
@@ -215,6 +239,7 @@ def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims, workspace
     dev = require_device(input, grad_out, grad_weight)
     workspace, workspace_bytes = _workspace(kind_x, "weight", grad_weight, dims, workspace,
                                             workspace_bytes)
+    _same_dtype(input, grad_out, grad_weight)
     fn = getattr(lib, "mellin_corr2d_backward_weight_" + suffix(grad_weight.dtype))
     with torch.cuda.device(dev):
         _check(fn(kind_x, _dp(input), _dp(grad_out), *dims, _dp(grad_weight),

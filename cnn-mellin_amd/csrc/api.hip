@@ -426,6 +426,31 @@ int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, doubl
   batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
   ux, uy
 
+// ---- half-precision entry points: half tensors, fp32 arithmetic -------------------
+// Each operand is copied to fp32 in the workspace, the fp32 kernels run there, and
+// the result is copied back to half.  Regions are 256-byte aligned.
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+struct HalfLayout {
+  size_t in_off, w_off, b_off, out_off, inner_off, total;   // byte offsets of the fp32 copies
+};
+
+// a, b: element counts of the two operands; bias: of the bias (forward only); r: of the result
+HalfLayout half_layout(i64 a, i64 b, i64 bias, i64 r, size_t inner) {
+  HalfLayout l;
+  l.in_off = 0;
+  l.w_off = l.in_off + align256((size_t)a * 4);
+  l.b_off = l.w_off + align256((size_t)b * 4);
+  l.out_off = l.b_off + align256((size_t)bias * 4);
+  l.inner_off = l.out_off + align256((size_t)r * 4);
+  l.total = l.inner_off + align256(inner);
+  return l;
+}
+
+#define CORR2D_COUNTS                                                              \
+  const i64 n_in = batch * c_in * ngx * ngy, n_w = c_out * c_in * nfx * nfy,      \
+            n_out = batch * c_out * nhx * nhy
+
 extern "C" {
 
 int mellin_version(void) { return 100; }
@@ -433,6 +458,93 @@ int mellin_version(void) { return 100; }
 const char *mellin_last_error(void) { return g_error; }
 
 const char *mellin_last_variant(void) { return g_variant; }
+
+size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  CORR2D_COUNTS;
+  return half_layout(n_in, n_w, c_out, n_out, 0).total;
+}
+int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight, const void *bias,
+                              MELLIN_CORR2D_DIMS, void *out, void *workspace, size_t workspace_bytes,
+                              void *stream) {
+  int rc;
+  if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
+  CORR2D_COUNTS;
+  if (n_out == 0) return MELLIN_OK;
+  const HalfLayout l = half_layout(n_in, n_w, c_out, n_out, 0);
+  if (!workspace || workspace_bytes < l.total)
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, l.total, workspace_bytes);
+  if (!out || (n_in && !input) || (n_w && !weight)) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  char *ws = (char *)workspace;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e = launch_half_to_float(input, (float *)(ws + l.in_off), n_in, st);
+  if (e == hipSuccess) e = launch_half_to_float(weight, (float *)(ws + l.w_off), n_w, st);
+  if (e == hipSuccess && bias) e = launch_half_to_float(bias, (float *)(ws + l.b_off), c_out, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  rc = corr2d_forward<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
+                             bias ? (const float *)(ws + l.b_off) : nullptr, CORR2D_ARGS,
+                             (float *)(ws + l.out_off), stream);
+  if (rc) return rc;
+  e = launch_float_to_half((const float *)(ws + l.out_off), out, n_out, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  CORR2D_COUNTS;
+  return half_layout(n_w, n_out, 0, n_in, mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS)).total;
+}
+int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void *grad_out, MELLIN_CORR2D_DIMS,
+                                     void *grad_input, void *workspace, size_t workspace_bytes, void *stream) {
+  int rc;
+  if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
+  CORR2D_COUNTS;
+  if (n_in == 0) return MELLIN_OK;
+  const size_t inner = mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS);
+  const HalfLayout l = half_layout(n_w, n_out, 0, n_in, inner);
+  if (!workspace || workspace_bytes < l.total)
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, l.total, workspace_bytes);
+  if (!grad_input || (n_w && !weight) || (n_out && !grad_out)) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  char *ws = (char *)workspace;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e = launch_half_to_float(weight, (float *)(ws + l.in_off), n_w, st);
+  if (e == hipSuccess) e = launch_half_to_float(grad_out, (float *)(ws + l.w_off), n_out, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  rc = corr2d_backward_input<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
+                                    CORR2D_ARGS, (float *)(ws + l.out_off), ws + l.inner_off, inner, stream);
+  if (rc) return rc;
+  e = launch_float_to_half((const float *)(ws + l.out_off), grad_input, n_in, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+size_t mellin_corr2d_backward_weight_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  CORR2D_COUNTS;
+  return half_layout(n_in, n_out, 0, n_w, mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS)).total;
+}
+int mellin_corr2d_backward_weight_f16(int kind_x, const void *input, const void *grad_out, MELLIN_CORR2D_DIMS,
+                                      void *grad_weight, void *workspace, size_t workspace_bytes, void *stream) {
+  int rc;
+  if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
+  CORR2D_COUNTS;
+  if (n_w == 0) return MELLIN_OK;
+  const size_t inner = mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS);
+  const HalfLayout l = half_layout(n_in, n_out, 0, n_w, inner);
+  if (!workspace || workspace_bytes < l.total)
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, l.total, workspace_bytes);
+  if (!grad_weight || (n_in && !input) || (n_out && !grad_out)) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  char *ws = (char *)workspace;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e = launch_half_to_float(input, (float *)(ws + l.in_off), n_in, st);
+  if (e == hipSuccess) e = launch_half_to_float(grad_out, (float *)(ws + l.w_off), n_out, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  rc = corr2d_backward_weight<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
+                                     CORR2D_ARGS, (float *)(ws + l.out_off), ws + l.inner_off, inner, stream);
+  if (rc) return rc;
+  e = launch_float_to_half((const float *)(ws + l.out_off), grad_weight, n_w, st);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  return MELLIN_OK;
+}
 
 int mellin_log_lift_forward_f32(const float *x, double eps, double tau, int flags, int64_t outer, int64_t t,
                                 int64_t inner, float *y, void *stream) {

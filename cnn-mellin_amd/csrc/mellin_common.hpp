@@ -110,4 +110,8 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
                                     i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
                                     hipStream_t stream);
 
+// half <-> float copies of n elements (16-byte aligned buffers)
+hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream);
+hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream);
+
 }  // namespace mellin

@@ -168,6 +168,60 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
   return hipGetLastError();
 }
 
+// ---- half <-> float copies (the half-precision entry points compute in fp32) ------
+namespace {
+
+// eight elements per thread where the run allows 16-byte accesses, singly otherwise
+__global__ __launch_bounds__(kPwThreads) void half_to_float_kernel(const _Float16 *__restrict__ src,
+                                                                   float *__restrict__ dst, i64 n) {
+  const i64 i0 = ((i64)blockIdx.x * kPwThreads + threadIdx.x) * 8;
+  if (i0 + 8 <= n) {
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    const half8 v = *(const half8 *)(src + i0);
+    float4 a = make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+    float4 b = make_float4((float)v[4], (float)v[5], (float)v[6], (float)v[7]);
+    *(float4 *)(dst + i0) = a;
+    *(float4 *)(dst + i0 + 4) = b;
+  } else {
+    for (i64 i = i0; i < n; ++i) dst[i] = (float)src[i];
+  }
+}
+
+__global__ __launch_bounds__(kPwThreads) void float_to_half_kernel(const float *__restrict__ src,
+                                                                   _Float16 *__restrict__ dst, i64 n) {
+  const i64 i0 = ((i64)blockIdx.x * kPwThreads + threadIdx.x) * 8;
+  if (i0 + 8 <= n) {
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    const float4 a = *(const float4 *)(src + i0), b = *(const float4 *)(src + i0 + 4);
+    half8 v;
+    v[0] = (_Float16)a.x; v[1] = (_Float16)a.y; v[2] = (_Float16)a.z; v[3] = (_Float16)a.w;
+    v[4] = (_Float16)b.x; v[5] = (_Float16)b.y; v[6] = (_Float16)b.z; v[7] = (_Float16)b.w;
+    *(half8 *)(dst + i0) = v;
+  } else {
+    for (i64 i = i0; i < n; ++i) dst[i] = (_Float16)src[i];
+  }
+}
+
+}  // namespace
+
+// src and dst must be 16-byte aligned (torch allocations and 256-byte aligned
+// workspace regions are)
+hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const i64 blocks = (n + 8 * kPwThreads - 1) / (8 * kPwThreads);
+  hipLaunchKernelGGL(half_to_float_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream,
+                     (const _Float16 *)src, dst, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const i64 blocks = (n + 8 * kPwThreads - 1) / (8 * kPwThreads);
+  hipLaunchKernelGGL(float_to_half_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, src,
+                     (_Float16 *)dst, n);
+  return hipGetLastError();
+}
+
 template hipError_t launch_log_lift_forward<float>(const float *, float, float, bool, bool, i64, i64, i64,
                                                    float *, hipStream_t);
 template hipError_t launch_log_lift_forward<double>(const double *, double, double, bool, bool, i64, i64, i64,

@@ -198,7 +198,11 @@ def _dense_or_transposed(t: torch.Tensor):
 class _Corr2dFunction(torch.autograd.Function):
     """out = bias + correlation(input, weight); x axis Mellin or linear, y axis linear."""
 
+    # Under torch.autocast the floating-point arguments are cast to half and the op runs
+    # with autocast off, as the reference's Autocast registration does
+    # (ext/torch.cpp:405-430); the library then computes in fp32 and rounds once.
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
     def forward(ctx, input, weight, bias, kind_x, s, d, p, u, r, name):
         c_out, c_in, batch = _check_conv_args(name, 4, weight, input, bias)
         nf, ng = tuple(weight.shape[2:]), tuple(input.shape[2:])
@@ -215,6 +219,7 @@ class _Corr2dFunction(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         input, weight = ctx.saved_tensors
         grad_out = grad_out.contiguous()
@@ -323,10 +328,17 @@ def _check_col_args(c: str, dim: int, input: torch.Tensor):
 class _ToColFunction(torch.autograd.Function):
     """gg = x2col(input); backward is col2x (the adjoint gather)."""
 
+    # autocast: cast to half as the reference does (ext/torch.cpp:433-447).  Half tensors
+    # are widened for the library call: the gather moves values unchanged, and the
+    # adjoint's sums are then taken in fp32 and rounded once.
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
     def forward(ctx, input, nf, s, d, p, u, r, name):
         dim = len(nf)
         batch, c_in = _check_col_args(name, dim + 2, input)
+        narrow = input.dtype == torch.float16
+        if narrow:
+            input = input.float()
         ng = tuple(input.shape[2:])
         kinds = (_hip.AX_MCORR, _hip.AX_LCORR)[:dim]
         ngg = tuple(_VALID_SIZE[k](nf[i], ng[i], s[i], d[i], p[i], u[i]) + r[i]
@@ -340,9 +352,10 @@ class _ToColFunction(torch.autograd.Function):
                             tg, False)
             else:
                 _hip.col_op("spec2col", g, gg, c_in, batch, nf, ng, ngg, s, d, p, u, tg, False)
-        return gg
+        return gg.half() if narrow else gg
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         nf, ng, ngg, s, d, p, u, dim = ctx.args
         grad_input = _from_col(grad_out, ng, s, d, p, u, dim)
@@ -353,6 +366,8 @@ def _from_col(cols, ng, s, d, p, u, dim):
     """col2snd / col2spec (ext/torch_cuda.cu:208-235, :267-291)."""
     name = "col2snd" if dim == 1 else "col2spec"
     batch, c_in = _check_col_args(name, 2 + 2 * dim, cols)
+    if cols.dtype == torch.float16:
+        return _from_col(cols.float(), ng, s, d, p, u, dim).half()
     nf = tuple(cols.shape[2:2 + dim])
     ngg = tuple(cols.shape[2 + dim:])
     gg, tgg = _dense_or_transposed(cols)

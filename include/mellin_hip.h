@@ -161,6 +161,29 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       double *grad_weight, void *workspace,
                                       size_t workspace_bytes, void *stream);
 
+/* Half precision (the data type the reference's Autocast registration casts to,
+ * ext/torch.cpp:407-430, before it calls the CUDA kernels instantiated for
+ * c10::Half, ext/torch_cuda.cu:45-177): tensors hold IEEE binary16 values in
+ * the layouts above; all arithmetic is fp32 (operands are widened, products are
+ * accumulated in fp32, the result is rounded to half once).  Every pass needs
+ * scratch memory: the byte count comes from the matching *_workspace() call
+ * (it includes what the fp32 pass underneath needs; 256-byte aligned buffer). */
+size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS);
+int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight,
+                              const void *bias, MELLIN_CORR2D_DIMS, void *out,
+                              void *workspace, size_t workspace_bytes,
+                              void *stream);
+size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS);
+int mellin_corr2d_backward_input_f16(int kind_x, const void *weight,
+                                     const void *grad_out, MELLIN_CORR2D_DIMS,
+                                     void *grad_input, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+size_t mellin_corr2d_backward_weight_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS);
+int mellin_corr2d_backward_weight_f16(int kind_x, const void *input,
+                                      const void *grad_out, MELLIN_CORR2D_DIMS,
+                                      void *grad_weight, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------
  * 3. Column ops: the gather behind the reference's matrix-multiply path and
  *    its adjoint.

@@ -1,0 +1,145 @@
+"""Half precision and autocast (the reference's Autocast registration,
+ext/torch.cpp:405-447, and its tests, tests/test_mconv.py:814-891).
+
+Through the C ABI: half operands, fp32 arithmetic, one rounding of the result.  The
+expected values are the float64 checker on the SAME half-rounded operands, so the only
+error left is the final rounding to half (relative 2^-11) plus the fp32 accumulation
+(rtol 1e-5, atol 1e-5 * sqrt(fan_in)): asserted as rtol 1e-3, atol 1e-3 * sqrt(fan_in) * 1e-2
+-- ten times tighter than the 1e-2 the reference's own autocast tests allow.
+"""
+import numpy as np
+import pytest
+import torch
+
+import _mellin_hip as hip
+import mconv
+from _gpu import to_gpu, to_np
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # kind, n, c_in, c_out, nf, ng, s, d, p, u, r
+    ("mcorr", 3, 4, 10, (5, 3), (40, 17), (1, 1), (2, 1), (1, 1), (1, 1), (0, 0)),
+    ("lcorr", 2, 3, 64, (8, 4), (60, 41), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),     # fused input gradient underneath
+    ("mcorr", 2, 3, 64, (8, 4), (96, 41), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),     # tap products underneath
+    ("lcorr", 2, 40, 70, (3, 3), (30, 20), (2, 1), (1, 2), (1, 1), (1, 1), (1, 0)),    # many channels
+    ("mcorr", 4, 6, 9, (6, 1), (50, 1), (1, 1), (1, 1), (2, 0), (2, 1), (0, 0)),       # 1-D
+]
+
+
+def _close(got, exp, fan_in, what):
+    got = to_np(got.float()).astype(np.float64)
+    tol = 1e-3 * np.abs(exp) + 1e-5 * np.sqrt(fan_in)
+    bad = np.abs(got - exp) > tol
+    assert not bad.any(), "%s: %d of %d off, worst %g" % (what, bad.sum(), bad.size, np.abs(got - exp).max())
+
+
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_half_passes_match_checker_on_the_same_operands(case):
+    kind, n, c_in, c_out, nf, ng, s, d, p, u, r = case
+    kind_x = hip.AX_MCORR if kind == "mcorr" else hip.AX_LCORR
+    fwd = oracle.mcorrlcorr if kind == "mcorr" else oracle.lcorrlcorr
+    bwd = oracle.mcorrlcorr_backward if kind == "mcorr" else oracle.lcorrlcorr_backward
+    rng = np.random.default_rng(800 + CASES.index(case))
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float16)
+    w = (rng.standard_normal((c_out, c_in) + nf) / np.sqrt(c_in * nf[0] * nf[1])).astype(np.float16)
+    b = rng.standard_normal(c_out).astype(np.float16)
+    x64, w64, b64 = x.astype(np.float64), w.astype(np.float64), b.astype(np.float64)
+    exp = fwd(x64, w64, b64, s, d, p, u, r)
+    nh = exp.shape[2:]
+    assert min(nh) > 0
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, u)
+    xg, wg, bg = to_gpu(x), to_gpu(w), to_gpu(b)
+    out = torch.full((n, c_out) + nh, float("nan"), dtype=torch.float16, device="cuda")
+    hip.corr2d_forward(kind_x, xg, wg, bg, out, dims)
+    _close(out, exp, c_in * nf[0] * nf[1], "forward %s" % (case,))
+    go = rng.standard_normal(exp.shape).astype(np.float16)
+    egi, egw, _ = bwd(x64, w64, go.astype(np.float64), s, d, p, u)
+    gi = torch.full_like(xg, float("nan"))
+    hip.corr2d_backward_input(kind_x, wg, to_gpu(go), gi, dims)
+    _close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
+    gw = torch.full_like(wg, float("nan"))
+    hip.corr2d_backward_weight(kind_x, xg, to_gpu(go), gw, dims)
+    _close(gw, egw, n * nh[0] * nh[1], "grad_weight %s" % (case,))
+
+
+def test_workspace_is_required_and_sized():
+    dims = hip._dims(2, 3, 8, (4, 2), (20, 9), (4, 8), (1, 1), (1, 1), (0, 0), (1, 1))
+    x = torch.randn(2, 3, 20, 9, device="cuda").half()
+    w = torch.randn(8, 3, 4, 2, device="cuda").half()
+    out = torch.empty(2, 8, 4, 8, device="cuda", dtype=torch.float16)
+    need = hip.lib.mellin_corr2d_forward_f16_workspace(hip.AX_MCORR, *dims)
+    assert need >= 4 * (x.numel() + w.numel() + out.numel())
+    small = torch.empty(need - 1, dtype=torch.uint8, device="cuda")
+    rc = hip.lib.mellin_corr2d_forward_f16(hip.AX_MCORR, x.data_ptr(), w.data_ptr(), None, *dims, out.data_ptr(),
+                                           small.data_ptr(), need - 1, None)
+    assert rc == 3 and "workspace" in hip.last_error()
+    with pytest.raises(RuntimeError, match="share one dtype"):
+        hip.corr2d_forward(hip.AX_MCORR, x, w.float(), None, out, dims)
+
+
+# ---- autocast: the reference's tests (tests/test_mconv.py:814-891), reduced in size ----
+def test_autocast_mcorrlcorr_func():
+    n, c_in, c_out, t_in, f_in, t_k, f_k = 16, 16, 64, 64, 32, 8, 4
+    input = torch.rand(n, c_in, t_in, f_in, device="cuda", dtype=torch.half).float()
+    weight = torch.rand(c_out, c_in, t_k, f_k, dtype=torch.half, device="cuda").float()
+    bias = torch.rand(c_out, device="cuda", dtype=torch.half).float()
+    out_a = mconv.mcorrlcorr(input, weight, bias).half()
+    with torch.autocast("cuda"):
+        out_b = mconv.mcorrlcorr(input, weight, bias)
+    assert out_b.dtype == torch.half
+    assert torch.allclose(out_a, out_b, rtol=1e-2, atol=1e-2)
+    # here the two differ by the output rounding alone
+    assert torch.allclose(out_a.float(), out_b.float(), rtol=2e-3, atol=1e-3)
+
+
+def test_autocast_mcorr1d_func():
+    n, c_in, c_out, t_in, t_k = 32, 16, 64, 128, 16
+    input = torch.rand(n, c_in, t_in, device="cuda", dtype=torch.half).float()
+    weight = torch.rand(c_out, c_in, t_k, dtype=torch.half, device="cuda").float()
+    bias = torch.rand(c_out, device="cuda", dtype=torch.half).float()
+    out_a = mconv.mcorr1d(input, weight, bias).half()
+    with torch.autocast("cuda"):
+        out_b = mconv.mcorr1d(input, weight, bias)
+    assert out_b.dtype == torch.half
+    assert torch.allclose(out_a, out_b, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("two_d", [False, True], ids=["mcorr1d", "mcorrlcorr"])
+def test_autocast_layer_trains_with_a_grad_scaler(two_d):
+    torch.manual_seed(3)
+    if two_d:
+        layer = mconv.MCorrLCorr(16, 8, (4, 2)).cuda()
+        input = torch.randn(32, 16, 16, 8, device="cuda")
+    else:
+        layer = mconv.MCorr1d(16, 8, 8).cuda()
+        input = torch.randn(32, 16, 16, device="cuda")
+    before = [p_.detach().clone() for p_ in layer.parameters()]
+    optimizer = torch.optim.Adam(layer.parameters())
+    scaler = torch.amp.GradScaler("cuda", init_scale=128.0)     # 65536, the default, overflows half at once
+    optimizer.zero_grad()
+    with torch.autocast("cuda"):
+        output = layer(input)
+        assert output.dtype == torch.half
+        loss = output.float().mean()                    # (a plain sum overflows half in the bias gradient)
+    scaler.scale(loss).backward()
+    for p_ in layer.parameters():
+        assert p_.grad is not None and p_.grad.dtype == torch.float32 and torch.isfinite(p_.grad).all()
+    # the same gradients, unscaled, as the fp32 layer gives (to half accuracy)
+    ref = [torch.autograd.grad(layer(input).mean(), p_)[0] for p_ in layer.parameters()]
+    scale = scaler.get_scale()
+    for p_, g_ in zip(layer.parameters(), ref):
+        assert torch.allclose(p_.grad / scale, g_, rtol=2e-2, atol=2e-2 * float(g_.abs().max()))
+    scaler.step(optimizer)
+    scaler.update()
+    assert any(not torch.equal(a, b_) for a, b_ in zip(before, layer.parameters()))
+
+
+def test_autocast_column_ops():
+    x = torch.randn(3, 2, 30, 11, device="cuda")
+    full = mconv.spec2col(x.half().float(), (4, 3))
+    with torch.autocast("cuda"):
+        cols = mconv.spec2col(x, (4, 3))
+    assert cols.dtype == torch.half
+    assert torch.equal(cols.float(), full)               # a gather moves values unchanged
