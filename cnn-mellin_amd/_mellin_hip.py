@@ -63,6 +63,7 @@ for _t in ("f32", "f64"):
     SYMBOLS["mellin_log_lift_forward_" + _t] = (_int, [_ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr])
     SYMBOLS["mellin_log_lift_backward_" + _t] = (
         _int, [_ptr, _ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
+    SYMBOLS["mellin_corr2d_forward_act_" + _t] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_backward_input_" + _t] = (
         _int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
@@ -190,18 +191,23 @@ def _same_dtype(*tensors):
         raise RuntimeError("operands must share one dtype, got %s" % sorted(str(d) for d in dts))
 
 
-def corr2d_forward(kind_x, input, weight, bias, out, dims):
+ACT_NONE, ACT_RELU = 0, 1
+
+
+def corr2d_forward(kind_x, input, weight, bias, out, dims, activation=ACT_NONE):
     dev = require_device(input, weight, bias, out)
     _same_dtype(input, weight, bias, out)
     with torch.cuda.device(dev):
         if out.dtype == torch.float16:
+            if activation != ACT_NONE:
+                raise RuntimeError("the fused activation is available in float32 and float64")
             need = lib.mellin_corr2d_forward_f16_workspace(kind_x, *dims)
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
             _check(lib.mellin_corr2d_forward_f16(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out),
                                                  _ptr(ws.data_ptr()), need, _stream(dev)))
         else:
-            fn = getattr(lib, "mellin_corr2d_forward_" + suffix(out.dtype))
-            _check(fn(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))
+            fn = getattr(lib, "mellin_corr2d_forward_act_" + suffix(out.dtype))
+            _check(fn(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))
     return out
 
 

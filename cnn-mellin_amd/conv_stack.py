@@ -19,7 +19,7 @@ import torch
 
 import mconv
 
-__all__ = ["ConvStackParams", "ConvStack", "layer_plan"]
+__all__ = ["ConvStackParams", "ConvStack", "layer_plan", "pack_windows"]
 
 
 class ConvStackParams:
@@ -89,6 +89,24 @@ def layer_plan(params: ConvStackParams, time_dim: int, freq_dim: int) -> List[di
     return plan
 
 
+def pack_windows(x: torch.Tensor, lens: torch.Tensor, window_size: int, window_stride: int):
+    """Feature batch ``(N, T, F)`` with lengths -> the windows the convolutions see.
+
+    As ``AcousticModel.forward`` (models.py:395-411): pad ``window_size - 1`` frames at the
+    end, cut windows of ``window_size`` frames every ``window_stride``, keep only the
+    ``(len - 1) // stride + 1`` windows of each utterance that start on a real frame, and fuse
+    utterance and window index (time-major, as ``pack_padded_sequence`` orders them).  Returns
+    the windows ``(N', 1, window_size, F)``, the convolution stack's input, and the
+    ``PackedSequence`` whose ``batch_sizes`` / ``unsorted_indices`` undo the packing."""
+    if window_size > 1:
+        x = torch.nn.functional.pad(x, (0, 0, 0, window_size - 1))
+    windows = x.unfold(1, window_size, window_stride).transpose(2, 3)      # (N, T', w, F)
+    lens_ = torch.div(lens - 1, window_stride, rounding_mode="trunc") + 1
+    packed = torch.nn.utils.rnn.pack_padded_sequence(windows, lens_.cpu(), batch_first=True,
+                                                     enforce_sorted=False)
+    return packed.data.unsqueeze(1).contiguous(), packed
+
+
 class ConvStack(torch.nn.Module):
     """``x (N, C_in, T, F) -> (N, C_out, T', F')`` through the planned layers."""
 
@@ -119,8 +137,11 @@ class ConvStack(torch.nn.Module):
             conv.reset_parameters()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # ReLU, the reference's default (models.py:96-101), is applied by the convolution
+        # kernel itself on the way out; any other callable runs as a pass of its own
+        fused = self.params.nonlinearity in (torch.relu, torch.nn.functional.relu)
         for lay, conv in zip(self.plan, self.convs):
-            x = self.params.nonlinearity(conv(x))
+            x = conv(x, activation="relu") if fused else self.params.nonlinearity(conv(x))
             if lay["pool"]:
                 x = torch.nn.functional.max_pool2d(x, (1, 2))
         return x

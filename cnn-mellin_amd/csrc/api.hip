@@ -147,10 +147,13 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
                    const T *bias, i64 batch, i64 c_in, i64 c_out, i64 nfx,
                    i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy,
                    i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, T *out,
-                   void *stream) {
+                   void *stream, int activation = MELLIN_ACT_NONE) {
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
+  if (activation != MELLIN_ACT_NONE && activation != MELLIN_ACT_RELU)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: activation must be MELLIN_ACT_NONE or MELLIN_ACT_RELU (got %d)", fn,
+                activation);
   const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
   if (batch * c_out * nh == 0) return MELLIN_OK;
   if (!out || (c_in * nf * ng != 0 && (!input || !weight)))
@@ -164,6 +167,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
   pr.g_n = c_in * ng; pr.g_c = ng;
   pr.h_n = c_out * nh; pr.h_m = nh;
   pr.accumulate = 0;
+  pr.relu = activation == MELLIN_ACT_RELU;
   return check_hip(run_sepconv<T>(pr, weight, input, bias, out, (hipStream_t)stream), fn);
 }
 
@@ -459,6 +463,14 @@ const char *mellin_last_error(void) { return g_error; }
 
 const char *mellin_last_variant(void) { return g_variant; }
 
+int mellin_corr2d_forward_act_f32(int kind_x, int activation, const float *input, const float *weight,
+                                  const float *bias, MELLIN_CORR2D_DIMS, float *out, void *stream) {
+  return corr2d_forward<float>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream, activation);
+}
+int mellin_corr2d_forward_act_f64(int kind_x, int activation, const double *input, const double *weight,
+                                  const double *bias, MELLIN_CORR2D_DIMS, double *out, void *stream) {
+  return corr2d_forward<double>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream, activation);
+}
 size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;

@@ -47,7 +47,8 @@ __global__ __launch_bounds__(kThreads) void sepconv_generic_kernel(
     if (pr.accumulate) {
       if (live) *out += acc;
     } else {
-      *out = (bias ? bias[m] : T(0)) + acc;
+      const T v = (bias ? bias[m] : T(0)) + acc;
+      *out = (pr.relu && v < T(0)) ? T(0) : v;
     }
   }
 }

@@ -31,6 +31,7 @@ struct SepConv {
   i64 g_n, g_c;                  // signal strides; spatial part is dense (ngx, ngy)
   i64 h_n, h_m;                  // output strides; spatial part is dense (nhx, nhy)
   int accumulate;                // 1: h += result (h pre-initialised); 0: h = bias + result
+  int relu = 0;                  // with accumulate == 0: h = max(0, bias + result)
 };
 
 // Reduction form used by the weight gradient:

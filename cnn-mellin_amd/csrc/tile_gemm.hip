@@ -201,7 +201,16 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
         }
     }
   };
+  const bool relu = !ACC && pl.relu;
   auto epilogue = [&]() {
+    if (relu) {                                           // the layer's non-linearity, on the way out
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][t][r] = fmaxf(acc[i][t][r], 0.f);
+    }
     if (full_m) write_tile(std::true_type());
     else write_tile(std::false_type());
   };
@@ -314,6 +323,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.nox_eff = (int)X.nh_eff; pl.noy_eff = (int)Y.nh_eff;
   pl.f_m = pr.f_m; pl.f_c = pr.f_c; pl.g_n = pr.g_n; pl.g_c = pr.g_c; pl.h_n = pr.h_n; pl.h_m = pr.h_m;
   pl.accumulate = pr.accumulate;
+  pl.relu = pr.relu && !pr.accumulate;
   pl.kind_x = X.kind; pl.sx = (int)X.s; pl.dx = (int)X.d; pl.px = (int)X.p; pl.ux = (int)X.u;
   pl.uy = (int)Y.u;
 

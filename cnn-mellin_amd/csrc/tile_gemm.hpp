@@ -14,6 +14,7 @@ struct TilePlan {
   int nox_eff, noy_eff;            // outputs at or past these have no tap
   i64 f_m, f_c, g_n, g_c, h_n, h_m;
   int accumulate;
+  int relu;                        // clamp the result at zero before it is stored (accumulate == 0)
   // x axis: Mellin kinds evaluate taps per (row, filter row); linear kinds use
   // the coordinate ax * ox + bx * fx + cx (divided by ux)
   int kind_x, sx, dx, px, ux;

@@ -203,8 +203,12 @@ class _Corr2dFunction(torch.autograd.Function):
     # (ext/torch.cpp:405-430); the library then computes in fp32 and rounds once.
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.float16)
-    def forward(ctx, input, weight, bias, kind_x, s, d, p, u, r, name):
+    def forward(ctx, input, weight, bias, kind_x, s, d, p, u, r, name, activation=None):
         c_out, c_in, batch = _check_conv_args(name, 4, weight, input, bias)
+        if activation not in (None, "relu"):
+            raise RuntimeError('activation must be None or "relu", got %r (while checking arguments for %s)'
+                               % (activation, name))
+        fused = activation == "relu" and input.dtype != torch.float16
         nf, ng = tuple(weight.shape[2:]), tuple(input.shape[2:])
         nh = (_VALID_SIZE[kind_x](nf[0], ng[0], s[0], d[0], p[0], u[0]) + r[0],
               lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], u[1]) + r[1])
@@ -212,8 +216,11 @@ class _Corr2dFunction(torch.autograd.Function):
         input_c, weight_c = input.contiguous(), weight.contiguous()
         bias_c = None if bias is None else bias.contiguous()
         dims = _hip._dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u)
-        _hip.corr2d_forward(kind_x, input_c, weight_c, bias_c, out, dims)
-        ctx.save_for_backward(input_c, weight_c)
+        _hip.corr2d_forward(kind_x, input_c, weight_c, bias_c, out, dims,
+                            _hip.ACT_RELU if fused else _hip.ACT_NONE)
+        if activation == "relu" and not fused:             # half: the library has no fused form
+            out = out.clamp_(min=0)
+        ctx.save_for_backward(input_c, weight_c, *([out] if activation == "relu" else []))
         ctx.has_bias = bias is not None
         ctx.kind_x, ctx.dims = kind_x, dims
         return out
@@ -221,7 +228,9 @@ class _Corr2dFunction(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
-        input, weight = ctx.saved_tensors
+        input, weight = ctx.saved_tensors[:2]
+        if len(ctx.saved_tensors) == 3:                     # through the fused ReLU: pass where out > 0
+            grad_out = grad_out * (ctx.saved_tensors[2] > 0)
         grad_out = grad_out.contiguous()
         grad_input = grad_weight = grad_bias = None
         if ctx.needs_input_grad[0]:
@@ -232,41 +241,43 @@ class _Corr2dFunction(torch.autograd.Function):
                 ctx.kind_x, input, grad_out, torch.empty_like(weight), ctx.dims)
         if ctx.has_bias and ctx.needs_input_grad[2]:
             grad_bias = grad_out.sum((0, 2, 3))
-        return grad_input, grad_weight, grad_bias, None, None, None, None, None, None, None
+        return grad_input, grad_weight, grad_bias, None, None, None, None, None, None, None, None
 
 
-def _corr2d(kind_x, name, input, weight, bias, s, d, p, u, r):
-    return _Corr2dFunction.apply(input, weight, bias, kind_x, s, d, p, u, r, name)
+def _corr2d(kind_x, name, input, weight, bias, s, d, p, u, r, activation=None):
+    return _Corr2dFunction.apply(input, weight, bias, kind_x, s, d, p, u, r, name, activation)
 
 
-def _corr1d(kind, name, input, weight, bias, s, d, p, u, r):
+def _corr1d(kind, name, input, weight, bias, s, d, p, u, r, activation=None):
     # a 1-D layer is the 2-D layer with a unit second axis
     _check_dim(name, weight, "weight", 2, 3)
     _check_dim(name, input, "input", 1, 3)
     out = _Corr2dFunction.apply(
         input.unsqueeze(-1), weight.unsqueeze(-1), bias, kind,
-        (s, 1), (d, 1), (p, 0), (u, 1), (r, 0), name)
+        (s, 1), (d, 1), (p, 0), (u, 1), (r, 0), name, activation)
     return out.squeeze(-1)
 
 
-def _ext_mcorr1d(input, weight, bias=None, s=1, d=1, p=0, u=1, r=0):
+def _ext_mcorr1d(input, weight, bias=None, s=1, d=1, p=0, u=1, r=0, activation=None):
     """``torch.ops.mellin.mcorr1d`` (ext/torch.cpp:469): Mellin correlation, differentiable."""
-    return _corr1d(AX_MCORR, "mcorr1d", input, weight, bias, s, d, p, u, r)
+    return _corr1d(AX_MCORR, "mcorr1d", input, weight, bias, s, d, p, u, r, activation)
 
 
-def _ext_mcorrlcorr(input, weight, bias=None, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1), r=(0, 0)):
+def _ext_mcorrlcorr(input, weight, bias=None, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1), r=(0, 0),
+                    activation=None):
     """``torch.ops.mellin.mcorrlcorr`` (ext/torch.cpp:470)."""
     s, d, p, u, r = (_pair("mcorrlcorr", k, v) for k, v in zip("sdpur", (s, d, p, u, r)))
-    return _corr2d(AX_MCORR, "mcorrlcorr", input, weight, bias, s, d, p, u, r)
+    return _corr2d(AX_MCORR, "mcorrlcorr", input, weight, bias, s, d, p, u, r, activation)
 
 
-def _ext_lcorr1d(input, weight, bias=None, s=1, d=1, p=0, u=1, r=0):
-    return _corr1d(AX_LCORR, "lcorr1d", input, weight, bias, s, d, p, u, r)
+def _ext_lcorr1d(input, weight, bias=None, s=1, d=1, p=0, u=1, r=0, activation=None):
+    return _corr1d(AX_LCORR, "lcorr1d", input, weight, bias, s, d, p, u, r, activation)
 
 
-def _ext_lcorrlcorr(input, weight, bias=None, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1), r=(0, 0)):
+def _ext_lcorrlcorr(input, weight, bias=None, s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1), r=(0, 0),
+                    activation=None):
     s, d, p, u, r = (_pair("lcorrlcorr", k, v) for k, v in zip("sdpur", (s, d, p, u, r)))
-    return _corr2d(AX_LCORR, "lcorrlcorr", input, weight, bias, s, d, p, u, r)
+    return _corr2d(AX_LCORR, "lcorrlcorr", input, weight, bias, s, d, p, u, r, activation)
 
 
 # ---------------------------------------------------------------------------
@@ -416,32 +427,40 @@ def _pick_impl(c: str, _impl):
 
 
 def mcorr1d(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-            s: int = 1, d: int = 1, p: int = 0, r: int = 0, _impl=None) -> torch.Tensor:
+            s: int = 1, d: int = 1, p: int = 0, r: int = 0, _impl=None,
+            activation: Optional[str] = None) -> torch.Tensor:
     """1-D Mellin correlation of ``(batch, in_channels, T_in)`` input with
-    ``(out_channels, in_channels, T_kern)`` weight; see :class:`MCorr1d`."""
+    ``(out_channels, in_channels, T_kern)`` weight; see :class:`MCorr1d`.
+
+    ``activation="relu"`` (not in the reference) returns ``relu(result)`` from the same kernel."""
     _pick_impl("mcorr1d", _impl)
-    return _ext_mcorr1d(input, weight, bias, s, d, p, 1, r)
+    return _ext_mcorr1d(input, weight, bias, s, d, p, 1, r, activation)
 
 
 def mcorrlcorr(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               s: Any = 1, d: Any = 1, p: Any = 0, r: Any = 0, _impl=None) -> torch.Tensor:
-    """2-D correlation, Mellin along axis 2 and linear along axis 3; see :class:`MCorrLCorr`."""
+               s: Any = 1, d: Any = 1, p: Any = 0, r: Any = 0, _impl=None,
+               activation: Optional[str] = None) -> torch.Tensor:
+    """2-D correlation, Mellin along axis 2 and linear along axis 3; see :class:`MCorrLCorr`.
+
+    ``activation="relu"`` (not in the reference) returns ``relu(result)`` from the same kernel."""
     s_, d_, p_, r_ = (_pair("mcorrlcorr", k, v) for k, v in zip("sdpr", (s, d, p, r)))
     _pick_impl("mcorrlcorr", _impl)
-    return _ext_mcorrlcorr(input, weight, bias, s_, d_, p_, (1, 1), r_)
+    return _ext_mcorrlcorr(input, weight, bias, s_, d_, p_, (1, 1), r_, activation)
 
 
 def lcorr1d(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-            s: int = 1, d: int = 1, p: int = 0, r: int = 0) -> torch.Tensor:
+            s: int = 1, d: int = 1, p: int = 0, r: int = 0,
+            activation: Optional[str] = None) -> torch.Tensor:
     """1-D linear correlation with left padding ``p`` and right padding ``r``."""
-    return _ext_lcorr1d(input, weight, bias, s, d, p, 1, r)
+    return _ext_lcorr1d(input, weight, bias, s, d, p, 1, r, activation)
 
 
 def lcorrlcorr(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               s: Any = 1, d: Any = 1, p: Any = 0, r: Any = 0) -> torch.Tensor:
+               s: Any = 1, d: Any = 1, p: Any = 0, r: Any = 0,
+               activation: Optional[str] = None) -> torch.Tensor:
     """2-D linear correlation ("lconv2d") with asymmetric padding ``p`` (left) / ``r`` (right)."""
     s_, d_, p_, r_ = (_pair("lcorrlcorr", k, v) for k, v in zip("sdpr", (s, d, p, r)))
-    return _ext_lcorrlcorr(input, weight, bias, s_, d_, p_, (1, 1), r_)
+    return _ext_lcorrlcorr(input, weight, bias, s_, d_, p_, (1, 1), r_, activation)
 
 
 def snd2col(input: torch.Tensor, kernel_width: int, s: int = 1, d: int = 1, p: int = 0,
@@ -513,8 +532,9 @@ class MCorr1d(_CorrNd):
         p, r = _single("MCorr1d", "p", p), _single("MCorr1d", "r", r)
         super().__init__(in_channels, out_channels, kernel_size, s, d, p, r, bias)
 
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return mcorr1d(input, self.weight, self.bias, self.s[0], self.d[0], self.p[0], self.r[0])
+    def forward(self, input: torch.Tensor, activation: Optional[str] = None) -> torch.Tensor:
+        return mcorr1d(input, self.weight, self.bias, self.s[0], self.d[0], self.p[0], self.r[0],
+                       activation=activation)
 
 
 class MCorrLCorr(_CorrNd):
@@ -537,8 +557,8 @@ class MCorrLCorr(_CorrNd):
         p, r = _pair("MCorrLCorr", "p", p), _pair("MCorrLCorr", "r", r)
         super().__init__(in_channels, out_channels, kernel_size, s, d, p, r, bias)
 
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return mcorrlcorr(input, self.weight, self.bias, self.s, self.d, self.p, self.r)
+    def forward(self, input: torch.Tensor, activation: Optional[str] = None) -> torch.Tensor:
+        return mcorrlcorr(input, self.weight, self.bias, self.s, self.d, self.p, self.r, activation=activation)
 
 
 class LCorr1d(_CorrNd):
@@ -551,8 +571,9 @@ class LCorr1d(_CorrNd):
         p, r = _single("LCorr1d", "p", p), _single("LCorr1d", "r", r)
         super().__init__(in_channels, out_channels, kernel_size, s, d, p, r, bias)
 
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return lcorr1d(input, self.weight, self.bias, self.s[0], self.d[0], self.p[0], self.r[0])
+    def forward(self, input: torch.Tensor, activation: Optional[str] = None) -> torch.Tensor:
+        return lcorr1d(input, self.weight, self.bias, self.s[0], self.d[0], self.p[0], self.r[0],
+                       activation=activation)
 
 
 class LCorrLCorr(_CorrNd):
@@ -567,5 +588,5 @@ class LCorrLCorr(_CorrNd):
         p, r = _pair("LCorrLCorr", "p", p), _pair("LCorrLCorr", "r", r)
         super().__init__(in_channels, out_channels, kernel_size, s, d, p, r, bias)
 
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return lcorrlcorr(input, self.weight, self.bias, self.s, self.d, self.p, self.r)
+    def forward(self, input: torch.Tensor, activation: Optional[str] = None) -> torch.Tensor:
+        return lcorrlcorr(input, self.weight, self.bias, self.s, self.d, self.p, self.r, activation=activation)

@@ -161,6 +161,20 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       double *grad_weight, void *workspace,
                                       size_t workspace_bytes, void *stream);
 
+/* forward with the layer's non-linearity applied on the way out: the acoustic
+ * model runs every convolution as nonlinearity(conv(x)) (models.py:423-425), and
+ * with ReLU, its default, that is out = max(0, bias + correlation) in the same
+ * pass instead of a second read and write of the output.  activation:
+ * MELLIN_ACT_NONE (same as mellin_corr2d_forward_*) or MELLIN_ACT_RELU. */
+#define MELLIN_ACT_NONE 0
+#define MELLIN_ACT_RELU 1
+int mellin_corr2d_forward_act_f32(int kind_x, int activation, const float *input,
+                                  const float *weight, const float *bias,
+                                  MELLIN_CORR2D_DIMS, float *out, void *stream);
+int mellin_corr2d_forward_act_f64(int kind_x, int activation, const double *input,
+                                  const double *weight, const double *bias,
+                                  MELLIN_CORR2D_DIMS, double *out, void *stream);
+
 /* Half precision (the data type the reference's Autocast registration casts to,
  * ext/torch.cpp:407-430, before it calls the CUDA kernels instantiated for
  * c10::Half, ext/torch_cuda.cu:45-177): tensors hold IEEE binary16 values in

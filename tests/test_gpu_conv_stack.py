@@ -138,3 +138,65 @@ def test_full_size_stack_runs_and_is_deterministic():
     for a, b in zip(results[0][2], results[1][2]):
         assert bool(torch.isfinite(a).all())
         assert torch.equal(a, b)
+
+
+# ---- the non-linearity applied by the convolution kernel itself ---------------------
+RELU_CASES = [
+    # op, input shape, weight shape, kwargs
+    ("mcorrlcorr", (3, 3, 60, 20), (40, 3, 5, 3), dict(s=(1, 1), d=(2, 1), p=(1, 1), r=(2, 0))),
+    ("lcorrlcorr", (2, 3, 70, 41), (64, 3, 8, 4), dict()),
+    ("lcorrlcorr", (2, 40, 30, 12), (70, 40, 3, 3), dict(d=(2, 1), p=(2, 1), r=(2, 1))),   # several channel chunks
+    ("mcorr1d", (4, 6, 80), (9, 6, 7), dict(p=2)),
+    ("lcorr1d", (4, 6, 80), (33, 6, 7), dict(s=2)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", RELU_CASES, ids=[c[0] + str(i) for i, c in enumerate(RELU_CASES)])
+def test_fused_relu_equals_relu_of_the_plain_op(case, dtype):
+    name, xs, ws, kw = case
+    op = getattr(mconv, name)
+    torch.manual_seed(RELU_CASES.index(case))
+    x = torch.randn(*xs, device="cuda", dtype=dtype)
+    w = torch.randn(*ws, device="cuda", dtype=dtype) / float(np.prod(ws[1:])) ** 0.5
+    b = torch.randn(ws[0], device="cuda", dtype=dtype) * 0.1
+    xa, wa, ba = (t.clone().requires_grad_(True) for t in (x, w, b))
+    xb, wb, bb = (t.clone().requires_grad_(True) for t in (x, w, b))
+    ya = op(xa, wa, ba, activation="relu", **kw)
+    yb = torch.relu(op(xb, wb, bb, **kw))
+    assert torch.equal(ya, yb)                             # same kernel, same sums: bit for bit
+    assert float((ya == 0).float().mean()) > 0.2           # the clamp is exercised
+    g = torch.randn_like(ya)
+    ya.backward(g)
+    yb.backward(g)
+    for a, b_ in ((xa, xb), (wa, wb), (ba, bb)):
+        assert torch.equal(a.grad, b_.grad)
+    with pytest.raises(RuntimeError, match="activation must be None"):
+        op(x, w, b, activation="tanh", **kw)
+
+
+def test_windows_make_utterances_independent_of_their_batch():
+    """The reference's padding-invariance check (tests/test_models.py:101-152) at the level of
+    the convolution stack: the windows of an utterance give the same features whether the
+    utterance is processed alone or inside a zero-padded batch."""
+    from conv_stack import pack_windows
+    torch.manual_seed(7)
+    n, t_max, f, w_size, w_stride = 4, 50, 12, 10, 3
+    lens = torch.tensor([50, 17, 33, 8])
+    x = torch.randn(n, t_max, f, device="cuda")
+    for i in range(n):
+        x[i, lens[i]:] = 0
+    params = ConvStackParams(layers=3, mellin=True, kernel_time=3, kernel_freq=3, initial_channels=8, seed=5)
+    stack = ConvStack(w_size, f, params).cuda()
+    windows, packed = pack_windows(x, lens, w_size, w_stride)
+    lens_ = (lens - 1) // w_stride + 1
+    assert windows.shape == (int(lens_.sum()), 1, w_size, f)
+    together = stack(windows)
+    feats = torch.nn.utils.rnn.pad_packed_sequence(
+        torch.nn.utils.rnn.PackedSequence(together.sum(2).flatten(1), packed.batch_sizes,
+                                          packed.sorted_indices, packed.unsorted_indices), batch_first=True)[0]
+    for i in range(n):
+        alone, _ = pack_windows(x[i:i + 1, :lens[i]], lens[i:i + 1], w_size, w_stride)
+        ya = stack(alone).sum(2).flatten(1)
+        assert ya.shape[0] == int(lens_[i])
+        np.testing.assert_allclose(to_np(feats[i, :lens_[i]]), to_np(ya), rtol=1e-5, atol=1e-5)
