@@ -12,6 +12,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
+constexpr int kNarrowRow = 17;                     // staged rows this short are loaded 64 words at a time
 
 typedef __attribute__((address_space(3))) float *lds_float_ptr;
 
@@ -178,6 +179,48 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         int cl, r;
         by_R.divmod(wd, cl, r);
         if (r < tg.R_tile) {
+          int gx = -1;
+          if (mellin_x) {
+            int oxl, fx;
+            by_nfx1.divmod(r, oxl, fx);
+            gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
+          } else {
+            const int vx = tg.vx_min + r;
+            if (vx >= 0) {
+              if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
+              else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
+            }
+          }
+          if (gx >= 0) src = cl * g_c + gx * pl.ngy + gy;
+        }
+      }
+      if (src >= 0) load_to_lds_at(Gimg, (unsigned)src * 4u, gs_addr + 4u * (unsigned)w0);
+      else if (wd < words) Gs[wd] = 0.f;
+    }
+    return;
+  }
+  if (pl.RS <= kNarrowRow && (i64)cc * g_c < ((i64)1 << 30)) {
+    // Narrow rows (1-D layers, the last layers of a stack whose frequency axis has shrunk
+    // to a few bins): a load per row would move a handful of words, so a load moves 64
+    // consecutive LDS words instead, lane j fetching the source element of word w0 + j
+    // (rows and columns without a source become zeros).
+    const int words = cc * pl.R * pl.RS;
+    const FastDiv by_RS(pl.RS), by_R(pl.R), by_nfx1(pl.nfx);
+    for (int w0 = wave * 64; w0 < words; w0 += 64 * NW) {
+      const int wd = w0 + lane;
+      int src = -1;
+      if (wd < words) {
+        int row, col, cl, r;
+        by_RS.divmod(wd, row, col);
+        by_R.divmod(row, cl, r);
+        int gy = -1;
+        const int vy = tg.vy_min + col;
+        if (col < tg.RSL && vy >= 0) {
+          if (pl.uy == 1) gy = vy;
+          else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
+          if (gy >= pl.ngy) gy = -1;
+        }
+        if (r < tg.R_tile && gy >= 0) {
           int gx = -1;
           if (mellin_x) {
             int oxl, fx;
