@@ -135,3 +135,31 @@ def test_tap_product_and_two_pass_match_checker(case):
     other, v2 = _grad_input(kind_x, w, go, (n, c_in) + ng, s, d, p, u, "two-pass")
     assert v2 != "mfma-taps+fold", v2
     assert_close(other, exp, fan_in, "%s %s" % (v2, case))
+
+
+WIDE_MELLIN_CASES = [
+    # (n, c_in, c_out, nf, ng, s, d, p, u): Mellin layers with many input channels whose output has
+    # well under 3/4 of the input's rows: dense first pass over grad_out's rows, then the fold
+    (2, 20, 40, (5, 3), (60, 17), (1, 1), (1, 1), (0, 1), (1, 1)),
+    (3, 41, 33, (8, 1), (100, 1), (1, 1), (2, 1), (3, 0), (1, 1)),                  # 1-D, as BASELINE config 2
+    (2, 16, 64, (3, 3), (50, 12), (2, 1), (1, 2), (1, 0), (2, 1)),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_MELLIN_CASES, ids=[str(i) for i in range(len(WIDE_MELLIN_CASES))])
+def test_wide_mellin_layers_take_the_dense_two_pass_path(case):
+    n, c_in, c_out, nf, ng, s, d, p, u = case
+    rng = np.random.default_rng(900 + WIDE_MELLIN_CASES.index(case))
+    x = np.zeros((n, c_in) + ng, dtype=np.float32)
+    w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+    nh = oracle.mcorrlcorr(x, w, None, s, d, p, u, 0).shape[2:]
+    assert min(nh) > 0 and 4 * nh[0] <= 3 * ng[0]
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    exp, _, _ = oracle.mcorrlcorr_backward(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64),
+                                           s, d, p, u)
+    got, v = _grad_input(hip.AX_MCORR, w, go, (n, c_in) + ng, s, d, p, u, None)
+    assert v == "mfma+fold", v
+    assert_close(got, exp, c_out * nf[0] * nf[1], "two-pass %s" % (case,))
+    other, v2 = _grad_input(hip.AX_MCORR, w, go, (n, c_in) + ng, s, d, p, u, "generic")
+    assert v2 == "generic", v2
+    assert_close(other, exp, c_out * nf[0] * nf[1], "generic %s" % (case,))
