@@ -182,23 +182,35 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
       if (!live) continue;
       char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * 4;
 #pragma unroll
-      for (int i = 0; i < MT; ++i)
+      for (int i = 0; i < MT; ++i) {
+        float old[16];
+        if (ACC) {
+          // the 16 old values of this channel tile are fetched in one batch: one round
+          // trip to memory per 16 stores instead of one per store
+          char *q = o;
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int mo = i * 32 + g4 * 8;
+            old[4 * g4 + 0] = (FULL || mo < m_left) ? *(const float *)q : 0.f;
+            old[4 * g4 + 1] = (FULL || mo + 1 < m_left) ? *(const float *)(q + hm1) : 0.f;
+            old[4 * g4 + 2] = (FULL || mo + 2 < m_left) ? *(const float *)(q + hm2) : 0.f;
+            old[4 * g4 + 3] = (FULL || mo + 3 < m_left) ? *(const float *)(q + hm3) : 0.f;
+            q += hm8;
+          }
+        }
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int mo = i * 32 + g4 * 8;
-          auto put = [&](char *at, int row, float v) {
-            if (FULL || row < m_left) {
-              float *dst = (float *)at;
-              if (ACC) *dst += v;
-              else *dst = v;
-            }
+          auto put = [&](char *at, int row, int r) {
+            if (FULL || row < m_left) *(float *)at = ACC ? old[r] + acc[i][t][r] : acc[i][t][r];
           };
-          put(o, mo, acc[i][t][4 * g4]);
-          put(o + hm1, mo + 1, acc[i][t][4 * g4 + 1]);
-          put(o + hm2, mo + 2, acc[i][t][4 * g4 + 2]);
-          put(o + hm3, mo + 3, acc[i][t][4 * g4 + 3]);
+          put(o, mo, 4 * g4);
+          put(o + hm1, mo + 1, 4 * g4 + 1);
+          put(o + hm2, mo + 2, 4 * g4 + 2);
+          put(o + hm3, mo + 3, 4 * g4 + 3);
           o += hm8;                                        // next group of four channels: 8 further on
         }
+      }
     }
   };
   const bool relu = !ACC && pl.relu;
@@ -330,8 +342,10 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   *mt = pr.c_out > 32 ? 2 : 1;
   const int M_T = *mt * 32;
   const i64 m_tiles = (pr.c_out + M_T - 1) / M_T;
-  // two N tiles per wavefront once that still leaves every CU several tiles
-  *nt = (pr.batch * ((Q + 255) / 256) * m_tiles >= 4 * 256) ? 2 : 1;
+  // two N tiles per wavefront once that still leaves every CU several tiles (not when
+  // accumulating into the output: with the old values to fetch as well, that instance
+  // runs out of registers and measured 2-3 times slower than one tile per wavefront)
+  *nt = (!pr.accumulate && pr.batch * ((Q + 255) / 256) * m_tiles >= 4 * 256) ? 2 : 1;
   if (force_nt) *nt = force_nt;
   const int P = kWaves * (*nt) * 32;
 
