@@ -8,8 +8,16 @@
 // relation on y; snd2col / col2snd are the nfy = ngy = nggy = 1 instances.
 // col2spec is written as a gather over the inverse relation (the convolution
 // kind with s and u exchanged), so each output sums its taps in ascending
-// (fx, fy): a fixed order, no atomics.  One thread per output element,
-// coalesced along y; both are pure data movement (HBM bound).
+// (fx, fy): a fixed order, no atomics.  Both are pure data movement (HBM bound).
+//
+// The *_plane kernels are the ones that run unless an extent is out of their
+// 32-bit range: a thread owns one position of the (x, y) plane, works out its taps
+// once (float-reciprocal index splits, no integer division) and then walks over
+// the (image, channel) pairs, so the index arithmetic is amortised and consecutive
+// threads touch consecutive words.  The generic kernels (one thread per element,
+// 64-bit arithmetic throughout) remain for everything else.
+#include <algorithm>
+
 #include "mellin_common.hpp"
 
 namespace mellin {
@@ -67,6 +75,87 @@ __global__ __launch_bounds__(256) void col2spec_kernel(const T *__restrict__ gg,
   }
 }
 
+// gg[nc, tap, q] = g[nc', tap source of q] for q in the (x.nh, y.nh) plane
+template <typename T>
+__global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict__ g, T *__restrict__ gg,
+                                                             Axis x, Axis y, int c_in, int batch,
+                                                             int transposed_g, int transposed_gg) {
+  const int plane = (int)(x.nh * y.nh), ng = (int)(x.ng * y.ng), nfy = (int)y.nf;
+  const int q = blockIdx.x * 256 + threadIdx.x;
+  if (q >= plane) return;
+  const int tap = blockIdx.y, fx = tap / nfy, fy = tap - fx * nfy;
+  int ox = (int)((float)q * (1.0f / (float)y.nh));
+  int oy = q - ox * (int)y.nh;
+  if (oy < 0) { --ox; oy += (int)y.nh; } else if (oy >= (int)y.nh) { ++ox; oy -= (int)y.nh; }
+  const int gx = tap32(x.kind, ox, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u);
+  const int gy = tap32(y.kind, oy, fy, (int)y.ng, (int)y.s, (int)y.d, (int)y.p, (int)y.u);
+  const int src = (gx >= 0 && gy >= 0) ? gx * (int)y.ng + gy : -1;
+  const int taps = (int)(x.nf * y.nf), pairs = batch * c_in;
+#pragma unroll 4
+  for (int nc = blockIdx.z; nc < pairs; nc += gridDim.z) {       // nc: (image, channel) in gg's own order
+    int nc_g = nc;
+    if (transposed_g != transposed_gg) {
+      const int a = transposed_gg ? nc / batch : nc / c_in;       // ci : bt
+      const int b = transposed_gg ? nc - a * batch : nc - a * c_in;
+      nc_g = transposed_gg ? b * c_in + a : b * batch + a;
+    }
+    const T v = src >= 0 ? g[(i64)nc_g * ng + src] : T(0);
+    gg[((i64)nc * taps + tap) * plane + q] = v;
+  }
+}
+
+// g[nc', q] = sum over taps of gg[nc, tap, source of q] for q in the (x.nh, y.nh) signal plane;
+// four (image, channel) pairs per thread share the tap arithmetic
+template <typename T>
+__global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict__ gg, T *__restrict__ g,
+                                                             Axis x, Axis y, int c_in, int batch,
+                                                             int transposed_g, int transposed_gg) {
+  constexpr int NB = 4;
+  const int plane = (int)(x.nh * y.nh), cols = (int)(x.ng * y.ng), nfx = (int)x.nf, nfy = (int)y.nf;
+  const int q = blockIdx.x * 256 + threadIdx.x;
+  if (q >= plane) return;
+  int gx = (int)((float)q * (1.0f / (float)y.nh));
+  int gy = q - gx * (int)y.nh;
+  if (gy < 0) { --gx; gy += (int)y.nh; } else if (gy >= (int)y.nh) { ++gx; gy -= (int)y.nh; }
+  const int pairs = batch * c_in;
+  const i64 per_pair = (i64)nfx * nfy * cols;
+  for (int nc0 = blockIdx.z * NB; nc0 < pairs; nc0 += gridDim.z * NB) {   // nc: pairs in g's own order
+    const T *src[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      int nc = min(nc0 + b, pairs - 1), nc_gg = nc;
+      if (transposed_g != transposed_gg) {
+        const int a = transposed_g ? nc / batch : nc / c_in;
+        const int r = transposed_g ? nc - a * batch : nc - a * c_in;
+        nc_gg = transposed_g ? r * c_in + a : r * batch + a;
+      }
+      src[b] = gg + (i64)nc_gg * per_pair;
+    }
+    T acc[NB] = {T(0), T(0), T(0), T(0)};
+    for (int fx = 0; fx < nfx; ++fx) {
+      const int ox = tap32(x.kind, gx, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u);
+      if (ox < 0) continue;
+      for (int fy = 0; fy < nfy; ++fy) {
+        const int oy = tap32(y.kind, gy, fy, (int)y.ng, (int)y.s, (int)y.d, (int)y.p, (int)y.u);
+        if (oy < 0) continue;
+        const int off = ((fx * nfy + fy) * (int)x.ng + ox) * (int)y.ng + oy;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] += src[b][off];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+      if (nc0 + b < pairs) g[(i64)(nc0 + b) * plane + q] = acc[b];
+  }
+}
+
+// the plane kernels' range: tap numerators and plane sizes within the float-reciprocal
+// splits, per-pair extents within 32 bits
+bool fits_plane_kernels(const Axis &x, const Axis &y, i64 c_in, i64 batch, i64 plane, i64 per_pair) {
+  return axis_fits_tap32(x) && axis_fits_tap32(y) && plane < ((i64)1 << 22) && per_pair < ((i64)1 << 31) &&
+         batch * c_in < ((i64)1 << 30) && x.nf * y.nf <= 65535 && x.ng * y.ng < ((i64)1 << 31);
+}
+
 unsigned blocks_for(i64 total) {
   i64 b = (total + 255) / 256;
   if (b > (1 << 20)) b = 1 << 20;
@@ -80,6 +169,15 @@ hipError_t launch_spec2col(const Axis &x, const Axis &y, i64 c_in, i64 batch, in
                            int transposed_gg, const T *g, T *gg, hipStream_t stream) {
   const i64 total = batch * c_in * x.nf * y.nf * x.nh * y.nh;
   if (total == 0) return hipSuccess;
+  const i64 plane = x.nh * y.nh;
+  if (fits_plane_kernels(x, y, c_in, batch, plane, x.nf * y.nf * plane)) {
+    // enough workgroups to fill the chip, few enough that a thread's tap arithmetic is reused
+    const i64 gx = (plane + 255) / 256, gy = x.nf * y.nf;
+    const i64 gz = std::max<i64>(1, std::min<i64>(batch * c_in, std::min<i64>(65535, (8192 + gx * gy - 1) / (gx * gy))));
+    hipLaunchKernelGGL(spec2col_plane_kernel<T>, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0,
+                       stream, g, gg, x, y, (int)c_in, (int)batch, transposed_g, transposed_gg);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(spec2col_kernel<T>, dim3(blocks_for(total)), dim3(256), 0, stream, g, gg, x, y, c_in,
                      batch, transposed_g, transposed_gg);
   return hipGetLastError();
@@ -90,6 +188,14 @@ hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, in
                            int transposed_gg, const T *gg, T *g, hipStream_t stream) {
   const i64 total = batch * c_in * x.nh * y.nh;
   if (total == 0) return hipSuccess;
+  const i64 plane = x.nh * y.nh;
+  if (fits_plane_kernels(x, y, c_in, batch, plane, x.nf * y.nf * x.ng * y.ng)) {
+    const i64 gx = (plane + 255) / 256, groups = (batch * c_in + 3) / 4;
+    const i64 gz = std::max<i64>(1, std::min<i64>(groups, std::min<i64>(65535, (8192 + gx - 1) / gx)));
+    hipLaunchKernelGGL(col2spec_plane_kernel<T>, dim3((unsigned)gx, 1, (unsigned)gz), dim3(256), 0, stream, gg,
+                       g, x, y, (int)c_in, (int)batch, transposed_g, transposed_gg);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(col2spec_kernel<T>, dim3(blocks_for(total)), dim3(256), 0, stream, gg, g, x, y, c_in,
                      batch, transposed_g, transposed_gg);
   return hipGetLastError();

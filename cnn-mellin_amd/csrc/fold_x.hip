@@ -41,27 +41,6 @@ __global__ __launch_bounds__(256) void fold_x_kernel(Axis x, i64 batch_cin, i64 
   }
 }
 
-// Signal index chosen by (h, f) on one axis, or -1, in 32-bit arithmetic with a
-// float-reciprocal division.  Exact while numerators stay below 2^22 (the
-// launcher checks); p1 = p + 1.
-__device__ __forceinline__ int tap32(int kind, int h, int f, int ng, int s, int d, int p, int u) {
-  int num, den, off = 0;
-  switch (kind) {
-    case AX_MCORR: num = (h + s) * (f + d); den = p + 1; off = u; break;
-    case AX_MCONV: num = (p + 1) * (h + s); den = f + d; off = u; break;
-    case AX_LCORR: num = s * h + d * f - p; den = u; break;
-    default:       num = s * h - d * f + p; den = u; break;
-  }
-  if (num < 0) return -1;                               // linear kinds only; a negative index is no tap
-  int q = (int)((float)num * (1.0f / (float)den));
-  int r = num - q * den;
-  if (r < 0) { --q; r += den; }
-  else if (r >= den) { ++q; r -= den; }
-  if (r != 0) return -1;
-  const int g = q - off;
-  return (g >= 0 && g < ng) ? g : -1;
-}
-
 // Gather that finishes the tap-product input gradient:
 //
 //   grad_input[n, ci, gx, gy] = sum_{fx, fy} Z[n, ci, fx * nfy + fy, hx(gx, fx), hy(gy, fy)]
@@ -205,12 +184,7 @@ hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pa
   i64 blocks = (total + 255) / 256;
   if (blocks > (1 << 20)) blocks = 1 << 20;
   // the 32-bit path: every numerator of the tap relations and the flat index below 2^22 / 2^32
-  const auto small_axis = [](const Axis &a) {
-    const i64 lim = (i64)1 << 22;
-    return (a.nh + a.s) * (a.nf + a.d) < lim && (a.p + 1) * (a.nh + a.s) < lim &&
-           a.s * a.nh + a.d * a.nf + (a.p < 0 ? -a.p : a.p) < lim && a.u < lim && a.p + 1 < lim && a.nf + a.d < lim;
-  };
-  const bool small = small_axis(x) && small_axis(y) && total < ((i64)1 << 32);
+  const bool small = axis_fits_tap32(x) && axis_fits_tap32(y) && total < ((i64)1 << 32);
   const i64 row_blocks = batch_cin * ((x.nh + 31) / 32);
   if (small && x.nf <= 64 && y.nf <= 8 && row_blocks < ((i64)1 << 31) && batch_cin < ((i64)1 << 24) &&
       (i64)nf_pad * x.ng * y.ng < ((i64)1 << 30))

@@ -61,6 +61,34 @@ __host__ __device__ inline i64 tap_index(int kind, i64 h, i64 f, i64 ng, i64 s,
   return (g >= 0 && g < ng) ? g : -1;
 }
 
+// Signal index chosen by (h, f) on one axis, or -1, in 32-bit arithmetic with a
+// float-reciprocal division.  Exact while numerators stay below 2^22 (launchers check
+// axis_fits_tap32); p1 = p + 1.
+__device__ __forceinline__ int tap32(int kind, int h, int f, int ng, int s, int d, int p, int u) {
+  int num, den, off = 0;
+  switch (kind) {
+    case AX_MCORR: num = (h + s) * (f + d); den = p + 1; off = u; break;
+    case AX_MCONV: num = (p + 1) * (h + s); den = f + d; off = u; break;
+    case AX_LCORR: num = s * h + d * f - p; den = u; break;
+    default:       num = s * h - d * f + p; den = u; break;
+  }
+  if (num < 0) return -1;                               // linear kinds only; a negative index is no tap
+  int q = (int)((float)num * (1.0f / (float)den));
+  int r = num - q * den;
+  if (r < 0) { --q; r += den; }
+  else if (r >= den) { ++q; r -= den; }
+  if (r != 0) return -1;
+  const int g = q - off;
+  return (g >= 0 && g < ng) ? g : -1;
+}
+
+// Every numerator of the tap relations of `a` stays below 2^22 (what tap32 needs).
+inline bool axis_fits_tap32(const Axis &a) {
+  const i64 lim = (i64)1 << 22;
+  return (a.nh + a.s) * (a.nf + a.d) < lim && (a.p + 1) * (a.nh + a.s) < lim &&
+         a.s * a.nh + a.d * a.nf + (a.p < 0 ? -a.p : a.p) < lim && a.u < lim && a.p + 1 < lim && a.nf + a.d < lim;
+}
+
 inline i64 support_size(int kind, i64 nf, i64 ng, i64 s, i64 d, i64 p, i64 u) {
   i64 v;
   switch (kind) {
