@@ -202,7 +202,7 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   // (nhx well below ngx, as whenever r does not stretch the output): the first pass here
   // works on the nhx rows of grad_out, the gather form on the ngx rows of grad_input,
   // most of whose (position, filter row) pairs have no tap at all
-  const bool mellin_wide = kind_x == AX_MCORR && c_in >= 16 && 4 * nhx <= 3 * ngx;
+  const bool mellin_wide = kind_x == AX_MCORR && c_in >= 16 && 8 * nhx <= 7 * ngx;
   if ((c_in >= 16 && !mellin_wide) || nfx < 2) return false;
   if (mellin_wide && (double)batch * m2 * nhx * ngy * 4.0 > (double)kMaxTapProductBytes) return false;
   const i64 pad = ((m2 + 31) / 32) * 32;

@@ -10,36 +10,14 @@
 //
 //   grad_input[n, ci, gx, gy] = sum_{fx} Y[n, ci * nfx + fx, hx(gx, fx), gy]
 //
-// over the fx whose tap exists, in ascending fx (a fixed order: no atomics).
-// One thread per output element, coalesced along gy.
+// over the fx whose tap exists, in ascending fx (a fixed order: no atomics).  That
+// is the column-to-signal adjoint with a trivial y axis, so the column-op kernel
+// does it (col_ops.hip).
 #include "mellin_common.hpp"
 
 namespace mellin {
 
 namespace {
-
-__global__ __launch_bounds__(256) void fold_x_kernel(Axis x, i64 batch_cin, i64 ngx, i64 ngy,
-                                                     const float *__restrict__ Y,
-                                                     float *__restrict__ gi) {
-  // x: convolution-kind axis with nf = nfx, ng = nhx (rows of Y), nh = ngx (rows of grad_input)
-  const i64 total = batch_cin * ngx * ngy;
-  const i64 nhx = x.ng, nfx = x.nf;
-  const i64 step = (i64)gridDim.x * blockDim.x;
-  for (i64 i = (i64)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
-    const i64 gy = i % ngy;
-    const i64 r = i / ngy;
-    const i64 gx = r % ngx, nc = r / ngx;              // nc = n * c_in + ci
-    const float *Ync = Y + nc * nfx * nhx * ngy + gy;
-    float acc = 0.f;
-    if (gx < x.nh_eff) {
-      for (i64 fx = 0; fx < nfx; ++fx) {
-        const i64 hx = tap_index(x.kind, gx, fx, nhx, x.s, x.d, x.p, x.u);
-        if (hx >= 0) acc += Ync[(fx * nhx + hx) * ngy];
-      }
-    }
-    gi[i] = acc;
-  }
-}
 
 // Gather that finishes the tap-product input gradient:
 //
@@ -201,13 +179,11 @@ hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pa
 
 hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
                          float *grad_input, hipStream_t stream) {
-  const i64 total = batch_cin * ngx * ngy;
-  if (total == 0) return hipSuccess;
-  i64 blocks = (total + 255) / 256;
-  if (blocks > (1 << 20)) blocks = 1 << 20;
-  hipLaunchKernelGGL(fold_x_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, batch_cin, ngx,
-                     ngy, Y, grad_input);
-  return hipGetLastError();
+  // x: convolution-kind axis with nf = nfx, ng = nhx (rows of Y), nh = ngx (rows of grad_input);
+  // Y is (batch_cin, nfx, 1, nhx, ngy): columns with an identity y axis
+  (void)ngx;
+  const Axis y = make_axis(AX_LCONV, 1, ngy, ngy, 1, 1, 0, 1);
+  return launch_col2spec<float>(x, y, batch_cin, 1, 0, 0, Y, grad_input, stream);
 }
 
 }  // namespace mellin

@@ -139,7 +139,7 @@ def test_tap_product_and_two_pass_match_checker(case):
 
 WIDE_MELLIN_CASES = [
     # (n, c_in, c_out, nf, ng, s, d, p, u): Mellin layers with many input channels whose output has
-    # well under 3/4 of the input's rows: dense first pass over grad_out's rows, then the fold
+    # under 7/8 of the input's rows: dense first pass over grad_out's rows, then the fold
     (2, 20, 40, (5, 3), (60, 17), (1, 1), (1, 1), (0, 1), (1, 1)),
     (3, 41, 33, (8, 1), (100, 1), (1, 1), (2, 1), (3, 0), (1, 1)),                  # 1-D, as BASELINE config 2
     (2, 16, 64, (3, 3), (50, 12), (2, 1), (1, 2), (1, 0), (2, 1)),
@@ -153,7 +153,7 @@ def test_wide_mellin_layers_take_the_dense_two_pass_path(case):
     x = np.zeros((n, c_in) + ng, dtype=np.float32)
     w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
     nh = oracle.mcorrlcorr(x, w, None, s, d, p, u, 0).shape[2:]
-    assert min(nh) > 0 and 4 * nh[0] <= 3 * ng[0]
+    assert min(nh) > 0 and 8 * nh[0] <= 7 * ng[0]
     go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
     exp, _, _ = oracle.mcorrlcorr_backward(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64),
                                            s, d, p, u)
