@@ -105,20 +105,20 @@ __global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict
 }
 
 // g[nc', q] = sum over taps of gg[nc, tap, source of q] for q in the (x.nh, y.nh) signal plane;
-// four (image, channel) pairs per thread share the tap arithmetic
+// eight (image, channel) pairs per thread share the tap arithmetic
 template <typename T>
 __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict__ gg, T *__restrict__ g,
                                                              Axis x, Axis y, int c_in, int batch,
-                                                             int transposed_g, int transposed_gg) {
-  constexpr int NB = 4;
-  const int plane = (int)(x.nh * y.nh), cols = (int)(x.ng * y.ng), nfx = (int)x.nf, nfy = (int)y.nf;
+                                                             int transposed_g, int transposed_gg,
+                                                             i64 per_pair) {   // words from one pair's columns to the next
+  constexpr int NB = 8;
+  const int plane = (int)(x.nh * y.nh), nfx = (int)x.nf, nfy = (int)y.nf;
   const int q = blockIdx.x * 256 + threadIdx.x;
   if (q >= plane) return;
   int gx = (int)((float)q * (1.0f / (float)y.nh));
   int gy = q - gx * (int)y.nh;
   if (gy < 0) { --gx; gy += (int)y.nh; } else if (gy >= (int)y.nh) { ++gx; gy -= (int)y.nh; }
   const int pairs = batch * c_in;
-  const i64 per_pair = (i64)nfx * nfy * cols;
   for (int nc0 = blockIdx.z * NB; nc0 < pairs; nc0 += gridDim.z * NB) {   // nc: pairs in g's own order
     const T *src[NB];
 #pragma unroll
@@ -131,7 +131,9 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
       }
       src[b] = gg + (i64)nc_gg * per_pair;
     }
-    T acc[NB] = {T(0), T(0), T(0), T(0)};
+    T acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b] = T(0);
     for (int fx = 0; fx < nfx; ++fx) {
       const int ox = tap32(x.kind, gx, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u);
       if (ox < 0) continue;
@@ -190,15 +192,29 @@ hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, in
   if (total == 0) return hipSuccess;
   const i64 plane = x.nh * y.nh;
   if (fits_plane_kernels(x, y, c_in, batch, plane, x.nf * y.nf * x.ng * y.ng)) {
-    const i64 gx = (plane + 255) / 256, groups = (batch * c_in + 3) / 4;
+    const i64 gx = (plane + 255) / 256, groups = (batch * c_in + 7) / 8;
     const i64 gz = std::max<i64>(1, std::min<i64>(groups, std::min<i64>(65535, (8192 + gx - 1) / gx)));
     hipLaunchKernelGGL(col2spec_plane_kernel<T>, dim3((unsigned)gx, 1, (unsigned)gz), dim3(256), 0, stream, gg,
-                       g, x, y, (int)c_in, (int)batch, transposed_g, transposed_gg);
+                       g, x, y, (int)c_in, (int)batch, transposed_g, transposed_gg, x.nf * y.nf * x.ng * y.ng);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(col2spec_kernel<T>, dim3(blocks_for(total)), dim3(256), 0, stream, gg, g, x, y, c_in,
                      batch, transposed_g, transposed_gg);
   return hipGetLastError();
+}
+
+// The same adjoint over columns whose tap planes are padded to `taps_padded` per pair
+// (the tap products of the input gradient); false if the plane kernel's range is exceeded.
+bool launch_col2spec_padded(const Axis &x, const Axis &y, i64 pairs, i64 taps_padded, const float *gg,
+                            float *g, hipStream_t stream, hipError_t *err) {
+  const i64 plane = x.nh * y.nh, per_pair = taps_padded * x.ng * y.ng;
+  if (!fits_plane_kernels(x, y, pairs, 1, plane, per_pair)) return false;
+  const i64 gx = (plane + 255) / 256, groups = (pairs + 7) / 8;
+  const i64 gz = std::max<i64>(1, std::min<i64>(groups, std::min<i64>(65535, (8192 + gx - 1) / gx)));
+  hipLaunchKernelGGL(col2spec_plane_kernel<float>, dim3((unsigned)gx, 1, (unsigned)gz), dim3(256), 0, stream, gg,
+                     g, x, y, (int)pairs, 1, 0, 0, per_pair);
+  *err = hipGetLastError();
+  return true;
 }
 
 template hipError_t launch_spec2col<float>(const Axis &, const Axis &, i64, i64, int, int, const float *,

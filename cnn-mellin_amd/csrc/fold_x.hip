@@ -89,86 +89,23 @@ __global__ __launch_bounds__(256) void fold_xy_kernel(Axis x, Axis y, i64 batch_
   }
 }
 
-// The same gather, one wavefront per 8 consecutive grad_input rows of one
-// (image, channel), lanes along gy.  The y taps of a column do not depend on
-// the row, so a lane works them out once; the x taps of a row do not depend on
-// the column, so lane fx works out tap fx and the wavefront reads them back as
-// scalars.  For filters of at most 64 x 8 taps and indices on the 32-bit path.
-__global__ __launch_bounds__(256) void fold_xy_rows_kernel(Axis x, Axis y, int batch_cin, int nf_pad,
-                                                           const float *__restrict__ Z,
-                                                           float *__restrict__ gi) {
-  const int ngx = (int)x.nh, ngy = (int)y.nh, nhx = (int)x.ng, nhy = (int)y.ng;
-  const int nfx = (int)x.nf, nfy = (int)y.nf;
-  const i64 nh = (i64)nhx * nhy;
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int blocks_per_nc = (ngx + 31) >> 5;
-  const int nc = blockIdx.x / blocks_per_nc;
-  const int gx0 = (blockIdx.x - nc * blocks_per_nc) * 32 + wave * 8;
-  const float *Znc = Z + (i64)nc * nf_pad * nh;
-  float *out = gi + (i64)nc * ngx * ngy;
-  for (int gy0 = 0; gy0 < ngy; gy0 += 64) {
-    const int gy = gy0 + lane;
-    const bool live = gy < ngy;
-    // word of this column's tap fy inside a (channel, filter row, grad_out row) block
-    // of Z: fy * nh + hy, or -1
-    int yoff[8];
-#pragma unroll
-    for (int fy = 0; fy < 8; ++fy) {
-      const int hy = (live && gy < (int)y.nh_eff && fy < nfy)
-                         ? tap32(y.kind, gy, fy, nhy, (int)y.s, (int)y.d, (int)y.p, (int)y.u) : -1;
-      yoff[fy] = hy < 0 ? -1 : fy * (int)nh + hy;
-    }
-    for (int r = 0; r < 8; ++r) {
-      const int gx = gx0 + r;
-      if (gx >= ngx) break;
-      const int hx_lane = (lane < nfx && gx < (int)x.nh_eff)
-                              ? tap32(x.kind, gx, lane, nhx, (int)x.s, (int)x.d, (int)x.p, (int)x.u) : -1;
-      float acc = 0.f;
-      // eight filter rows at a time: every load is issued before the first sum, so a
-      // row costs one memory round trip rather than one per tap; the sums keep
-      // their (fx, fy) order.  Row bases are scalars, lane offsets 32-bit.
-      for (int fxc = 0; fxc < nfx; fxc += 8) {
-        float v[8][8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int fx = fxc + j;
-          const int hx = fx < nfx ? __builtin_amdgcn_readlane(hx_lane, fx & 63) : -1;
-          if (hx >= 0) {
-            const unsigned row = (unsigned)(fx * nfy) * (unsigned)nh + (unsigned)(hx * nhy);
-#pragma unroll
-            for (int fy = 0; fy < 8; ++fy) v[j][fy] = yoff[fy] >= 0 ? Znc[row + (unsigned)yoff[fy]] : 0.f;
-          } else {
-#pragma unroll
-            for (int fy = 0; fy < 8; ++fy) v[j][fy] = 0.f;
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-          for (int fy = 0; fy < 8; ++fy) acc += v[j][fy];
-      }
-      if (live) out[(i64)gx * ngy + gy] = acc;
-    }
-  }
-}
-
 }  // namespace
 
 hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
                           float *grad_input, hipStream_t stream) {
   const i64 total = batch_cin * x.nh * y.nh;
   if (total == 0) return hipSuccess;
+  {
+    // the column-to-signal adjoint over padded tap planes: a thread works out a
+    // position's taps once for eight (image, channel) pairs
+    hipError_t e = hipSuccess;
+    if (launch_col2spec_padded(x, y, batch_cin, nf_pad, Z, grad_input, stream, &e)) return e;
+  }
   i64 blocks = (total + 255) / 256;
   if (blocks > (1 << 20)) blocks = 1 << 20;
   // the 32-bit path: every numerator of the tap relations and the flat index below 2^22 / 2^32
   const bool small = axis_fits_tap32(x) && axis_fits_tap32(y) && total < ((i64)1 << 32);
-  const i64 row_blocks = batch_cin * ((x.nh + 31) / 32);
-  if (small && x.nf <= 64 && y.nf <= 8 && row_blocks < ((i64)1 << 31) && batch_cin < ((i64)1 << 24) &&
-      (i64)nf_pad * x.ng * y.ng < ((i64)1 << 30))
-    hipLaunchKernelGGL(fold_xy_rows_kernel, dim3((unsigned)row_blocks), dim3(256), 0, stream, x, y,
-                       (int)batch_cin, nf_pad, Z, grad_input);
-  else if (small)
+  if (small)
     hipLaunchKernelGGL(fold_xy_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, x, y, batch_cin,
                        nf_pad, Z, grad_input);
   else

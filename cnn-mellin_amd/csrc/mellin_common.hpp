@@ -126,6 +126,9 @@ template <typename T>
 hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
                            int transposed_gg, const T *gg, T *g, hipStream_t stream);
 
+bool launch_col2spec_padded(const Axis &x, const Axis &y, i64 pairs, i64 taps_padded, const float *gg,
+                            float *g, hipStream_t stream, hipError_t *err);
+
 hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
                           float *grad_input, hipStream_t stream);
 
