@@ -159,60 +159,21 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
                          gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + count4));
     return;
   }
-  if (pl.RS == 1 && (i64)cc * g_c < ((i64)1 << 30)) {
-    // Single-column rows (1-D layers): a virtual row is one word, so a load moves 64
-    // of them, lane j fetching the source element of LDS word w0 + j.  The column
-    // (and whether it exists at all) is the same for every row.
-    const int vy = tg.vy_min;
-    int gy = -1;
-    if (vy >= 0) {
-      if (pl.uy == 1) gy = vy;
-      else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
-      if (gy >= pl.ngy) gy = -1;
-    }
-    const int words = cc * pl.R;
-    const FastDiv by_R(pl.R), by_nfx1(pl.nfx);
-    for (int w0 = wave * 64; w0 < words; w0 += 64 * NW) {
-      const int wd = w0 + lane;
-      int src = -1;
-      if (wd < words && gy >= 0) {
-        int cl, r;
-        by_R.divmod(wd, cl, r);
-        if (r < tg.R_tile) {
-          int gx = -1;
-          if (mellin_x) {
-            int oxl, fx;
-            by_nfx1.divmod(r, oxl, fx);
-            gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
-          } else {
-            const int vx = tg.vx_min + r;
-            if (vx >= 0) {
-              if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
-              else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
-            }
-          }
-          if (gx >= 0) src = cl * g_c + gx * pl.ngy + gy;
-        }
-      }
-      if (src >= 0) load_to_lds_at(Gimg, (unsigned)src * 4u, gs_addr + 4u * (unsigned)w0);
-      else if (wd < words) Gs[wd] = 0.f;
-    }
-    return;
-  }
   if (pl.RS <= kNarrowRow && (i64)cc * g_c < ((i64)1 << 30)) {
     // Narrow rows (1-D layers, the last layers of a stack whose frequency axis has shrunk
     // to a few bins): a load per row would move a handful of words, so a load moves 64
-    // consecutive LDS words instead, lane j fetching the source element of word w0 + j
-    // (rows and columns without a source become zeros).
-    const int words = cc * pl.R * pl.RS;
-    const FastDiv by_RS(pl.RS), by_R(pl.R), by_nfx1(pl.nfx);
-    for (int w0 = wave * 64; w0 < words; w0 += 64 * NW) {
+    // consecutive LDS words of one channel's block instead, lane j fetching the source
+    // element of word w0 + j (rows and columns without a source become zeros).  Where a
+    // word comes from does not depend on the channel, so a lane works it out once per
+    // block of 64 words and the loads of all the chunk's channels reuse it.
+    const int plane = pl.R * pl.RS;                           // words per channel
+    const FastDiv by_RS(pl.RS), by_nfx1(pl.nfx);
+    for (int w0 = wave * 64; w0 < plane; w0 += 64 * NW) {
       const int wd = w0 + lane;
       int src = -1;
-      if (wd < words) {
-        int row, col, cl, r;
-        by_RS.divmod(wd, row, col);
-        by_R.divmod(row, cl, r);
+      if (wd < plane) {
+        int r = wd, col = 0;
+        if (pl.RS > 1) by_RS.divmod(wd, r, col);
         int gy = -1;
         const int vy = tg.vy_min + col;
         if (col < tg.RSL && vy >= 0) {
@@ -233,11 +194,13 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
               else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
             }
           }
-          if (gx >= 0) src = cl * g_c + gx * pl.ngy + gy;
+          if (gx >= 0) src = gx * pl.ngy + gy;
         }
       }
-      if (src >= 0) load_to_lds_at(Gimg, (unsigned)src * 4u, gs_addr + 4u * (unsigned)w0);
-      else if (wd < words) Gs[wd] = 0.f;
+      for (int cl = 0; cl < cc; ++cl) {
+        if (src >= 0) load_to_lds_at(Gimg + cl * g_c, (unsigned)src * 4u, gs_addr + 4u * (unsigned)(cl * plane + w0));
+        else if (wd < plane) Gs[cl * plane + wd] = 0.f;
+      }
     }
     return;
   }
