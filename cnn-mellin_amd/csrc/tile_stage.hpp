@@ -204,14 +204,17 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
     }
     return;
   }
-  const FastDiv by_rows(tg.R_tile), by_nfx(pl.nfx);
-  for (int base = 0; base < total_rows; base += 64 * NW) {
-    // per-lane: row base + 4 * lane + wave
-    const int rr = base + NW * lane + wave;
-    int src_off = -1, dst_off = 0;
-    if (rr < total_rows) {
-      int cl, r;
-      by_rows.divmod(rr, cl, r);
+  // Which signal row a virtual row holds does not depend on the channel: the lanes work
+  // it out for 64 rows of a channel's block at a time, and the loads of every channel of
+  // the chunk reuse it.
+  const FastDiv by_nfx(pl.nfx);
+  const int plane = pl.R * pl.RS;                              // words per channel
+  (void)total_rows;
+  for (int base = 0; base < tg.R_tile; base += 64 * NW) {
+    // per-lane: row base + NW * lane + wave of the channel's block
+    const int r = base + NW * lane + wave;
+    int src_off = -1;
+    if (r < tg.R_tile) {
       int gx = -1;
       if (mellin_x) {
         int oxl, fx;
@@ -224,10 +227,10 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
           else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
         }
       }
-      if (gx >= 0) src_off = cl * g_c + gx * pl.ngy;
-      dst_off = (cl * pl.R + r) * pl.RS;
+      if (gx >= 0) src_off = gx * pl.ngy;
     }
-    const int mine = min(64, (total_rows - base - wave + NW - 1) / NW);
+    const int dst_off = r * pl.RS;
+    const int mine = min(64, (tg.R_tile - base - wave + NW - 1) / NW);
     for (int cb = 0; cb < tg.RSL; cb += 64) {
       const int col = cb + lane;
       const int vy = tg.vy_min + col;
@@ -238,23 +241,19 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
         if (gy >= pl.ngy) gy = -1;
       }
-      // lanes whose column has a source: one load per row that has a source
-      if (gy >= 0) {
-        const unsigned voff = (unsigned)gy * 4u;
-        for (int j = 0; j < mine; ++j) {
-          const int s_src = __builtin_amdgcn_readlane(src_off, j);
-          if (s_src >= 0) {
-            const int s_dst = __builtin_amdgcn_readlane(dst_off, j);
-            load_to_lds_at(Gimg + s_src, voff, gs_addr + 4u * (unsigned)(s_dst + cb));
+      const unsigned voff = (unsigned)max(gy, 0) * 4u;
+      const bool pad_col = gy < 0;
+      for (int j = 0; j < mine; ++j) {
+        const int s_src = __builtin_amdgcn_readlane(src_off, j);
+        const int s_dst = __builtin_amdgcn_readlane(dst_off, j) + cb;
+        if (s_src >= 0) {
+          // lanes whose column has a source load it; padding columns become zeros
+          for (int cl = 0; cl < cc; ++cl) {
+            if (!pad_col) load_to_lds_at(Gimg + cl * g_c + s_src, voff, gs_addr + 4u * (unsigned)(cl * plane + s_dst));
+            else if (in_row) Gs[cl * plane + s_dst + lane] = 0.f;
           }
-        }
-      }
-      // zeros: padding columns of every row, and whole rows without a source
-      if (in_row) {
-        const bool pad_col = gy < 0;
-        for (int j = 0; j < mine; ++j) {
-          const int s_src = __builtin_amdgcn_readlane(src_off, j);
-          if (pad_col || s_src < 0) Gs[__builtin_amdgcn_readlane(dst_off, j) + col] = 0.f;
+        } else if (in_row) {
+          for (int cl = 0; cl < cc; ++cl) Gs[cl * plane + s_dst + lane] = 0.f;   // a row without a source
         }
       }
     }
