@@ -47,7 +47,10 @@ namespace {
 #define MELLIN_PROBE_DECL
 #endif
 
-template <int MT, int NT, bool ACC>
+// MB: 64-word blocks per wave whose staging sources are kept from a tile's first
+// chunk for its other chunks (0: nothing kept; the instance for layers whose
+// channels fit in one or two chunks).
+template <int MT, int NT, bool ACC, int MB>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H) {
@@ -57,6 +60,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   // they are used instead of all being held in scalar registers for the whole
   // kernel, which had the register allocator spill hundreds of them to vector
   // lanes around the stores and the staging code.
+  constexpr int kMemo = MB;
   typedef const __attribute__((address_space(4))) TilePlan ConstPlan;
   ConstPlan *const plan_base = (ConstPlan *)__builtin_amdgcn_kernarg_segment_ptr();
   ConstPlan *plp = plan_base;
@@ -77,7 +81,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   const int tid = threadIdx.x;
   // the wave index is wave-uniform: say so, and everything derived from it (row
   // loops, base addresses) is computed on the scalar unit
-  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, wave_id = __builtin_amdgcn_readfirstlane(tid >> 6), wave = wave_id;
   const int half = lane >> 5, l32 = lane & 31;
   const int m0 = blockIdx.y * M_T;
   const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
@@ -87,37 +91,63 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   // direct loads, coalesced along the taps; taps past the chunk and channels past M
   // are zero
   const unsigned lds_base = lds_address(lds);
-  auto issue_filter = [&](int c0, int cc, int ws_word) {        // ws_word: where the block starts in lds[]
+  // (cl * f_c + t) * 4 of tap k = lane of a chunk: the same in every stage
+  unsigned w_voff0;
+  {
+    const FastDiv by_nf(pl.nf);
+    int cl, t;
+    by_nf.divmod(lane, cl, t);
+    w_voff0 = (unsigned)(((i64)cl * pl.f_c + t) * 4);              // < 4 GB: checked by the plan
+  }
+  // first: the buffer has not been filled by this workgroup before.  Rows of channels
+  // that do not exist and the odd tap's partner are zeros that no load overwrites, so
+  // they are written on the first fill only (and again by a last, shorter chunk).
+  auto issue_filter = [&](int c0, int cc, int ws_word, bool first) {   // ws_word: where the block starts in lds[]
     const int KC = cc * pl.nf;
     const int m_live = max(0, min(M_T, pl.M - m0));       // channels of this block that exist
     const int KC4 = KC & ~3;
+    const bool zero_cols = first || cc < pl.CC;
+    const float *row = F + (i64)(m0 + wave) * pl.f_m + (i64)c0 * pl.f_c;   // this wave's first channel
+    const i64 row_step = (i64)kWaves * pl.f_m;
+    unsigned dst = lds_base + 4u * (unsigned)(ws_word + wave * pl.WSS);
+    const unsigned dst_step = 4u * (unsigned)(kWaves * pl.WSS);
     if (pl.f_c == pl.nf && ((KC4 + 255) >> 8) + (KC4 < KC) < ((pl.KCp + 63) >> 6)) {
       // the taps of consecutive channels are one run of KC words per output channel:
       // 16 bytes per lane, then the last KC % 4 words singly (taken when that is
       // fewer instructions than 64 single words at a time)
       for (int m = wave; m < m_live; m += kWaves) {
-        const float *row = F + (i64)(m0 + m) * pl.f_m + (i64)c0 * pl.f_c;
-        const unsigned dst = lds_base + 4u * (unsigned)(ws_word + m * pl.WSS);
         for (int kb = 0; kb < KC4; kb += 256)
           if (kb + 4 * lane < KC4) load16_to_lds_at(row, (unsigned)(kb + 4 * lane) * 4u, dst + 4u * (unsigned)kb);
         if (lane < KC - KC4) load_to_lds_at(row, (unsigned)(KC4 + lane) * 4u, dst + 4u * (unsigned)KC4);
-        if (lane < pl.KCp - KC) lds[ws_word + m * pl.WSS + KC + lane] = 0.f;     // KCp - KC <= 1
+        if (zero_cols && lane < pl.KCp - KC) lds[ws_word + m * pl.WSS + KC + lane] = 0.f;
+        row += row_step;
+        dst += dst_step;
       }
-      for (int m = m_live + wave; m < M_T; m += kWaves)
-        for (int k = lane; k < pl.KCp; k += 64) lds[ws_word + m * pl.WSS + k] = 0.f;
+      if (first)
+        for (int m = m_live + wave; m < M_T; m += kWaves)
+          for (int k = lane; k < pl.KCp; k += 64) lds[ws_word + m * pl.WSS + k] = 0.f;
       return;
     }
     const FastDiv by_nf(pl.nf);
     for (int kb = 0; kb < pl.KCp; kb += 64) {
       const int k = kb + lane;
-      int cl, t;
-      by_nf.divmod(k, cl, t);
-      const unsigned voff = (unsigned)(((i64)(c0 + cl) * pl.f_c + t) * 4);   // < 4 GB: checked by the plan
+      unsigned voff = w_voff0;
+      if (kb > 0) {
+        int cl, t;
+        by_nf.divmod(k, cl, t);
+        voff = (unsigned)(((i64)cl * pl.f_c + t) * 4);
+      }
       if (k < KC) {
-        for (int m = wave; m < m_live; m += kWaves)
-          load_to_lds_at(F + (i64)(m0 + m) * pl.f_m, voff, lds_base + 4u * (unsigned)(ws_word + m * pl.WSS + kb));
-        for (int m = m_live + wave; m < M_T; m += kWaves) lds[ws_word + m * pl.WSS + k] = 0.f;
-      } else if (k < pl.KCp) {
+        const float *r = row;
+        unsigned d = dst + 4u * (unsigned)kb;
+        for (int m = wave; m < m_live; m += kWaves) {
+          load_to_lds_at(r, voff, d);
+          r += row_step;
+          d += dst_step;
+        }
+        if (first)
+          for (int m = m_live + wave; m < M_T; m += kWaves) lds[ws_word + m * pl.WSS + k] = 0.f;
+      } else if (zero_cols && k < pl.KCp && (first || k == KC)) {
         for (int m = wave; m < M_T; m += kWaves) lds[ws_word + m * pl.WSS + k] = 0.f;
       }
     }
@@ -128,12 +158,21 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   const int my_tiles = (int)blockIdx.x < pl.total_tiles
                            ? (pl.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
   const int my_stages = my_tiles * chunks;
+  StageMemo<kMemo> memo = {};
+  // (stage_zero: a zero renewed every stage that the compiler cannot see through; adding
+  // it to the wave index keeps the staging addresses from being worked out once for the
+  // whole kernel and then held in registers across the matrix loops)
+  unsigned stage_zero = 0;
   auto issue_stage = [&](int st, int ti, int ch) {           // st = ti * chunks + ch
+    const int wave = wave_id + (int)stage_zero;
     const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
     const int c0 = ch * pl.CC, cc = min(pl.CC, pl.C - c0);
     const int sb = (st & 1) * (pl.sbuf - 1) * g_words;    // sbuf == 1: a workgroup has one stage only
-    issue_signal(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave);
-    if (!single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words);
+    // the sources worked out for a tile's first chunk serve its other chunks; a buffer's
+    // zeros (padding, rows without a tap) survive from the tile's chunk two stages back
+    issue_signal<kWaves, kMemo>(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave,
+                               &memo, ch == 0, ch < 2);
+    if (!single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
   };
 
   {
@@ -149,7 +188,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   }
   MELLIN_STAMP(0);
   if (my_stages > 0) {
-    if (single_chunk) issue_filter(0, pl.C, ws_word0);
+    if (single_chunk) issue_filter(0, pl.C, ws_word0, true);
     issue_stage(0, 0, 0);
   }
   MELLIN_STAMP(1);
@@ -231,6 +270,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
       unsigned zero;                                      // a zero the compiler cannot see through
       asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
       plp = (ConstPlan *)((const __attribute__((address_space(4))) char *)plan_base + zero);
+      stage_zero = zero;
     }
     // every wave's loads for this stage have landed, and every wave is done
     // reading the buffer the next stage will fill
@@ -288,10 +328,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
 #undef pl
 }
 
-template <int MT, int NT, bool ACC>
+template <int MT, int NT, bool ACC, int MB>
 hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const float *f,
                           const float *g, const float *bias, float *h, hipStream_t stream) {
-  auto kern = tile_gemm_kernel<MT, NT, ACC>;
+  auto kern = tile_gemm_kernel<MT, NT, ACC, MB>;
   if (lds_bytes > 64 * 1024) {
     // opt in to more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per CU)
     static thread_local size_t granted = 0;
@@ -458,10 +498,16 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   gx = std::min(gx, pl.total_tiles);
   if (pl.sbuf == 1 && gx < pl.total_tiles) return hipErrorInvalidValue;   // one buffer: one stage per workgroup
   dim3 grid((unsigned)gx, (unsigned)m_tiles);
+  // layers staged in three or more chunks of channels keep a tile's staging sources
+  const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
-  if (mt == MT_ && nt == NT_)                                                                \
-    return pl.accumulate ? launch_variant<MT_, NT_, true>(pl, lds_bytes, grid, f, g, bias, h, stream) \
-                         : launch_variant<MT_, NT_, false>(pl, lds_bytes, grid, f, g, bias, h, stream);
+  if (mt == MT_ && nt == NT_) {                                                              \
+    if (pl.accumulate)                                                                       \
+      return memo ? launch_variant<MT_, NT_, true, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)  \
+                  : launch_variant<MT_, NT_, true, 0>(pl, lds_bytes, grid, f, g, bias, h, stream); \
+    return memo ? launch_variant<MT_, NT_, false, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)   \
+                : launch_variant<MT_, NT_, false, 0>(pl, lds_bytes, grid, f, g, bias, h, stream);  \
+  }
   MELLIN_TILE_CASE(2, 2)
   MELLIN_TILE_CASE(2, 1)
   MELLIN_TILE_CASE(1, 2)

@@ -127,17 +127,49 @@ __device__ __forceinline__ TileGeom tile_geometry(const PL &pl, int tile_id, boo
 
 
 // ---- signal rows of one (tile, channel range) --------------------------------
+// Where a staged word comes from depends on the tile, not on the channel, and a
+// layer with many channels stages the same tile once per chunk of channels: a
+// wave can keep what it worked out for the tile's first chunk (a few registers
+// per lane) and spend the later chunks on load instructions only.
+template <int MB>                                  // MB: 64-word blocks per wave whose sources are kept
+struct StageMemo {
+  int row_src, row_dst;                            // row-wise staging: lane j <-> the wave's j-th row
+  int word_src[MB > 0 ? MB : 1];                   // word-wise staging: lane's word of the wave's b-th block
+};
+
+// The same LDS target in every channel of a chunk: channel cl reads cl * g_c floats
+// further on and lands cl planes further on.
+__device__ __forceinline__ void load_channels(const float *base, int g_c, unsigned voff, unsigned lds_addr,
+                                              unsigned plane_bytes, int cc) {
+  for (int cl = 0; cl < cc; ++cl) {
+    load_to_lds_at(base, voff, lds_addr);
+    base += g_c;
+    lds_addr += plane_bytes;
+  }
+}
+__device__ __forceinline__ void zero_channels(float *at, int plane, int cc) {
+  for (int cl = 0; cl < cc; ++cl) { *at = 0.f; at += plane; }
+}
+
 // wave w of the NW that stage together owns virtual rows w, w + NW, ...; 64 lanes
 // first work out the source of 64 such rows, then direct loads are issued per row
 // with the lanes on columns; columns or rows without a source are written as zeros.
-template <int NW = kWaves, class PL>
+// Words without a source are written only when `fresh` (the buffer last held
+// another tile: within a tile the same words are zeros in every chunk).  MB > 0:
+// `memo` carries the tile's sources from the call with new_tile set to the calls
+// for the tile's other chunks.  MB < 0: no memo, and everything is written on
+// every call.
+template <int NW = kWaves, int MB = -1, class PL>
 __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
                                              const float *__restrict__ G, int c0, int cc,
                                              float *Gs, unsigned gs_addr, bool mellin_x, int lane,
-                                             int wave) {
-  const int total_rows = cc * tg.R_tile;
+                                             int wave, StageMemo<MB> *memo = nullptr, bool new_tile = true,
+                                             bool fresh = true) {
   const float *Gimg = G + (i64)tg.n * pl.g_n + (i64)c0 * pl.g_c;
   const int g_c = (int)pl.g_c;                         // fits: c_in * ngx * ngy < 2^31
+  constexpr bool MEMO = MB > 0;
+  if (MB < 0) fresh = true;
+  if (!MEMO) new_tile = true;
   if (pl.contig && tg.vx_min >= 0 && tg.vx_min + tg.R_tile <= pl.ngx) {
     // the virtual rows ARE the signal rows vx_min ... of each channel, with the
     // signal's own row pitch: one run of R_tile * ngy words per channel, moved
@@ -159,6 +191,8 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
                          gs_addr + 4u * (unsigned)(cl * pl.R * pl.RS + count4));
     return;
   }
+  const int plane = pl.R * pl.RS;                              // words per channel
+  const unsigned plane_bytes = 4u * (unsigned)plane;
   if (pl.RS <= kNarrowRow && (i64)cc * g_c < ((i64)1 << 30)) {
     // Narrow rows (1-D layers, the last layers of a stack whose frequency axis has shrunk
     // to a few bins): a load per row would move a handful of words, so a load moves 64
@@ -166,59 +200,26 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
     // element of word w0 + j (rows and columns without a source become zeros).  Where a
     // word comes from does not depend on the channel, so a lane works it out once per
     // block of 64 words and the loads of all the chunk's channels reuse it.
-    const int plane = pl.R * pl.RS;                           // words per channel
     const FastDiv by_RS(pl.RS), by_nfx1(pl.nfx);
-    for (int w0 = wave * 64; w0 < plane; w0 += 64 * NW) {
+    // source element of word w0 + lane: >= 0 its index in the channel plane, -1 none
+    // (a zero), -2 past the end of the block
+    auto source_of = [&](int w0) -> int {
       const int wd = w0 + lane;
-      int src = -1;
-      if (wd < plane) {
-        int r = wd, col = 0;
-        if (pl.RS > 1) by_RS.divmod(wd, r, col);
-        int gy = -1;
-        const int vy = tg.vy_min + col;
-        if (col < tg.RSL && vy >= 0) {
-          if (pl.uy == 1) gy = vy;
-          else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
-          if (gy >= pl.ngy) gy = -1;
-        }
-        if (r < tg.R_tile && gy >= 0) {
-          int gx = -1;
-          if (mellin_x) {
-            int oxl, fx;
-            by_nfx1.divmod(r, oxl, fx);
-            gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
-          } else {
-            const int vx = tg.vx_min + r;
-            if (vx >= 0) {
-              if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
-              else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
-            }
-          }
-          if (gx >= 0) src = gx * pl.ngy + gy;
-        }
+      if (wd >= plane) return -2;
+      int r = wd, col = 0;
+      if (pl.RS > 1) by_RS.divmod(wd, r, col);
+      int gy = -1;
+      const int vy = tg.vy_min + col;
+      if (col < tg.RSL && vy >= 0) {
+        if (pl.uy == 1) gy = vy;
+        else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
+        if (gy >= pl.ngy) gy = -1;
       }
-      for (int cl = 0; cl < cc; ++cl) {
-        if (src >= 0) load_to_lds_at(Gimg + cl * g_c, (unsigned)src * 4u, gs_addr + 4u * (unsigned)(cl * plane + w0));
-        else if (wd < plane) Gs[cl * plane + wd] = 0.f;
-      }
-    }
-    return;
-  }
-  // Which signal row a virtual row holds does not depend on the channel: the lanes work
-  // it out for 64 rows of a channel's block at a time, and the loads of every channel of
-  // the chunk reuse it.
-  const FastDiv by_nfx(pl.nfx);
-  const int plane = pl.R * pl.RS;                              // words per channel
-  (void)total_rows;
-  for (int base = 0; base < tg.R_tile; base += 64 * NW) {
-    // per-lane: row base + NW * lane + wave of the channel's block
-    const int r = base + NW * lane + wave;
-    int src_off = -1;
-    if (r < tg.R_tile) {
+      if (r >= tg.R_tile || gy < 0) return -1;
       int gx = -1;
       if (mellin_x) {
         int oxl, fx;
-        by_nfx.divmod(r, oxl, fx);
+        by_nfx1.divmod(r, oxl, fx);
         gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
       } else {
         const int vx = tg.vx_min + r;
@@ -227,9 +228,64 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
           else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
         }
       }
-      if (gx >= 0) src_off = gx * pl.ngy;
+      return gx >= 0 ? gx * pl.ngy + gy : -1;
+    };
+    auto move = [&](int w0, int src) {
+      if (src >= 0) load_channels(Gimg, g_c, (unsigned)src * 4u, gs_addr + 4u * (unsigned)w0, plane_bytes, cc);
+      else if (fresh && src == -1) zero_channels(Gs + w0 + lane, plane, cc);
+    };
+    if (MEMO) {
+      // the wave's first MB blocks from the memo, any further ones worked out each time
+      if (new_tile) {
+        int blk = 0;
+        for (int w0 = wave * 64; w0 < plane && blk < MB; w0 += 64 * NW, ++blk) {
+          const int src = source_of(w0);
+#pragma unroll
+          for (int b = 0; b < MB; ++b) memo->word_src[b] = b == blk ? src : memo->word_src[b];
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const int w0 = (wave + NW * b) * 64;
+        if (w0 < plane) move(w0, memo->word_src[b]);
+      }
+      for (int w0 = (wave + NW * MB) * 64; w0 < plane; w0 += 64 * NW) move(w0, source_of(w0));
+      return;
     }
-    const int dst_off = r * pl.RS;
+    for (int w0 = wave * 64; w0 < plane; w0 += 64 * NW) move(w0, source_of(w0));
+    return;
+  }
+  // Which signal row a virtual row holds does not depend on the channel: the lanes work
+  // it out for 64 rows of a channel's block at a time, and the loads of every channel of
+  // the chunk reuse it.
+  const FastDiv by_nfx(pl.nfx);
+  for (int base = 0; base < tg.R_tile; base += 64 * NW) {
+    // per-lane: row base + NW * lane + wave of the channel's block
+    int src_off, dst_off;
+    if (MEMO && base == 0 && !new_tile) {
+      src_off = memo->row_src;
+      dst_off = memo->row_dst;
+    } else {
+      const int r = base + NW * lane + wave;
+      src_off = -1;
+      if (r < tg.R_tile) {
+        int gx = -1;
+        if (mellin_x) {
+          int oxl, fx;
+          by_nfx.divmod(r, oxl, fx);
+          gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
+        } else {
+          const int vx = tg.vx_min + r;
+          if (vx >= 0) {
+            if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
+            else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
+          }
+        }
+        if (gx >= 0) src_off = gx * pl.ngy;
+      }
+      dst_off = r * pl.RS;
+      if (MEMO && base == 0) { memo->row_src = src_off; memo->row_dst = dst_off; }
+    }
     const int mine = min(64, (tg.R_tile - base - wave + NW - 1) / NW);
     for (int cb = 0; cb < tg.RSL; cb += 64) {
       const int col = cb + lane;
@@ -248,12 +304,10 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         const int s_dst = __builtin_amdgcn_readlane(dst_off, j) + cb;
         if (s_src >= 0) {
           // lanes whose column has a source load it; padding columns become zeros
-          for (int cl = 0; cl < cc; ++cl) {
-            if (!pad_col) load_to_lds_at(Gimg + cl * g_c + s_src, voff, gs_addr + 4u * (unsigned)(cl * plane + s_dst));
-            else if (in_row) Gs[cl * plane + s_dst + lane] = 0.f;
-          }
-        } else if (in_row) {
-          for (int cl = 0; cl < cc; ++cl) Gs[cl * plane + s_dst + lane] = 0.f;   // a row without a source
+          if (!pad_col) load_channels(Gimg + s_src, g_c, voff, gs_addr + 4u * (unsigned)s_dst, plane_bytes, cc);
+          if (fresh && pad_col && in_row) zero_channels(Gs + s_dst + lane, plane, cc);
+        } else if (fresh && in_row) {
+          zero_channels(Gs + s_dst + lane, plane, cc);         // a row without a source
         }
       }
     }
