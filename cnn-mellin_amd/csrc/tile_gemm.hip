@@ -406,6 +406,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.total_tiles = pl.batch * pl.tiles_per_image;
   auto magic = [](int d) { return d <= 1 ? 0xFFFFFFFFu : (unsigned)(0x100000000ull / (unsigned)d); };
   pl.mg_tpi = magic(pl.tiles_per_image); pl.mg_cpr = magic(pl.chunks_per_row); pl.mg_noy = magic(pl.noy);
+  pl.mg_p1 = magic((int)X.p + 1);
   const int RT = pl.segment ? 1 : std::min(pl.nox, (P - 1 + pl.noy - 1) / pl.noy + 1);
   const int oy_span = pl.segment ? P : pl.noy;
   const i64 RSL = (i64)pl.ay * (oy_span - 1) + pl.by_span + 1;

@@ -25,6 +25,7 @@ struct TilePlan {
   // tiling
   int segment, chunks_per_row, tiles_per_image, total_tiles;
   unsigned mg_tpi, mg_cpr, mg_noy;  // floor(2^32 / d) for tiles_per_image, chunks_per_row, noy (see udiv)
+  unsigned mg_p1;                   // the same for px + 1 (Mellin correlation taps)
   int R, RS;                       // virtual rows per channel and their stride (words)
   int sbuf;                        // signal buffers in LDS: 2, or 1 when no workgroup has a second stage
   int contig;                      // virtual rows coincide with the signal's rows (same pitch): block copies

@@ -56,13 +56,31 @@ __device__ __forceinline__ void wait_all_memory() {
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 }
 
+// x / d for 0 <= x < 2^31 and d >= 1 with m = floor(2^32 / d) (0xFFFFFFFF for d = 1):
+// the product's high word is the quotient or one less.  On wave-uniform values this
+// is a handful of scalar instructions; a plain integer division goes through the
+// vector unit's reciprocal, and vector instructions queue behind the matrix ones.
+__device__ __forceinline__ int udiv(int x, int d, unsigned m) {
+  unsigned q = __umulhi((unsigned)x, m);
+  if ((unsigned)x - q * (unsigned)d >= (unsigned)d) ++q;
+  return (int)q;
+}
+
 // Signal row chosen by (output row, filter row) on a Mellin axis, in 32-bit
 // arithmetic (the plan guarantees that the products fit).  p1 = p + 1.
-__device__ __forceinline__ int mellin_tap32(int kind, int h, int f, int ng, int s, int d, int p1, int u) {
+// mg_p1 = floor(2^32 / p1) (0xFFFFFFFF for p1 = 1).
+__device__ __forceinline__ int mellin_tap32(int kind, int h, int f, int ng, int s, int d, int p1, int u,
+                                            unsigned mg_p1) {
   int num, den;
-  if (kind == AX_MCORR) { num = (h + s) * (f + d); den = p1; }
-  else { num = p1 * (h + s); den = f + d; }
-  const int q = num / den;
+  int q;
+  if (kind == AX_MCORR) {
+    // the divisor is the same for every tap: multiply-high by its reciprocal
+    num = (h + s) * (f + d); den = p1;
+    q = udiv(num, p1, mg_p1);
+  } else {
+    num = p1 * (h + s); den = f + d;
+    q = num / den;
+  }
   if (q * den != num) return -1;
   const int g = q - u;
   return (g >= 0 && g < ng) ? g : -1;
@@ -80,16 +98,6 @@ struct FastDiv {
     else if (r >= d) { ++q; r -= d; }
   }
 };
-
-// x / d for 0 <= x < 2^31 and d >= 1 with m = floor(2^32 / d) (0xFFFFFFFF for d = 1):
-// the product's high word is the quotient or one less.  On wave-uniform values this
-// is a handful of scalar instructions; a plain integer division goes through the
-// vector unit's reciprocal, and vector instructions queue behind the matrix ones.
-__device__ __forceinline__ int udiv(int x, int d, unsigned m) {
-  unsigned q = __umulhi((unsigned)x, m);
-  if ((unsigned)x - q * (unsigned)d >= (unsigned)d) ++q;
-  return (int)q;
-}
 
 // Uniform description of one position tile.
 struct TileGeom {
@@ -220,7 +228,7 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
       if (mellin_x) {
         int oxl, fx;
         by_nfx1.divmod(r, oxl, fx);
-        gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
+        gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux, pl.mg_p1);
       } else {
         const int vx = tg.vx_min + r;
         if (vx >= 0) {
@@ -273,7 +281,7 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         if (mellin_x) {
           int oxl, fx;
           by_nfx.divmod(r, oxl, fx);
-          gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux);
+          gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux, pl.mg_p1);
         } else {
           const int vx = tg.vx_min + r;
           if (vx >= 0) {

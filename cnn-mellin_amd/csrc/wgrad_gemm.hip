@@ -222,6 +222,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
 // vector instruction saved in the loop is matrix throughput gained.)
 // grad_out rows arrive by 16-byte direct loads (the four rows of a unit are
 // contiguous per channel); the input rows are staged as in the forward kernel.
+constexpr int kRowsMemo = 8;                       // 64-word blocks per wave whose staging sources are kept
 template <int MT, int JT>
 __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     WgradPlan wp, const float *__restrict__ A, const float *__restrict__ G,
@@ -270,17 +271,23 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     }
   }
 
+  // Units are numbered with the image running fastest and a workgroup takes a
+  // contiguous range of them: consecutive units are then the same rows of successive
+  // images, and where a staged word comes from (and which words are zeros) stays what
+  // it was for the unit before.
   const int units_per_image = (pl.nox_eff + RB - 1) / RB;
   const int total_units = pl.batch * units_per_image;
-  const int my_units = (int)blockIdx.x < total_units
-                           ? (total_units - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+  const int share = total_units / (int)gridDim.x, extra = total_units - share * (int)gridDim.x;
+  const int my_units = share + ((int)blockIdx.x < extra ? 1 : 0);
+  const int first_unit = (int)blockIdx.x * share + min((int)blockIdx.x, extra);
   const unsigned lds_base = lds_address(lds);
   const unsigned as_addr = lds_base + 4u * (unsigned)(wp.nbuf * x_words);
 
   auto unit_geometry = [&](int unit) {
     TileGeom g;
-    g.n = unit / units_per_image;
-    g.ox_lo = (unit - g.n * units_per_image) * RB;
+    const int u = unit / pl.batch;
+    g.n = unit - u * pl.batch;
+    g.ox_lo = u * RB;
     const int rows = min(RB, pl.nox_eff - g.ox_lo);
     g.oy_lo = 0;
     g.q0 = g.ox_lo * pl.noy;
@@ -291,11 +298,20 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     g.RSL = pl.ay * (pl.noy - 1) + pl.by_span + 1;
     return g;
   };
+  StageMemo<kRowsMemo> memo = {};
   auto issue_stage = [&](int ui) {
-    const TileGeom tg = unit_geometry(blockIdx.x + ui * gridDim.x);
+    const TileGeom tg = unit_geometry(first_unit + ui);
     const int b = wp.nbuf == 2 ? (ui & 1) : 0;
-    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words), mellin_x,
-                 lane, wave);
+    // units since the rows last changed (or since this workgroup started): the memo is
+    // renewed at 0, and a buffer's zeros are written the first time it holds these rows
+    const int run = min(tg.n, ui);
+    // (a zero the compiler cannot see through, added to the wave index: the staging
+    // addresses are then worked out here and not once for the whole kernel, where
+    // they would sit in registers across the matrix loops)
+    unsigned zero;
+    asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
+    issue_signal<kWaves, kRowsMemo>(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words),
+                                    mellin_x, lane, wave + (int)zero, &memo, run == 0, run < wp.nbuf);
     // grad_out: the unit's rows are one run of `count` words per channel
     const float *An = A + (i64)tg.n * wp.a_n;
     const int count4 = tg.count & ~3;
@@ -321,8 +337,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
 
   const int pairs = pl.noy >> 1;
   auto multiply_unit = [&](int ui) {
-    const int unit = blockIdx.x + ui * gridDim.x;
-    const int ox_lo = (unit % units_per_image) * RB;
+    const int ox_lo = ((first_unit + ui) / pl.batch) * RB;
     for (int row = wave; row < RB && ox_lo + row < pl.nox_eff; row += kWaves) {   // this wavefront's rows
       const int b = wp.nbuf == 2 ? (ui & 1) : 0;
       const float *Xs = Xs0 + b * x_words;
@@ -351,33 +366,30 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
 #pragma unroll
         for (int t = 0; t < JT; ++t) bo[t] += 16;
       }
-      for (; s < pairs; ++s) {
-        float a[MT], b[JT];
+      // the row's last up-to-seven pairs and, if the row is odd, its last position alone:
+      // every step sits at a fixed distance from where the groups of eight stopped, so
+      // the reads take immediate offsets and the steps cost no vector arithmetic
+      const int left = pairs - s + (pl.noy & 1);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a[i] = As[ao + i * 32 * wp.GSS];
+      for (int k = 0; k < 8; ++k) {
+        if (k < left) {
+          float a[MT], b[JT];
 #pragma unroll
-        for (int t = 0; t < JT; ++t) b[t] = Xs[bo[t]];
+          for (int i = 0; i < MT; ++i) a[i] = As[ao + i * 32 * wp.GSS + 2 * k];
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+          for (int t = 0; t < JT; ++t) b[t] = Xs[bo[t] + 2 * k];
+          if (s + k == pairs) {                           // a position alone: the other half-wave multiplies zeros
 #pragma unroll
-          for (int t = 0; t < JT; ++t)
-            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
-        ao += 2;
+            for (int i = 0; i < MT; ++i) a[i] = half ? 0.f : a[i];
 #pragma unroll
-        for (int t = 0; t < JT; ++t) bo[t] += 2;
-      }
-      if (pl.noy & 1) {
-        // the row's last position stands alone: the other half-wave multiplies zeros
-        float a[MT], b[JT];
+            for (int t = 0; t < JT; ++t) b[t] = half ? 0.f : b[t];
+          }
 #pragma unroll
-        for (int i = 0; i < MT; ++i) a[i] = half ? 0.f : As[ao + i * 32 * wp.GSS];
+          for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int t = 0; t < JT; ++t) b[t] = half ? 0.f : Xs[bo[t]];
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int t = 0; t < JT; ++t)
-            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+            for (int t = 0; t < JT; ++t)
+              acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
+        }
       }
     }
   };
