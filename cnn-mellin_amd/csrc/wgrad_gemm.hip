@@ -28,6 +28,7 @@ namespace mellin {
 
 namespace {
 
+constexpr int kGemmMemo = 8;                       // 64-word blocks per wave whose staging sources are kept
 template <int MT, int JT, int NT>
 __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
     WgradPlan wp, const float *__restrict__ A, const float *__restrict__ G,
@@ -74,36 +75,67 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
   }
 
   const FastDiv by_noy(pl.noy);
-  const int my_tiles = (int)blockIdx.x < pl.total_tiles
-                           ? (pl.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+  // Tiles are numbered with the image running fastest and a workgroup takes a
+  // contiguous range of them: consecutive tiles are then the same positions of
+  // successive images, and where a staged word comes from, which words are zeros and
+  // the positions' tap offsets stay what they were for the tile before.
+  const int share = pl.total_tiles / (int)gridDim.x, extra = pl.total_tiles - share * (int)gridDim.x;
+  const int my_tiles = share + ((int)blockIdx.x < extra ? 1 : 0);
+  const int first_tile = (int)blockIdx.x * share + min((int)blockIdx.x, extra);
+  auto tile_of = [&](int ti, int &n) {                    // the tile's number in the (image, tile) order
+    const int i = first_tile + ti, t = i / pl.batch;
+    n = i - t * pl.batch;
+    return n * pl.tiles_per_image + t;
+  };
 
+  StageMemo<kGemmMemo> memo = {};
   auto issue_stage = [&](int ti) {
-    const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
+    int n_img;
+    const TileGeom tg = tile_geometry<P>(pl, tile_of(ti, n_img), mellin_x);
     const int b = ti & 1;
-    issue_signal(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words), mellin_x,
-                 lane, wave);
+    // tiles since the positions last changed (or since this workgroup started): the
+    // memo is renewed at 0, and each of the two buffers gets its zeros and tap
+    // offsets the first time it holds these positions
+    const int run = min(n_img, ti);
+    const bool fresh = run < 2;
+    // (a zero the compiler cannot see through, added to the wave index: the staging
+    // addresses are then worked out here and not once for the whole kernel, where
+    // they would sit in registers across the matrix loops)
+    unsigned zero;
+    asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
+    const int wv = wave + (int)zero;
+    issue_signal<kWaves, kGemmMemo>(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words),
+                                    mellin_x, lane, wv, &memo, run == 0, fresh);
     // grad_out rows: P consecutive positions per output channel, zeros past the tile
-    const float *An = A + (i64)tg.n * wp.a_n + tg.q0;
     float *As = As0 + b * a_words;
-    const int m_live = min(M_T, pl.M - m0);
+    const int m_live = max(0, min(M_T, pl.M - m0));
+    const i64 row_step = (i64)kWaves * wp.a_m;
+    const unsigned dst_step = 4u * (unsigned)(kWaves * wp.GSS);
     for (int pb = 0; pb < P; pb += 64) {
       const int p = pb + lane;
       if (p < tg.count) {
-        for (int m = wave; m < m_live; m += kWaves)
-          load_to_lds_at(An + (i64)(m0 + m) * wp.a_m, (unsigned)p * 4u,
-                         lds_base + 4u * (unsigned)(2 * x_words + b * a_words + m * wp.GSS + pb));
-        for (int m = max(m_live, 0) + wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
-      } else {
-        for (int m = wave; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
+        const float *row = A + (i64)tg.n * wp.a_n + tg.q0 + (i64)(m0 + wv) * wp.a_m;
+        unsigned dst = lds_base + 4u * (unsigned)(2 * x_words + b * a_words + wv * wp.GSS + pb);
+        for (int m = wv; m < m_live; m += kWaves) {
+          load_to_lds_at(row, (unsigned)p * 4u, dst);
+          row += row_step;
+          dst += dst_step;
+        }
+        if (fresh)
+          for (int m = m_live + wv; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
+      } else if (fresh) {
+        for (int m = wv; m < M_T; m += kWaves) As[m * wp.GSS + p] = 0.f;
       }
     }
     // LDS word of every position's (fx = 0, fy = 0) tap
-    int *posoff = posoff0 + b * P;
-    for (int p = tid; p < P; p += kThreads) {
-      const int q = tg.q0 + (p < tg.count ? p : 0);       // past the tile: any valid position
-      int ox, oy;
-      by_noy.divmod(q, ox, oy);
-      posoff[p] = (pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min;
+    if (fresh) {
+      int *posoff = posoff0 + b * P;
+      for (int p = tid; p < P; p += kThreads) {
+        const int q = tg.q0 + (p < tg.count ? p : 0);       // past the tile: any valid position
+        int ox, oy;
+        by_noy.divmod(q, ox, oy);
+        posoff[p] = (pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min;
+      }
     }
   };
 
@@ -122,8 +154,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
     __syncthreads();
     if (ti + 1 < my_tiles) issue_stage(ti + 1);
 
-    const int tile_id = blockIdx.x + ti * gridDim.x;
-    const int n = tile_id / pl.tiles_per_image, tile = tile_id - n * pl.tiles_per_image;
+    const int tile = (first_tile + ti) / pl.batch;
     int count;
     if (pl.segment) count = min(P, pl.noy - (tile % pl.chunks_per_row) * P);
     else count = min(P, pl.Q - tile * P);
