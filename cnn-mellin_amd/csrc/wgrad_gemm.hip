@@ -581,9 +581,21 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
     const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
     const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
     const int rpw_auto = std::max(2, std::min(16, (76 + pl.noy - 1) / pl.noy));
-    const int shapes[4][2] = {{rpw_auto, 1}, {std::max(1, rpw_auto / 2), 2}, {std::max(1, rpw_auto / 2), 1},
-                              {1, 1}};   // {rows per wavefront, buffers}
-    for (const auto &shape : shapes) {
+    // Candidate shapes {rows per wavefront, buffers}: the largest unit with a single
+    // buffer first (several workgroups per CU cover each other's loads), then smaller
+    // units, which need less LDS.  Every workgroup lives for the whole launch, so what counts
+    // is how evenly S * blocks fill the chip: the CU that gets the most workgroups sets
+    // the time, and a CU runs k workgroups at eff[k] of its full rate.
+    int shapes[32][2], n_shapes = 0;
+    for (int r = rpw_auto; r >= 1; --r) {
+      shapes[n_shapes][0] = r; shapes[n_shapes++][1] = 1;
+      shapes[n_shapes][0] = r; shapes[n_shapes++][1] = 2;
+    }
+    static const double eff[7] = {0, 0.45, 0.79, 1.0, 1.0, 1.0, 1.0};   // fitted to measured layers
+    const int vgpr_cap = wp.jt == 3 ? 3 : (wp.jt == 2 ? 4 : 5);   // wavefronts per SIMD the registers allow
+    double best = 0;
+    for (int si = 0; si < n_shapes; ++si) {
+      const int *shape = shapes[si];
       const int rpw = rows_opt_rpw > 0 ? rows_opt_rpw : shape[0];
       const int nbuf = rows_opt_nbuf > 0 ? rows_opt_nbuf : shape[1];
       const int rb = kWaves * rpw;
@@ -600,24 +612,37 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
         bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), (size_t)32 * J_T);
       }
       if (Rr > 8192 || pitch * 32 * 4 >= 65536 || bytes > (mt_rows == 2 ? 150 : 78) * 1024) continue;
-      wp.rows_mode = 1;
-      pl.R = (int)Rr;
-      wp.GSS = pitch;
-      wp.CCj = ccj;
-      wp.lds_bytes = bytes;
-      wp.nbuf = nbuf;
-      wp.rpw = rpw;
-      wp.mt = mt_rows;
-      wp.m_groups = (pl.M + mt_rows * 32 - 1) / (mt_rows * 32);
-      wp.M_pad = wp.m_groups * mt_rows * 32;
-      const int blocks_y_rows = wp.m_groups * wp.j_groups;
+      const int m_groups = (pl.M + mt_rows * 32 - 1) / (mt_rows * 32);
+      const int blocks_y_rows = m_groups * wp.j_groups;
       const i64 units = (i64)pl.batch * ((pl.nox_eff + rb - 1) / rb);
-      int per_cu = std::max(1, std::min((int)((160 * 1024) / (bytes + 512)), nbuf == 2 ? 4 : 6));
-      i64 S = std::max<i64>(1, (256 * per_cu) / blocks_y_rows);
-      wp.S = (int)std::min<i64>(S, units);
-      wp.ws_bytes = (size_t)wp.S * wp.M_pad * wp.J_pad * sizeof(float);
-      return true;
+      const int per_cu = std::max(1, std::min((int)((160 * 1024) / (bytes + 512)), mt_rows == 2 ? 2 : vgpr_cap));
+      // S for every number k of workgroups per CU that fits; rate = work done per unit time
+      for (int k = per_cu; k >= 1; --k) {
+        i64 S = std::min<i64>(std::max<i64>(1, (256 * k) / blocks_y_rows), units);
+        const i64 total = S * blocks_y_rows;
+        const i64 rounds = (total + 256 * per_cu - 1) / (256 * per_cu);      // > 1 only when S == 1 cannot fit at once
+        const int kmax = (int)std::min<i64>(per_cu, (total + 255) / 256);
+        // small units pay their set-up more often; a second buffer hides the loads
+        const double unit = 1.0 + 40.0 / (rpw * pl.noy) + (nbuf == 2 ? -0.07 : 0.0);
+        const double rate = (double)total / rounds * eff[kmax] / kmax / unit;
+        if (rate <= best * 1.01) continue;                // earlier candidates win ties
+        best = rate;
+        wp.rows_mode = 1;
+        pl.R = (int)Rr;
+        wp.GSS = pitch;
+        wp.CCj = ccj;
+        wp.lds_bytes = bytes;
+        wp.nbuf = nbuf;
+        wp.rpw = rpw;
+        wp.mt = mt_rows;
+        wp.m_groups = m_groups;
+        wp.M_pad = wp.m_groups * mt_rows * 32;
+        wp.S = (int)S;
+        wp.ws_bytes = (size_t)wp.S * wp.M_pad * wp.J_pad * sizeof(float);
+      }
+      if (rows_opt_rpw > 0 && rows_opt_nbuf > 0) break;   // a forced shape: nothing else to try
     }
+    if (wp.rows_mode) return true;
   }
   const int P = kWaves * nt * 32;
   wp.GSS = P + 1;
