@@ -388,6 +388,19 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // accumulating into the output: with the old values to fetch as well, that instance
   // runs out of registers and measured 2-3 times slower than one tile per wavefront)
   *nt = (!pr.accumulate && pr.batch * ((Q + 255) / 256) * m_tiles >= 4 * 256) ? 2 : 1;
+  if (*nt == 2) {
+    // Workgroups are persistent and take whole tiles: the launch lasts as long as the
+    // workgroup with the most tiles.  2400 tiles on 768 resident workgroups are four
+    // rounds for 3.1 rounds of work; the same layer cut into 4800 half-size tiles on
+    // 1024 workgroups is five rounds for 4.7.  A half-size tile runs at about 0.9 of the
+    // full one's rate (measured), so the smaller tile wins when it fills its last round
+    // that much better.
+    const i64 big = pr.batch * ((Q + 255) / 256) * m_tiles, small = pr.batch * ((Q + 127) / 128) * m_tiles;
+    const i64 slots_big = 256 * 3, slots_small = 256 * 4;
+    const double fill_big = (double)big / (double)(((big + slots_big - 1) / slots_big) * slots_big);
+    const double fill_small = (double)small / (double)(((small + slots_small - 1) / slots_small) * slots_small);
+    if (0.9 * fill_small > 1.05 * fill_big) *nt = 1;       // only on a clear margin: layers staged in chunks lose more
+  }
   if (force_nt) *nt = force_nt;
   const int P = kWaves * (*nt) * 32;
 
