@@ -147,7 +147,8 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
                    const T *bias, i64 batch, i64 c_in, i64 c_out, i64 nfx,
                    i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy,
                    i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, T *out,
-                   void *stream, int activation = MELLIN_ACT_NONE) {
+                   void *stream, int activation = MELLIN_ACT_NONE, void *half_out = nullptr,
+                   bool *wrote_half = nullptr) {
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
@@ -168,6 +169,22 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
   pr.h_n = c_out * nh; pr.h_m = nh;
   pr.accumulate = 0;
   pr.relu = activation == MELLIN_ACT_RELU;
+  if (wrote_half) *wrote_half = false;
+  if (half_out && sizeof(T) == 4 && g_forced != 1) {
+    // the matrix-core kernel can round its fp32 results to half precision as it stores
+    // them: no fp32 copy of the output, no second pass over it
+    TilePlan pl;
+    size_t lds = 0;
+    int mt = 0, nt = 0;
+    pr.out_half = 1;
+    if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
+      g_variant = "mfma";
+      if (wrote_half) *wrote_half = true;
+      return check_hip(launch_tile_gemm(pl, lds, mt, nt, (const float *)weight, (const float *)input,
+                                        (const float *)bias, (float *)half_out, (hipStream_t)stream), fn);
+    }
+    pr.out_half = 0;
+  }
   return check_hip(run_sepconv<T>(pr, weight, input, bias, out, (hipStream_t)stream), fn);
 }
 
@@ -229,7 +246,8 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
                           i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy,
                           i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux,
                           i64 uy, T *grad_input, void *workspace, size_t workspace_bytes,
-                          void *stream) {
+                          void *stream, void *half_out = nullptr, bool *wrote_half = nullptr) {
+  if (wrote_half) *wrote_half = false;
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
@@ -296,6 +314,20 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   pr.g_n = c_out * nh; pr.g_c = nh;
   pr.h_n = c_in * ng; pr.h_m = ng;
   pr.accumulate = 0;
+  if (half_out && sizeof(T) == 4 && g_forced != 1) {
+    // as in the forward pass: the matrix-core kernel stores half precision itself
+    TilePlan pl;
+    size_t lds = 0;
+    int mt = 0, nt = 0;
+    pr.out_half = 1;
+    if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
+      g_variant = "mfma";
+      if (wrote_half) *wrote_half = true;
+      return check_hip(launch_tile_gemm(pl, lds, mt, nt, (const float *)weight, (const float *)grad_out, nullptr,
+                                        (float *)half_out, (hipStream_t)stream), fn);
+    }
+    pr.out_half = 0;
+  }
   return check_hip(run_sepconv<T>(pr, weight, grad_out, (const T *)nullptr, grad_input,
                                   (hipStream_t)stream), fn);
 }
@@ -437,8 +469,11 @@ int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, doubl
   ux, uy
 
 // ---- half-precision entry points: half tensors, fp32 arithmetic -------------------
-// Each operand is copied to fp32 in the workspace, the fp32 kernels run there, and
-// the result is copied back to half.  Regions are 256-byte aligned.
+// Each operand is copied to fp32 in the workspace and the fp32 kernels run there.  The
+// matrix-core tile kernel (forward, and the input gradient of layers with many input
+// channels) rounds its results to half precision as it stores them; the other kernels
+// write fp32 into the workspace and the result is copied back to half.  Regions are
+// 256-byte aligned.
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
 struct HalfLayout {
@@ -499,10 +534,12 @@ int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight,
   if (e == hipSuccess) e = launch_half_to_float(weight, (float *)(ws + l.w_off), n_w, st);
   if (e == hipSuccess && bias) e = launch_half_to_float(bias, (float *)(ws + l.b_off), c_out, st);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  bool wrote_half = false;
   rc = corr2d_forward<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
                              bias ? (const float *)(ws + l.b_off) : nullptr, CORR2D_ARGS,
-                             (float *)(ws + l.out_off), stream);
+                             (float *)(ws + l.out_off), stream, MELLIN_ACT_NONE, out, &wrote_half);
   if (rc) return rc;
+  if (wrote_half) return MELLIN_OK;
   e = launch_float_to_half((const float *)(ws + l.out_off), out, n_out, st);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
   return MELLIN_OK;
@@ -528,9 +565,12 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
   hipError_t e = launch_half_to_float(weight, (float *)(ws + l.in_off), n_w, st);
   if (e == hipSuccess) e = launch_half_to_float(grad_out, (float *)(ws + l.w_off), n_out, st);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
+  bool wrote_half = false;
   rc = corr2d_backward_input<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
-                                    CORR2D_ARGS, (float *)(ws + l.out_off), ws + l.inner_off, inner, stream);
+                                    CORR2D_ARGS, (float *)(ws + l.out_off), ws + l.inner_off, inner, stream,
+                                    grad_input, &wrote_half);
   if (rc) return rc;
+  if (wrote_half) return MELLIN_OK;
   e = launch_float_to_half((const float *)(ws + l.out_off), grad_input, n_in, st);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", __func__, hipGetErrorString(e));
   return MELLIN_OK;

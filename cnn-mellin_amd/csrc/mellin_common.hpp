@@ -32,6 +32,7 @@ struct SepConv {
   i64 h_n, h_m;                  // output strides; spatial part is dense (nhx, nhy)
   int accumulate;                // 1: h += result (h pre-initialised); 0: h = bias + result
   int relu = 0;                  // with accumulate == 0: h = max(0, bias + result)
+  int out_half = 0;              // with accumulate == 0: h is half-precision storage (matrix-core kernel only)
 };
 
 // Reduction form used by the weight gradient:

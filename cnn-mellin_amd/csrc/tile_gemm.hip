@@ -50,7 +50,9 @@ namespace {
 // MB: 64-word blocks per wave whose staging sources are kept from a tile's first
 // chunk for its other chunks (0: nothing kept; the instance for layers whose
 // channels fit in one or two chunks).
-template <int MT, int NT, bool ACC, int MB>
+// HOUT: H is half-precision storage (not with ACC): the fp32 results are rounded to
+// nearest even as they are stored.
+template <int MT, int NT, bool ACC, int MB, bool HOUT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H) {
@@ -201,14 +203,15 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   // ---- stores: 32 consecutive lanes write 32 consecutive positions of one
   // channel; each lane walks one pointer down the channels in steps of whole
   // channel strides, so the only scalars the stores need are four byte strides.
-  const i64 hm1 = pl.h_m * 4, hm2 = 2 * hm1, hm3 = 3 * hm1, hm8 = 8 * hm1;
+  constexpr int ES = HOUT ? 2 : 4;                      // bytes per stored element
+  const i64 hm1 = pl.h_m * ES, hm2 = 2 * hm1, hm3 = 3 * hm1, hm8 = 8 * hm1;
   const bool full_m = m0 + M_T <= pl.M;
   const int m_left = pl.M - m0 - half * 4;              // channels from this lane's first row on
   // They run one stage late, after the next stage's loads are issued and before
   // its multiplies, so that they drain behind the next matrix loop.
   auto write_tile = [&](auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
-    char *Himg = (char *)(H + (i64)tg.n * pl.h_n + (i64)m0 * pl.h_m);
+    char *Himg = (char *)H + ((i64)tg.n * pl.h_n + (i64)m0 * pl.h_m) * ES;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int local = (wave * NT + t) * 32 + l32;
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
         live = live && ox < pl.nox_eff && oy < pl.noy_eff;
       }
       if (!live) continue;
-      char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * 4;
+      char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * ES;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
         float old[16];
@@ -241,7 +244,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
         for (int g4 = 0; g4 < 4; ++g4) {
           const int mo = i * 32 + g4 * 8;
           auto put = [&](char *at, int row, int r) {
-            if (FULL || row < m_left) *(float *)at = ACC ? old[r] + acc[i][t][r] : acc[i][t][r];
+            if (FULL || row < m_left) {
+              if (HOUT) *(_Float16 *)at = (_Float16)acc[i][t][r];
+              else *(float *)at = ACC ? old[r] + acc[i][t][r] : acc[i][t][r];
+            }
           };
           put(o, mo, 4 * g4);
           put(o + hm1, mo + 1, 4 * g4 + 1);
@@ -328,10 +334,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
 #undef pl
 }
 
-template <int MT, int NT, bool ACC, int MB>
+template <int MT, int NT, bool ACC, int MB, bool HOUT = false>
 hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const float *f,
                           const float *g, const float *bias, float *h, hipStream_t stream) {
-  auto kern = tile_gemm_kernel<MT, NT, ACC, MB>;
+  auto kern = tile_gemm_kernel<MT, NT, ACC, MB, HOUT>;
   if (lds_bytes > 64 * 1024) {
     // opt in to more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per CU)
     static thread_local size_t granted = 0;
@@ -376,6 +382,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.f_m = pr.f_m; pl.f_c = pr.f_c; pl.g_n = pr.g_n; pl.g_c = pr.g_c; pl.h_n = pr.h_n; pl.h_m = pr.h_m;
   pl.accumulate = pr.accumulate;
   pl.relu = pr.relu && !pr.accumulate;
+  pl.out_half = pr.out_half && !pr.accumulate;
   pl.kind_x = X.kind; pl.sx = (int)X.s; pl.dx = (int)X.d; pl.px = (int)X.p; pl.ux = (int)X.u;
   pl.uy = (int)Y.u;
 
@@ -523,6 +530,9 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
     if (pl.accumulate)                                                                       \
       return memo ? launch_variant<MT_, NT_, true, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)  \
                   : launch_variant<MT_, NT_, true, 0>(pl, lds_bytes, grid, f, g, bias, h, stream); \
+    if (pl.out_half)                                                                         \
+      return memo ? launch_variant<MT_, NT_, false, 8, true>(pl, lds_bytes, grid, f, g, bias, h, stream)  \
+                  : launch_variant<MT_, NT_, false, 0, true>(pl, lds_bytes, grid, f, g, bias, h, stream); \
     return memo ? launch_variant<MT_, NT_, false, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)   \
                 : launch_variant<MT_, NT_, false, 0>(pl, lds_bytes, grid, f, g, bias, h, stream);  \
   }

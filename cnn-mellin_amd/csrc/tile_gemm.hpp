@@ -15,6 +15,7 @@ struct TilePlan {
   i64 f_m, f_c, g_n, g_c, h_n, h_m;
   int accumulate;
   int relu;                        // clamp the result at zero before it is stored (accumulate == 0)
+  int out_half;                    // results are rounded to half precision as they are stored (accumulate == 0)
   // x axis: Mellin kinds evaluate taps per (row, filter row); linear kinds use
   // the coordinate ax * ox + bx * fx + cx (divided by ux)
   int kind_x, sx, dx, px, ux;

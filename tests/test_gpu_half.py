@@ -143,3 +143,31 @@ def test_autocast_column_ops():
         cols = mconv.spec2col(x, (4, 3))
     assert cols.dtype == torch.half
     assert torch.equal(cols.float(), full)               # a gather moves values unchanged
+
+
+@pytest.mark.parametrize("shape", [
+    # (kind, n, c_in, c_out, nf, ng): few channels (forward stores half itself), many (so does the input gradient)
+    ("lcorr", 3, 3, 40, (8, 4), (70, 41)), ("mcorr", 2, 3, 64, (8, 4), (64, 41)),
+    ("lcorr", 2, 48, 70, (3, 3), (30, 21)), ("mcorr", 2, 40, 33, (4, 4), (40, 5)),
+], ids=["lcorr-few", "mcorr-few", "lcorr-many", "mcorr-many"])
+def test_half_results_are_the_fp32_results_rounded_once(shape):
+    """The half entry points compute in fp32 on the widened operands: whichever kernel
+    stores the result, it must equal the fp32 result rounded to nearest even, bit for bit."""
+    kind, n, c_in, c_out, nf, ng = shape
+    kind_x = hip.AX_MCORR if kind == "mcorr" else hip.AX_LCORR
+    op = mconv.mcorrlcorr if kind == "mcorr" else mconv.lcorrlcorr
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn((n, c_in) + ng, generator=gen).half().cuda()
+    w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_in * nf[0] * nf[1]) ** -0.5).half().cuda()
+    b = torch.randn(c_out, generator=gen).half().cuda()
+    ref = op(x.float(), w.float(), b.float())
+    out = op(x, w, b)
+    assert out.dtype == torch.float16 and torch.equal(out, ref.half())
+    nh = tuple(ref.shape[2:])
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), (0, 0), (1, 1))
+    go = torch.randn(ref.shape, generator=gen).half().cuda()
+    gi32 = torch.empty_like(x, dtype=torch.float32)
+    hip.corr2d_backward_input(kind_x, w.float(), go.float(), gi32, dims)
+    gi16 = torch.empty_like(x)
+    hip.corr2d_backward_input(kind_x, w, go, gi16, dims)
+    assert torch.equal(gi16, gi32.half())
