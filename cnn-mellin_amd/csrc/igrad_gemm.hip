@@ -250,7 +250,6 @@ __global__ __launch_bounds__((KSTEPS * NT <= 128 ? 768 : 512)) void igrad_kernel
       }
       wait_all_memory();
       __syncthreads();               // tile p has landed for every wavefront; the block of tile p - 1 is free
-      if (p >= 1 && p + 2 < ntiles) issue_tile(p + 2);
       const float *blk = Bs + (p % NBUF) * K * 32 + bsrc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) cur[r] = 0.f;
@@ -264,6 +263,11 @@ __global__ __launch_bounds__((KSTEPS * NT <= 128 ? 768 : 512)) void igrad_kernel
 #pragma unroll
         for (int s = c4 * SPB; s < (c4 + 1) * SPB; ++s)
           cur = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], blk[64 * s], cur, 0, 0, 0);
+        // the refill of tile p - 1's block is requested here, behind the first batch of
+        // multiplies: its address arithmetic then runs while the matrix pipe is busy
+        // instead of right after the barrier, when every wavefront of the CU would do it
+        // at once with the pipe idle
+        if (c4 == 0 && p >= 1 && p + 2 < ntiles) issue_tile(p + 2);
         if (kPrev) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) plane[dprev + off[4 * j + c4]] = v[j] + prev[4 * j + c4];
