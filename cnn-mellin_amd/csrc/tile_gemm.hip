@@ -22,11 +22,14 @@
 //     a half-wave fall in 32 different banks.
 //
 // Staging uses the direct global->LDS loads of gfx950 (no VGPR round trip):
-// a wavefront issues one load per virtual row, 64 columns wide, and writes
-// zeros for the columns or rows that have no source.  The loads of stage i+1
-// are issued before the matrix-core loop of stage i (two LDS buffers), so a
-// persistent workgroup needs one barrier per stage and global latency hides
-// behind the multiplies.  A stage is one (tile, channel chunk) pair.
+// a wavefront issues one load per virtual row, 64 columns wide (64 consecutive
+// LDS words of any rows when rows are a few words long; 16 bytes per lane when
+// the virtual rows are the signal's own), and writes zeros for the columns or
+// rows that have no source.  The loads of stage i+1 are issued before the
+// matrix-core loop of stage i (two LDS buffers), so a persistent workgroup
+// needs one barrier per stage and global latency hides behind the multiplies.
+// A stage is one (tile, channel chunk) pair; where a tile's words come from and
+// which are zeros is worked out for its first chunk and kept for the others.
 //
 // One wavefront owns all M_T output channels of NT * 32 positions and keeps
 // MT * NT accumulator tiles (16 registers each).  Stores write 128-byte runs

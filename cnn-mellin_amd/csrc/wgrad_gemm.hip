@@ -5,10 +5,12 @@
 //
 // (A = grad_out, G = layer input) is a (M x positions) * (positions x J)
 // product, J = c_in * nfx * nfy, whose long dimension is the reduction.  The
-// reduction is split over persistent workgroups in a FIXED way: workgroup s
-// takes position tiles s, s + S, ... of the same (image, position) tiling the
-// forward kernel uses, each wavefront a quarter of every tile, and keeps its
-// MT x JT accumulator tiles in registers for its whole life.  At the end the
+// reduction is split over S persistent workgroups in a FIXED way: the position
+// tiles of the forward kernel's tiling are numbered with the image running
+// fastest and workgroup s takes the s-th contiguous range of them (the same
+// positions of successive images come one after the other, so what the staging
+// works out for one serves the next), each wavefront a quarter of every tile;
+// a workgroup keeps its MT x JT accumulator tiles in registers for its whole life.  At the end the
 // four wavefronts are summed through LDS in wave order, the workgroup writes
 // one partial block to the workspace, and a second kernel adds the S partials
 // in index order.  No floating-point atomics: the result is bit-reproducible.
@@ -242,8 +244,8 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
 }
 
 // Row-wise variant for layers whose outputs are walked a whole row at a time
-// (unit y stride, rows of at least 16 outputs that fit one tile).  A unit of work
-// is four consecutive output rows of one image, one row per wavefront.  Within
+// (unit y stride, rows of at least four outputs that fit one tile).  A unit of work
+// is 4 * rpw consecutive output rows of one image, rpw rows per wavefront.  Within
 // a row every operand address is affine in the column: position oy of output
 // row ox reads grad_out word  row_base + oy  and, for column j = (c, fx, fy),
 // input word  col_offset[j] + virtual_row(ox) * RS + oy - by_min,  so the loop
