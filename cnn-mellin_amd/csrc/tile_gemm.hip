@@ -389,9 +389,10 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.kind_x = X.kind; pl.sx = (int)X.s; pl.dx = (int)X.d; pl.px = (int)X.p; pl.ux = (int)X.u;
   pl.uy = (int)Y.u;
 
-  // 64 output channels per workgroup, unless the launch would then leave most CUs
-  // without a workgroup: 32 channels double the workgroups of a small problem
-  *mt = (pr.c_out > 32 && pr.batch * ((Q + 127) / 128) * ((pr.c_out + 63) / 64) >= 192) ? 2 : 1;
+  // 64 output channels per workgroup, unless the launch would then have fewer than two
+  // workgroups per CU: 32 channels double the workgroups of a small problem (1-D layers
+  // of 780 frames: input gradient 75 -> 61 us, forward up to 25 % faster)
+  *mt = (pr.c_out > 32 && pr.batch * ((Q + 127) / 128) * ((pr.c_out + 63) / 64) >= 512) ? 2 : 1;
   const int M_T = *mt * 32;
   const i64 m_tiles = (pr.c_out + M_T - 1) / M_T;
   // two N tiles per wavefront once that still leaves every CU several tiles (not when
