@@ -575,12 +575,15 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
   // the forward plan fixed the position tiling (nt) and the row geometry
   wp.nt = nt;
   wp.rows_mode = 0;
-  if (!pl.segment && pl.ay == 1 && pl.noy >= 4 && pl.nox_eff >= 1 && g_allow_rows) {
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+  // Rows of under eight outputs are three or four matrix steps long: on a linear x axis
+  // the position-tile kernel, which does not care where rows end, is then the faster one
+  // (rows of 5 and 7: 12 % and 25 %).  On a Mellin axis its tiles stage a virtual row per
+  // (row, filter row) pair for only 128 positions and the row-wise kernel stays ahead.
+  const int min_row = mellin_x ? 4 : 8;
+  if (!pl.segment && pl.ay == 1 && pl.noy >= min_row && pl.nox_eff >= 1 && g_allow_rows) {
     // Row-wise variant: units of kWaves * rpw output rows, about 300 positions per
-    // unit (two rows of 38 per wavefront, sixteen rows of 5).  Preferred shape: a
-    // single buffer (several workgroups per CU cover each other's loads); then half
-    // the rows with two buffers, then with one.
-    const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+    // unit (two rows of 38 per wavefront, sixteen rows of 5).
     const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
     const int rpw_auto = std::max(2, std::min(16, (76 + pl.noy - 1) / pl.noy));
     // Candidate shapes {rows per wavefront, buffers}: the largest unit with a single
@@ -653,10 +656,10 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
   const size_t red_words = (size_t)M_T * J_T;
   wp.lds_bytes = 4 * std::max(words, red_words);
   if (wp.lds_bytes > 96 * 1024) return false;
-  // position shares: persistent workgroups, at most two per CU over all output blocks
+  // position shares: persistent workgroups, at most three per CU (registers) over all output blocks
   const int blocks_y = wp.m_groups * wp.j_groups;
   int per_cu = (int)((160 * 1024) / (wp.lds_bytes + 512));
-  per_cu = std::max(1, std::min(per_cu, 2));
+  per_cu = std::max(1, std::min(per_cu, 3));
   int S = std::max(1, (256 * per_cu) / blocks_y);
   S = std::min(S, pl.total_tiles);
   wp.S = S;
