@@ -185,8 +185,8 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
     const int count = tg.R_tile * pl.ngy, count4 = count & ~3;
     const int pieces = (count4 + 255) >> 8;
     const float *src0 = Gimg + tg.vx_min * pl.ngy;
-    for (int cl = 0, pc = wave; ; pc += NW) {              // piece pc of channel cl; pieces go round the waves
-      while (pc >= pieces) { pc -= pieces; ++cl; }
+    for (int cl = 0, pc = wave; pieces > 0; pc += NW) {    // piece pc of channel cl; pieces go round the waves
+      while (pc >= pieces) { pc -= pieces; ++cl; }         // (no pieces at all: a run of under four words)
       if (cl >= cc) break;
       const int w0 = pc << 8, idx = w0 + 4 * lane;
       if (idx < count4)

@@ -91,3 +91,37 @@ def test_chunked_layer_is_run_to_run_deterministic():
     again = _run(kind_x, x, w, b, go, s, d, p, u)[:3]
     for a, c in zip(first, again):
         assert torch.equal(a, c)
+
+
+# When a tile's staged rows are the signal's own rows the kernels copy them as one run per
+# channel, 16 bytes per lane; a run of under four words has no 16-byte piece at all and is
+# moved by the tail alone.  Such runs come from last tiles that hold a single short row.
+SHORT_RUN_CASES = [
+    # (op, n, c_in, c_out, nf, ng, s, d, p, u, r)
+    # input gradient in two passes (wide Mellin layer): the first pass's last tile is one row of two words
+    ("mcorrlcorr", 3, 150, 33, (5, 1), (9, 1), (1, 1), (2, 2), (0, 0), (1, 1), (0, 1)),
+    # pointwise 1-D layer, 257 = 2 * 128 + 1 positions: the last tile is one word
+    ("lcorrlcorr", 2, 8, 32, (1, 1), (257, 1), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),
+    # rows of three words, a tile boundary that leaves one row to the last tile
+    ("lcorrlcorr", 2, 20, 40, (1, 1), (43, 3), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),
+    ("lcorrlcorr", 1, 3, 5, (1, 1), (3, 1), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),
+]
+
+
+@pytest.mark.parametrize("case", SHORT_RUN_CASES, ids=[str(i) for i in range(len(SHORT_RUN_CASES))])
+def test_block_copies_of_under_four_words(case):
+    op, n, c_in, c_out, nf, ng, s, d, p, u, r = case
+    kind_x, fwd, bwd = OPS[op]
+    rng = np.random.default_rng(3000 + SHORT_RUN_CASES.index(case))
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float32)
+    w = (rng.standard_normal((c_out, c_in) + nf) * (c_in * nf[0] * nf[1]) ** -0.5).astype(np.float32)
+    b = rng.standard_normal(c_out).astype(np.float32)
+    exp = fwd(x, w, b, s, d, p, u, r)
+    nh = exp.shape[2:]
+    assert min(nh) > 0
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    egi, egw, _ = bwd(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64), s, d, p, u)
+    out, gi, gw, _ = _run(kind_x, x, w, b, go, s, d, p, u)
+    assert_close(out, exp, c_in * nf[0] * nf[1], "out %s" % (case,))
+    assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
+    assert_close(gw, egw, n * nh[0] * nh[1], "grad_weight %s" % (case,))
