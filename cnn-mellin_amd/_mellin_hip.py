@@ -47,6 +47,7 @@ SYMBOLS = {
 for _n in ("forward", "backward_input", "backward_weight"):
     SYMBOLS["mellin_corr2d_%s_f16_workspace" % _n] = (_size_t, [_int] + _DIMS)
 SYMBOLS["mellin_corr2d_forward_f16"] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
+SYMBOLS["mellin_corr2d_forward_act_f16"] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_corr2d_backward_input_f16"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_corr2d_backward_weight_f16"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 _dbl = ctypes.c_double
@@ -199,12 +200,10 @@ def corr2d_forward(kind_x, input, weight, bias, out, dims, activation=ACT_NONE):
     _same_dtype(input, weight, bias, out)
     with torch.cuda.device(dev):
         if out.dtype == torch.float16:
-            if activation != ACT_NONE:
-                raise RuntimeError("the fused activation is available in float32 and float64")
             need = lib.mellin_corr2d_forward_f16_workspace(kind_x, *dims)
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
-            _check(lib.mellin_corr2d_forward_f16(kind_x, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out),
-                                                 _ptr(ws.data_ptr()), need, _stream(dev)))
+            _check(lib.mellin_corr2d_forward_act_f16(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims,
+                                                     _dp(out), _ptr(ws.data_ptr()), need, _stream(dev)))
         else:
             fn = getattr(lib, "mellin_corr2d_forward_act_" + suffix(out.dtype))
             _check(fn(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))

@@ -520,8 +520,17 @@ size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
 int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight, const void *bias,
                               MELLIN_CORR2D_DIMS, void *out, void *workspace, size_t workspace_bytes,
                               void *stream) {
+  return mellin_corr2d_forward_act_f16(kind_x, MELLIN_ACT_NONE, input, weight, bias, CORR2D_ARGS, out, workspace,
+                                       workspace_bytes, stream);
+}
+int mellin_corr2d_forward_act_f16(int kind_x, int activation, const void *input, const void *weight,
+                                  const void *bias, MELLIN_CORR2D_DIMS, void *out, void *workspace,
+                                  size_t workspace_bytes, void *stream) {
   int rc;
   if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
+  if (activation != MELLIN_ACT_NONE && activation != MELLIN_ACT_RELU)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: activation must be MELLIN_ACT_NONE or MELLIN_ACT_RELU (got %d)", __func__,
+                activation);
   CORR2D_COUNTS;
   if (n_out == 0) return MELLIN_OK;
   const HalfLayout l = half_layout(n_in, n_w, c_out, n_out, 0);
@@ -537,7 +546,7 @@ int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight,
   bool wrote_half = false;
   rc = corr2d_forward<float>(__func__, kind_x, (const float *)(ws + l.in_off), (const float *)(ws + l.w_off),
                              bias ? (const float *)(ws + l.b_off) : nullptr, CORR2D_ARGS,
-                             (float *)(ws + l.out_off), stream, MELLIN_ACT_NONE, out, &wrote_half);
+                             (float *)(ws + l.out_off), stream, activation, out, &wrote_half);
   if (rc) return rc;
   if (wrote_half) return MELLIN_OK;
   e = launch_float_to_half((const float *)(ws + l.out_off), out, n_out, st);

@@ -208,7 +208,7 @@ class _Corr2dFunction(torch.autograd.Function):
         if activation not in (None, "relu"):
             raise RuntimeError('activation must be None or "relu", got %r (while checking arguments for %s)'
                                % (activation, name))
-        fused = activation == "relu" and input.dtype != torch.float16
+        fused = activation == "relu"
         nf, ng = tuple(weight.shape[2:]), tuple(input.shape[2:])
         nh = (_VALID_SIZE[kind_x](nf[0], ng[0], s[0], d[0], p[0], u[0]) + r[0],
               lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], u[1]) + r[1])
@@ -218,8 +218,6 @@ class _Corr2dFunction(torch.autograd.Function):
         dims = _hip._dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u)
         _hip.corr2d_forward(kind_x, input_c, weight_c, bias_c, out, dims,
                             _hip.ACT_RELU if fused else _hip.ACT_NONE)
-        if activation == "relu" and not fused:             # half: the library has no fused form
-            out = out.clamp_(min=0)
         ctx.save_for_backward(input_c, weight_c, *([out] if activation == "relu" else []))
         ctx.has_bias = bias is not None
         ctx.kind_x, ctx.dims = kind_x, dims

@@ -187,6 +187,12 @@ int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight,
                               const void *bias, MELLIN_CORR2D_DIMS, void *out,
                               void *workspace, size_t workspace_bytes,
                               void *stream);
+/* The same with the fused activation of mellin_corr2d_forward_act_f32 (applied to the
+ * fp32 result, before the rounding); same workspace. */
+int mellin_corr2d_forward_act_f16(int kind_x, int activation, const void *input,
+                                  const void *weight, const void *bias,
+                                  MELLIN_CORR2D_DIMS, void *out, void *workspace,
+                                  size_t workspace_bytes, void *stream);
 size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS);
 int mellin_corr2d_backward_input_f16(int kind_x, const void *weight,
                                      const void *grad_out, MELLIN_CORR2D_DIMS,

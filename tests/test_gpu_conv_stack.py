@@ -151,7 +151,7 @@ RELU_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16], ids=["f32", "f64", "f16"])
 @pytest.mark.parametrize("case", RELU_CASES, ids=[c[0] + str(i) for i, c in enumerate(RELU_CASES)])
 def test_fused_relu_equals_relu_of_the_plain_op(case, dtype):
     name, xs, ws, kw = case
