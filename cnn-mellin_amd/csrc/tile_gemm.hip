@@ -289,7 +289,11 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
     MELLIN_STAMP(3);
     if (st + 1 < my_stages) {
       MELLIN_STAMP(7);
+      // (at raised priority: a staging wavefront otherwise gets an issue slot only now and
+      // then between the matrix instructions of its SIMD's other wavefronts)
+      __builtin_amdgcn_s_setprio(3);
       issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
+      __builtin_amdgcn_s_setprio(0);
       MELLIN_STAMP(8);
     }
     MELLIN_STAMP(4);

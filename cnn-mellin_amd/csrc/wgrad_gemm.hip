@@ -154,7 +154,11 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_gemm_kernel(
   for (int ti = 0; ti < my_tiles; ++ti) {
     wait_all_memory();
     __syncthreads();
-    if (ti + 1 < my_tiles) issue_stage(ti + 1);
+    if (ti + 1 < my_tiles) {
+      __builtin_amdgcn_s_setprio(3);                     // staging ahead of the other wavefronts' multiplies
+      issue_stage(ti + 1);
+      __builtin_amdgcn_s_setprio(0);
+    }
 
     const int tile = (first_tile + ti) / pl.batch;
     int count;
@@ -433,13 +437,19 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     for (int ui = 0; ui < my_units; ++ui) {
       wait_all_memory();
       __syncthreads();
-      if (ui + 1 < my_units) issue_stage(ui + 1);
+      if (ui + 1 < my_units) {
+        __builtin_amdgcn_s_setprio(3);
+        issue_stage(ui + 1);
+        __builtin_amdgcn_s_setprio(0);
+      }
       multiply_unit(ui);
     }
   } else {
     // one buffer and more workgroups per CU: they cover each other's loads
     for (int ui = 0; ui < my_units; ++ui) {
+      __builtin_amdgcn_s_setprio(3);                   // staging ahead of the other workgroups' multiplies
       issue_stage(ui);
+      __builtin_amdgcn_s_setprio(0);
       wait_all_memory();
       __syncthreads();
       multiply_unit(ui);
