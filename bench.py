@@ -38,7 +38,7 @@ FP32_PEAK_TFLOPS = 157.3     # MI355X fp32 matrix (MFMA) = packed vector fp32, p
 # WRITE_SIZE x 1.0.  The summary is kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {
     "mconv2d.forward": 35.3e6, "mconv2d.grad_input": 104.9e6, "mconv2d.grad_weight": 47.8e6,
-    "lconv2d.forward": 196.4e6, "lconv2d.grad_input": 189.9e6, "lconv2d.grad_weight": 217.5e6,
+    "lconv2d.forward": 195.5e6, "lconv2d.grad_input": 190.1e6, "lconv2d.grad_weight": 214.3e6,
 }
 MEASURED_TRAFFIC_VARIANTS = {
     "mconv2d.forward": "mfma", "mconv2d.grad_input": "mfma-taps+fold", "mconv2d.grad_weight": "mfma-rows",
