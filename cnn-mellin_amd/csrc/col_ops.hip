@@ -105,19 +105,29 @@ __global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict
 }
 
 // g[nc', q] = sum over taps of gg[nc, tap, source of q] for q in the (x.nh, y.nh) signal plane;
-// eight (image, channel) pairs per thread share the tap arithmetic
+// eight (image, channel) pairs per thread share the tap arithmetic.  The y taps are worked out
+// once per thread; for a filter row with a tap, the loads of four filter columns of all eight
+// pairs are requested before the first is summed (positions without a tap read a word that is
+// there and add zero), so a thread waits for memory once per filter row, not once per tap.
 template <typename T>
 __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict__ gg, T *__restrict__ g,
                                                              Axis x, Axis y, int c_in, int batch,
                                                              int transposed_g, int transposed_gg,
                                                              i64 per_pair) {   // words from one pair's columns to the next
-  constexpr int NB = 8;
+  constexpr int NB = 8, FY = 4;
   const int plane = (int)(x.nh * y.nh), nfx = (int)x.nf, nfy = (int)y.nf;
   const int q = blockIdx.x * 256 + threadIdx.x;
   if (q >= plane) return;
   int gx = (int)((float)q * (1.0f / (float)y.nh));
   int gy = q - gx * (int)y.nh;
   if (gy < 0) { --gx; gy += (int)y.nh; } else if (gy >= (int)y.nh) { ++gx; gy -= (int)y.nh; }
+  auto y_taps = [&](int fy0, int (&oy)[FY]) {
+#pragma unroll
+    for (int j = 0; j < FY; ++j)
+      oy[j] = fy0 + j < nfy ? tap32(y.kind, gy, fy0 + j, (int)y.ng, (int)y.s, (int)y.d, (int)y.p, (int)y.u) : -1;
+  };
+  int oy_first[FY];
+  y_taps(0, oy_first);
   const int pairs = batch * c_in;
   for (int nc0 = blockIdx.z * NB; nc0 < pairs; nc0 += gridDim.z * NB) {   // nc: pairs in g's own order
     const T *src[NB];
@@ -137,12 +147,26 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
     for (int fx = 0; fx < nfx; ++fx) {
       const int ox = tap32(x.kind, gx, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u);
       if (ox < 0) continue;
-      for (int fy = 0; fy < nfy; ++fy) {
-        const int oy = tap32(y.kind, gy, fy, (int)y.ng, (int)y.s, (int)y.d, (int)y.p, (int)y.u);
-        if (oy < 0) continue;
-        const int off = ((fx * nfy + fy) * (int)x.ng + ox) * (int)y.ng + oy;
+      for (int fy0 = 0; fy0 < nfy; fy0 += FY) {
+        int oy[FY];
+        if (fy0 == 0) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b) acc[b] += src[b][off];
+          for (int j = 0; j < FY; ++j) oy[j] = oy_first[j];
+        } else {
+          y_taps(fy0, oy);
+        }
+        T v[FY][NB];
+#pragma unroll
+        for (int j = 0; j < FY; ++j) {
+          const int fy = min(fy0 + j, nfy - 1);
+          const int off = ((fx * nfy + fy) * (int)x.ng + ox) * (int)y.ng + max(oy[j], 0);
+#pragma unroll
+          for (int b = 0; b < NB; ++b) v[j][b] = src[b][off];
+        }
+#pragma unroll
+        for (int j = 0; j < FY; ++j)
+#pragma unroll
+          for (int b = 0; b < NB; ++b) acc[b] += oy[j] >= 0 ? v[j][b] : T(0);
       }
     }
 #pragma unroll
