@@ -116,7 +116,14 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
                                                              i64 per_pair) {   // words from one pair's columns to the next
   constexpr int NB = 8, FY = 4;
   const int plane = (int)(x.nh * y.nh), nfx = (int)x.nf, nfy = (int)y.nf;
-  const int q = blockIdx.x * 256 + threadIdx.x;
+  // Workgroups are dealt to the eight dies in turn, each with an L2 of its own: renumber them so
+  // that a die takes one contiguous run of (pair group, 256-position block), whose neighbouring
+  // rows of gg share cache lines.
+  const unsigned total = gridDim.x * gridDim.z, lin = blockIdx.x + gridDim.x * blockIdx.z;
+  const unsigned die = lin & 7u, slot = lin >> 3;
+  const unsigned mine = die * (total >> 3) + min(die, total & 7u) + slot;
+  const unsigned block_z = mine / gridDim.x, block_x = mine - block_z * gridDim.x;
+  const int q = (int)block_x * 256 + threadIdx.x;
   if (q >= plane) return;
   int gx = (int)((float)q * (1.0f / (float)y.nh));
   int gy = q - gx * (int)y.nh;
@@ -129,7 +136,7 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
   int oy_first[FY];
   y_taps(0, oy_first);
   const int pairs = batch * c_in;
-  for (int nc0 = blockIdx.z * NB; nc0 < pairs; nc0 += gridDim.z * NB) {   // nc: pairs in g's own order
+  for (int nc0 = (int)block_z * NB; nc0 < pairs; nc0 += gridDim.z * NB) {   // nc: pairs in g's own order
     const T *src[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {

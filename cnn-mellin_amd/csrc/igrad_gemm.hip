@@ -590,14 +590,14 @@ bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64
   pl.ksteps = c_out <= 32 ? 16 : c_out <= 64 ? 32 : 64;
   const int max_waves = pl.ksteps == 64 ? 8 : 12;
   if (units > max_waves) return false;
+  // One image per workgroup: workgroups of a few wavefronts, several to a CU, spread over the
+  // chip more evenly than one large workgroup per CU and do not all wait for memory at once.
   pl.jobs = 1;
-  for (int j = 1; j <= 4; ++j)
-    if ((j * units) % 4 == 0 && j * units <= max_waves && j <= batch) { pl.jobs = j; break; }
   pl.chunks_per_image = (int)((nh + 63) / 64);
-  // chunks per workgroup: about two workgroups per CU in all, at least two chunks each
-  const i64 image_groups = (batch + pl.jobs - 1) / pl.jobs;
-  i64 cpw = (image_groups * pl.chunks_per_image + 511) / 512;
-  pl.cpw = (int)std::max<i64>(2, std::min<i64>(cpw, pl.chunks_per_image));
+  // chunks per workgroup: one, unless that makes more workgroups than the chip holds at once
+  const i64 image_groups = batch;
+  i64 cpw = (image_groups * pl.chunks_per_image + 2047) / 2048;
+  pl.cpw = (int)std::max<i64>(1, std::min<i64>(cpw, pl.chunks_per_image));
   pl.lds_bytes = 4 * (size_t)(2 * pl.ksteps * 64) * pl.jobs;
   pl.ws_bytes = 4 * (size_t)batch * c_in * pl.nf_pad * nh;
   if (image_groups * ((pl.chunks_per_image + pl.cpw - 1) / pl.cpw) >= ((i64)1 << 31)) return false;
