@@ -37,8 +37,8 @@ FP32_PEAK_TFLOPS = 157.3     # MI355X fp32 matrix (MFMA) = packed vector fp32, p
 # counters read for a plain 256 MiB device copy (--copy-calibration): FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0.  The summary is kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "mconv2d.forward": 35.3e6, "mconv2d.grad_input": 104.9e6, "mconv2d.grad_weight": 47.8e6,
-    "lconv2d.forward": 195.5e6, "lconv2d.grad_input": 190.1e6, "lconv2d.grad_weight": 214.3e6,
+    "mconv2d.forward": 35.3e6, "mconv2d.grad_input": 88.3e6, "mconv2d.grad_weight": 47.8e6,
+    "lconv2d.forward": 195.6e6, "lconv2d.grad_input": 190.1e6, "lconv2d.grad_weight": 214.3e6,
 }
 MEASURED_TRAFFIC_VARIANTS = {
     "mconv2d.forward": "mfma", "mconv2d.grad_input": "mfma-taps+fold", "mconv2d.grad_weight": "mfma-rows",
