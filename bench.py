@@ -175,8 +175,10 @@ def cpu_baseline(layers, slice_n, reps=25):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    # a step is a third of a millisecond and the first few milliseconds after an idle spell run
+    # 5-8 % slow (measured: 5 warm-up steps 0.358 ms/step, 50 or more 0.335), hence the defaults
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--variant", default=None, help="force a kernel variant (e.g. generic)")
     ap.add_argument("--cpu-slice", type=int, default=32, help="utterances in the CPU baseline sample")
