@@ -142,3 +142,29 @@ def test_transposed_input_is_used_where_it_lies():
     got = mconv.spec2col(x, (3, 2), 1, 1, 1, 0)
     exp = oracle.spec2col(np.ascontiguousarray(np.swapaxes(base, 0, 1)), (3, 2), 1, 1, 1, 1, 0)
     np.testing.assert_array_equal(to_np(got), exp)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_adjoint_with_more_than_four_filter_columns(dtype):
+    """The plane adjoint requests a filter row's loads four filter columns at a time: filters
+    5-9 columns wide take two or three such blocks per row, the last one part-filled, on
+    both kinds of x axis (spec: Mellin x linear; a unit x axis leaves the linear y alone)."""
+    rng = np.random.default_rng(23)
+    for trial, (nf, ng, s, d, p, r) in enumerate([
+            ((3, 5), (40, 23), (1, 1), (1, 1), (0, 0), (0, 0)),
+            ((2, 7), (31, 30), (1, 2), (1, 1), (1, 3), (0, 1)),
+            ((4, 9), (25, 41), (1, 1), (2, 2), (1, 2), (2, 0)),
+            ((1, 6), (1, 64), (1, 1), (1, 1), (0, 2), (0, 0)),
+            ((8, 8), (64, 20), (1, 1), (1, 1), (0, 0), (0, 0))]):
+        x = rng.standard_normal((9, 3) + ng).astype(dtype)               # 27 pairs: three groups of eight + three
+        exp = oracle.spec2col(x, nf, s, d, p, 1, r)
+        assert exp.size > 0
+        xt = to_gpu(x).requires_grad_(True)
+        got = mconv.spec2col(xt, nf, s, d, p, r)
+        np.testing.assert_array_equal(to_np(got), exp, err_msg="spec2col trial %d" % trial)
+        go = rng.standard_normal(exp.shape).astype(dtype)
+        got.backward(to_gpu(go))
+        gexp = oracle.col2spec(go, ng, s, d, p, 1)
+        tol = 2e-6 if dtype == np.float32 else 1e-12                     # sums of up to 72 terms of unit variance
+        np.testing.assert_allclose(to_np(xt.grad), gexp, rtol=tol, atol=tol * np.sqrt(nf[0] * nf[1]),
+                                   err_msg="col2spec trial %d" % trial)
