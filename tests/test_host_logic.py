@@ -38,13 +38,28 @@ def test_size_functions_equal_checker(name):
 
 
 def test_size_values_of_benchmark_configs():
-    # the table of output lengths the survey derives for the BASELINE configs
+    # output lengths of the reference's benchmark configurations, worked out by hand from mconv.py:73-118
     assert mconv.mcorr_valid_size(16, 256) == 16 and mconv.mconv_valid_size(16, 256) == 256
     grid = [(s, d, p) for s in (1, 2) for d in (1, 2) for p in (0, 3)]
     assert [mconv.mcorr_valid_size(8, 780, s, d, p) for s, d, p in grid] == [97, 390, 86, 346, 96, 389, 85, 345]
     assert [mconv.lcorr_valid_size(8, 780, s, d, p) for s, d, p in grid] == [773, 776, 766, 769, 387, 388, 383, 385]
     assert (mconv.mcorr_valid_size(8, 512), mconv.lcorr_valid_size(4, 41)) == (64, 38)
     assert (mconv.lcorr_valid_size(3, 256, 1, 2, 2), mconv.lcorr_valid_size(3, 41, 1, 1, 1)) == (254, 40)
+
+
+def test_timing_tool_counts_the_taps_that_exist():
+    """time_layers.py prices a pass by (output position, filter tap) pairs inside the input:
+    cfg3 has 512 such pairs on the Mellin axis and 152 on the linear one (64 x 8 and 38 x 4:
+    every tap of a valid-size output exists), config 2 the multiply counts of its (s, d, p) grid."""
+    import time_layers
+    assert time_layers.tap_pairs(hip.AX_MCORR, 8, 512, 64, 1, 1, 0) == 512
+    assert time_layers.tap_pairs(hip.AX_LCORR, 4, 41, 38, 1, 1, 0) == 152
+    grid = [(s, d, p) for s in (1, 2) for d in (1, 2) for p in (0, 3)]
+    gmac = [32 * 128 * 41 * time_layers.tap_pairs(hip.AX_MCORR, 8, 780, mconv.mcorr_valid_size(8, 780, s, d, p), s, d, p) / 1e9
+            for s, d, p in grid]
+    assert [round(v, 3) for v in gmac] == [0.130, 0.262, 0.116, 0.232, 0.129, 0.261, 0.114, 0.232]
+    brute = sum(1 for h in range(20) for f in range(5) if (3 * h + 2 * f - 4) >= 0 and (3 * h + 2 * f - 4) < 30)
+    assert time_layers.tap_pairs(hip.AX_LCORR, 5, 30, 20, 3, 2, 4) == brute
 
 
 def test_argument_errors_have_reference_wording():
