@@ -81,9 +81,17 @@ __global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict
                                                              Axis x, Axis y, int c_in, int batch,
                                                              int transposed_g, int transposed_gg) {
   const int plane = (int)(x.nh * y.nh), ng = (int)(x.ng * y.ng), nfy = (int)y.nf;
-  const int q = blockIdx.x * 256 + threadIdx.x;
+  // Workgroups are dealt to the eight dies in turn, each with an L2 of its own: renumber them so
+  // that a die writes one contiguous run of gg, and the cache lines that neighbouring blocks
+  // each write a part of are completed in one L2.
+  const unsigned per_z = gridDim.x * gridDim.y, total = per_z * gridDim.z;
+  const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const unsigned die = lin & 7u, mine = die * (total >> 3) + min(die, total & 7u) + (lin >> 3);
+  const unsigned block_z = mine / per_z, in_z = mine - block_z * per_z;
+  const unsigned block_y = in_z / gridDim.x, block_x = in_z - block_y * gridDim.x;
+  const int q = (int)block_x * 256 + threadIdx.x;
   if (q >= plane) return;
-  const int tap = blockIdx.y, fx = tap / nfy, fy = tap - fx * nfy;
+  const int tap = (int)block_y, fx = tap / nfy, fy = tap - fx * nfy;
   int ox = (int)((float)q * (1.0f / (float)y.nh));
   int oy = q - ox * (int)y.nh;
   if (oy < 0) { --ox; oy += (int)y.nh; } else if (oy >= (int)y.nh) { ++ox; oy -= (int)y.nh; }
@@ -92,7 +100,7 @@ __global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict
   const int src = (gx >= 0 && gy >= 0) ? gx * (int)y.ng + gy : -1;
   const int taps = (int)(x.nf * y.nf), pairs = batch * c_in;
 #pragma unroll 4
-  for (int nc = blockIdx.z; nc < pairs; nc += gridDim.z) {       // nc: (image, channel) in gg's own order
+  for (int nc = (int)block_z; nc < pairs; nc += gridDim.z) {     // nc: (image, channel) in gg's own order
     int nc_g = nc;
     if (transposed_g != transposed_gg) {
       const int a = transposed_gg ? nc / batch : nc / c_in;       // ci : bt
