@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "../../include/mellin_hip.h"
 #include "mellin_common.hpp"
 #include "igrad_gemm.hpp"
@@ -14,8 +16,10 @@ using namespace mellin;
 namespace {
 
 thread_local char g_error[512] = "";
-thread_local const char *g_variant = "";
-thread_local int g_forced = 0;   // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
+// Process-wide, not per thread: PyTorch runs the backward pass of device tensors on its
+// autograd thread, and a variant forced from the user's thread must hold there too.
+std::atomic<const char *> g_variant{""};
+std::atomic<int> g_forced{0};    // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
                                  // and without the row-wise weight gradient
 
 int fail(int code, const char *fmt, ...) {
@@ -31,9 +35,9 @@ int check_hip(hipError_t e, const char *what) {
   return fail(MELLIN_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
 }
 
-// The tap-product input gradient keeps c_in * taps values per grad_out element in
-// the workspace; past this size the two-pass variant is used instead.
-const size_t kMaxTapProductBytes = (size_t)1 << 30;
+// No form of the input gradient may ask for more scratch memory than this; a layer whose
+// specialised forms would need more runs in the gather form, which needs none.
+const size_t kMaxWorkspaceBytes = (size_t)1 << 30;
 
 bool mellin_kind(int k) { return k == AX_MCORR || k == AX_MCONV; }
 
@@ -60,6 +64,21 @@ int check_channels(const char *fn, i64 c_out, i64 c_in, i64 batch) {
   if (c_out < 0 || c_in < 0 || batch < 0)
     return fail(MELLIN_ERR_ARGUMENT, "%s: negative channel or batch count (c_out=%lld c_in=%lld batch=%lld)",
                 fn, (long long)c_out, (long long)c_in, (long long)batch);
+  // with the per-axis limit of 2^30, counts up to 2^20 keep every product of sizes the
+  // entry points form (a tensor's element count, a fan-in) inside 63 bits
+  const i64 lim = (i64)1 << 20;
+  if (c_out > lim || c_in > lim || batch > lim)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: channel or batch count beyond 2^20 (c_out=%lld c_in=%lld batch=%lld)",
+                fn, (long long)c_out, (long long)c_in, (long long)batch);
+  return MELLIN_OK;
+}
+
+// Element counts of the tensors of a call must stay below 2^60 (no such tensor can exist;
+// the test keeps every later product of sizes free of signed overflow).
+int check_counts(const char *fn, double a, double b, double c) {
+  const double lim = 1152921504606846976.0;   // 2^60
+  if (a >= lim || b >= lim || c >= lim)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: a tensor of this call would have 2^60 elements or more", fn);
   return MELLIN_OK;
 }
 
@@ -99,6 +118,8 @@ int accumulate_2d(const char *fn, int kind_x, int kind_y, const T *f, const T *g
   if ((rc = check_channels(fn, c_out, c_in, batch))) return rc;
   if ((rc = check_axis(fn, "x", kind_x, nfx, ngx, nhx, sx, dx, px, ux))) return rc;
   if ((rc = check_axis(fn, "y", kind_y, nfy, ngy, nhy, sy, dy, py, uy))) return rc;
+  if ((rc = check_counts(fn, (double)c_out * c_in * nfx * nfy, (double)batch * c_in * ngx * ngy,
+                         (double)batch * c_out * nhx * nhy))) return rc;
   const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
   if (batch * c_out * nh == 0) return MELLIN_OK;               // nothing to write
   if (c_in * nf * ng == 0) return MELLIN_OK;                   // empty sum: h unchanged
@@ -124,6 +145,8 @@ int check_corr2d(const char *fn, int kind_x, i64 batch, i64 c_in, i64 c_out,
   if ((rc = check_channels(fn, c_out, c_in, batch))) return rc;
   if ((rc = check_axis(fn, "x", kind_x, nfx, ngx, nhx, sx, dx, px, ux))) return rc;
   if ((rc = check_axis(fn, "y", AX_LCORR, nfy, ngy, nhy, sy, dy, py, uy))) return rc;
+  if ((rc = check_counts(fn, (double)c_out * c_in * nfx * nfy, (double)batch * c_in * ngx * ngy,
+                         (double)batch * c_out * nhx * nhy))) return rc;
   return MELLIN_OK;
 }
 
@@ -221,7 +244,7 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   // most of whose (position, filter row) pairs have no tap at all
   const bool mellin_wide = kind_x == AX_MCORR && c_in >= 16 && 8 * nhx <= 7 * ngx;
   if ((c_in >= 16 && !mellin_wide) || nfx < 2) return false;
-  if (mellin_wide && (double)batch * m2 * nhx * ngy * 4.0 > (double)kMaxTapProductBytes) return false;
+  if ((double)batch * m2 * nhx * ngy * 4.0 > (double)kMaxWorkspaceBytes) return false;
   const i64 pad = ((m2 + 31) / 32) * 32;
   if (pad * 2 > m2 * 3) return false;
   const i64 nf = nfx * nfy, nh = nhx * nhy;
@@ -240,6 +263,42 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   return true;
 }
 
+// Which form the fp32 input gradient takes, for the query and the call alike.  The three
+// specialised forms keep intermediate values in a workspace whose size grows with the
+// layer (partial rows, tap products, first-pass rows); a form whose workspace would pass
+// kMaxWorkspaceBytes is not taken, and the gather form (tiled or one thread per output),
+// which needs none, is the last resort.
+enum InputForm { IN_GATHER = 0, IN_FUSED, IN_TAPS, IN_TWO_PASS };
+struct InputPlans {
+  IgradPlan fused;
+  TapProductPlan taps;
+  TwoPassInput two;
+  size_t ws_bytes = 0;
+};
+
+int choose_input_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx,
+                      i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, InputPlans &ips) {
+  const int forced = g_forced;
+  ips.ws_bytes = 0;
+  if (forced == 1) return IN_GATHER;
+  if (forced == 0 && make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
+                                     px, py, ux, uy, ips.fused) && ips.fused.ws_bytes <= kMaxWorkspaceBytes) {
+    ips.ws_bytes = ips.fused.ws_bytes;
+    return IN_FUSED;
+  }
+  if (forced == 0 && make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, ips.taps) &&
+      ips.taps.ws_bytes <= kMaxWorkspaceBytes) {
+    ips.ws_bytes = ips.taps.ws_bytes;
+    return IN_TAPS;
+  }
+  if (plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py, ux, uy,
+                          ips.two) && ips.two.ws_bytes <= kMaxWorkspaceBytes) {
+    ips.ws_bytes = ips.two.ws_bytes;
+    return IN_TWO_PASS;
+  }
+  return IN_GATHER;
+}
+
 template <typename T>
 int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
                           const T *grad_out, i64 batch, i64 c_in, i64 c_out,
@@ -256,44 +315,33 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   if (!grad_input || (c_out * nf * nh != 0 && (!weight || !grad_out)))
     return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
-  if (sizeof(T) == 4 && g_forced == 0 && c_out * nf * nh != 0) {
-    IgradPlan ip;
-    if (make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
-                        px, py, ux, uy, ip)) {
-      if (ip.ws_bytes && (!workspace || workspace_bytes < ip.ws_bytes))
-        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
-                    ip.ws_bytes, workspace_bytes);
+  if (sizeof(T) == 4 && c_out * nf * nh != 0) {
+    InputPlans ips;
+    const int which = choose_input_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
+                                        px, py, ux, uy, ips);
+    if (which != IN_GATHER && ips.ws_bytes && (!workspace || workspace_bytes < ips.ws_bytes))
+      return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, ips.ws_bytes,
+                  workspace_bytes);
+    if (which == IN_FUSED) {
       g_variant = "mfma-fused";
-      return check_hip(launch_igrad(ip, (const float *)weight, (const float *)grad_out,
+      return check_hip(launch_igrad(ips.fused, (const float *)weight, (const float *)grad_out,
                                     (float *)grad_input, (float *)workspace, (hipStream_t)stream), fn);
     }
-  }
-  if (sizeof(T) == 4 && g_forced == 0 && c_out * nf * nh != 0) {
-    // tap products through the workspace, then a gather (any x axis kind)
-    TapProductPlan zp;
-    if (make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, zp) && zp.ws_bytes <= kMaxTapProductBytes) {
-      if (!workspace || workspace_bytes < zp.ws_bytes)
-        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
-                    zp.ws_bytes, workspace_bytes);
+    if (which == IN_TAPS) {
+      // tap products through the workspace, then a gather (any x axis kind)
       g_variant = "mfma-taps+fold";
-      hipError_t e = launch_tap_product(zp, (const float *)weight, (const float *)grad_out,
+      hipError_t e = launch_tap_product(ips.taps, (const float *)weight, (const float *)grad_out,
                                         (float *)workspace, (hipStream_t)stream);
       if (e == hipSuccess) {
         const Axis fx = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
         const Axis fy = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
-        e = launch_fold_xy(fx, fy, batch * c_in, zp.nf_pad, (const float *)workspace,
+        e = launch_fold_xy(fx, fy, batch * c_in, ips.taps.nf_pad, (const float *)workspace,
                            (float *)grad_input, (hipStream_t)stream);
       }
       return check_hip(e, fn);
     }
-  }
-  if (sizeof(T) == 4 && g_forced != 1 && c_out * nf * nh != 0) {
-    TwoPassInput tp;
-    if (plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy,
-                            dx, dy, px, py, ux, uy, tp)) {
-      if (!workspace || workspace_bytes < tp.ws_bytes)
-        return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
-                    tp.ws_bytes, workspace_bytes);
+    if (which == IN_TWO_PASS) {
+      const TwoPassInput &tp = ips.two;
       g_variant = "mfma+fold";
       hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight,
                                       (const float *)grad_out, nullptr, (float *)workspace,
@@ -377,6 +425,8 @@ int col_op(const char *fn, bool to_col, const T *src, i64 c_in, i64 batch, i64 n
   int rc = check_channels(fn, 0, c_in, batch);
   if (!rc) rc = check_axis(fn, "x", AX_MCORR, nfx, ngx, nggx, sx, dx, px, ux);
   if (!rc) rc = check_axis(fn, "y", AX_LCORR, nfy, ngy, nggy, sy, dy, py, uy);
+  if (!rc) rc = check_counts(fn, (double)batch * c_in * ngx * ngy,
+                             (double)batch * c_in * nfx * nfy * nggx * nggy, 0.0);
   if (rc) return rc;
   const i64 n_g = batch * c_in * ngx * ngy, n_gg = batch * c_in * nfx * nfy * nggx * nggy;
   if ((to_col ? n_gg : n_g) == 0) return MELLIN_OK;
@@ -687,16 +737,10 @@ size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
                                               MELLIN_CORR2D_DIMS) {
   if (elem_bytes != 4 || g_forced == 1) return 0;
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
-  if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
-  IgradPlan ip;
-  if (g_forced == 0 && make_igrad_plan(kind_x, CORR2D_ARGS, ip)) return ip.ws_bytes;
-  TapProductPlan zp;
-  if (g_forced == 0 && make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, zp) &&
-      zp.ws_bytes <= kMaxTapProductBytes)
-    return zp.ws_bytes;
-  TwoPassInput tp;
-  if (!plan_two_pass_input(kind_x, CORR2D_ARGS, tp)) return 0;
-  return tp.ws_bytes;
+  if (!batch || !c_in || !c_out || !nfx || !nfy || !ngx || !ngy || !nhx || !nhy) return 0;
+  InputPlans ips;
+  choose_input_plan(kind_x, CORR2D_ARGS, ips);
+  return ips.ws_bytes;
 }
 int mellin_corr2d_backward_input_f32(int kind_x, const float *weight,
                                      const float *grad_out, MELLIN_CORR2D_DIMS,
@@ -716,7 +760,7 @@ size_t mellin_corr2d_backward_weight_workspace(int kind_x, int elem_bytes,
                                                MELLIN_CORR2D_DIMS) {
   if (elem_bytes != 4 || g_forced == 1) return 0;
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
-  if (batch * c_in * c_out * nfx * nfy * ngx * ngy * nhx * nhy == 0) return 0;
+  if (!batch || !c_in || !c_out || !nfx || !nfy || !ngx || !ngy || !nhx || !nhy) return 0;
   WgradPlan wp;
   if (!make_wgrad_plan(forward_problem(kind_x, CORR2D_ARGS), wp, g_forced != 2)) return 0;
   return wp.ws_bytes;

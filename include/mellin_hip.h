@@ -124,8 +124,8 @@ MELLIN_DECL_2D(mellin_lconvlconv_f64, double);
  * mellin_corr2d_backward_*_workspace() for the byte count (0 = none) and pass
  * a device buffer of at least that size (256-byte aligned); its contents on
  * entry do not matter and are garbage on exit.  The count depends on the
- * variant in force on the calling thread (mellin_set_variant): query and call
- * under the same setting.
+ * variant in force (mellin_set_variant): query and call under the same
+ * setting.
  * ------------------------------------------------------------------------ */
 #define MELLIN_CORR2D_DIMS                                                     \
   int64_t batch, int64_t c_in, int64_t c_out, int64_t nfx, int64_t nfy,        \
@@ -281,15 +281,16 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
                                  void *workspace, size_t workspace_bytes,
                                  void *stream);
 
-/* Name of the kernel variant the most recent operator-level call on this
- * thread dispatched to (for tests and profiling): "generic", "mfma" (tiled
+/* Name of the kernel variant the most recent operator-level call of the
+ * process (on any thread: PyTorch runs backward passes on a thread of its own)
+ * dispatched to (for tests and profiling): "generic", "mfma" (tiled
  * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
  * (two-pass input gradient). */
 const char *mellin_last_variant(void);
 
-/* Force a variant for subsequent operator-level calls on this thread:
+/* Force a variant for subsequent operator-level calls of the process (all threads):
  * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
  * kernels; "two-pass" = automatic choice without the specialised gradient
  * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows"), i.e. the tiled ones.

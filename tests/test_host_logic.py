@@ -142,3 +142,37 @@ def test_cabi_rejects_bad_arguments_before_launch():
     assert lib.mellin_corr2d_forward_f32(hip.AX_MCORR, null, null, null, *empty, null, null) == 0
     assert lib.mellin_set_variant(b"no-such-variant") == 1
     assert lib.mellin_set_variant(b"") == 0
+
+
+def test_workspace_queries_are_bounded_and_overflow_safe():
+    """No form of the input gradient asks for more than 1 GiB of scratch memory (layers that
+    would run in the workspace-free gather form), the weight gradient's partial sums stay
+    small, and sizes whose product wraps to zero in 64 bits are not mistaken for empty."""
+    import random
+    cap = 1 << 30
+    # the layers that once asked for 773 GB and 5 GB
+    big = [(hip.AX_LCORR, 100, 15, 64, (33, 3), (780, 5000), (748, 4998)),
+           (hip.AX_MCORR, 100, 15, 64, (33, 3), (780, 5000), (23, 4998)),
+           (hip.AX_LCORR, 64, 8, 64, (16, 3), (2000, 80), (1985, 78))]
+    rnd = random.Random(5)
+    for _ in range(300):
+        nf = (rnd.randint(1, 40), rnd.randint(1, 8))
+        ng = (rnd.randint(nf[0], 4000), rnd.randint(nf[1], 600))
+        big.append((rnd.choice([hip.AX_LCORR, hip.AX_MCORR]), rnd.randint(1, 256), rnd.randint(1, 40),
+                    rnd.randint(1, 300), nf, ng, (rnd.randint(1, ng[0]), rnd.randint(1, ng[1]))))
+    for kind, n, c_in, c_out, nf, ng, nh in big:
+        dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), (0, 0), (1, 1))
+        assert hip.lib.mellin_corr2d_backward_input_workspace(kind, 4, *dims) <= cap, (kind, dims)
+        assert hip.lib.mellin_corr2d_backward_weight_workspace(kind, 4, *dims) <= cap, (kind, dims)
+    # extents whose nine-fold product wraps to zero in 64 bits: not an empty layer (an empty
+    # layer returns MELLIN_OK without looking at the pointers)
+    dims = hip._dims(1 << 16, 1 << 16, 1 << 16, (1, 1), (1 << 16, 1), (1 << 16, 1), (1, 1), (1, 1), (0, 0), (1, 1))
+    code = hip.lib.mellin_corr2d_backward_weight_f32(hip.AX_LCORR, None, None, *dims, None, None, 0, None)
+    assert code == 1 and "null pointer" in hip.last_error()
+    # tensors of 2^60 elements or more are refused outright
+    dims = hip._dims(1 << 20, 1 << 20, 1, (1, 1), (1 << 30, 1), (1 << 30, 1), (1, 1), (1, 1), (0, 0), (1, 1))
+    code = hip.lib.mellin_corr2d_backward_weight_f32(hip.AX_LCORR, None, None, *dims, None, None, 0, None)
+    assert code == 1 and "2^60" in hip.last_error()
+    dims = hip._dims(1 << 21, 1, 1, (1, 1), (4, 4), (4, 4), (1, 1), (1, 1), (0, 0), (1, 1))
+    code = hip.lib.mellin_corr2d_forward_f32(hip.AX_LCORR, None, None, None, *dims, None, None)
+    assert code == 1 and "2^20" in hip.last_error()
