@@ -44,6 +44,8 @@ SYMBOLS = {
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
 }
+SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
+SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
     SYMBOLS["mellin_corr2d_%s_f16_workspace" % _n] = (_size_t, [_int] + _DIMS)
 SYMBOLS["mellin_corr2d_forward_f16"] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
@@ -249,4 +251,18 @@ def corr2d_backward_weight(kind_x, input, grad_out, grad_weight, dims, workspace
     with torch.cuda.device(dev):
         _check(fn(kind_x, _dp(input), _dp(grad_out), *dims, _dp(grad_weight),
                   _dp(workspace), workspace_bytes, _stream(dev)))
+    return grad_weight
+
+
+def corr2d_backward_weight_static(kind_x, input, grad_out, grad_weight, dims):
+    """Weight gradient (fp32) with the partial sums in the library's static device array:
+    no allocation anywhere on the way.  Layers needing more than
+    mellin_static_scratch_bytes() raise; overlapping calls on one GPU race."""
+    dev = require_device(input, grad_out, grad_weight)
+    _same_dtype(input, grad_out, grad_weight)
+    if grad_weight.dtype != torch.float32:
+        raise RuntimeError("the allocation-free weight gradient takes float32 tensors, got %s" % grad_weight.dtype)
+    with torch.cuda.device(dev):
+        _check(lib.mellin_corr2d_backward_weight_static_f32(kind_x, _dp(input), _dp(grad_out), *dims,
+                                                            _dp(grad_weight), _stream(dev)))
     return grad_weight

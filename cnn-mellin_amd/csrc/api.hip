@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "../../include/mellin_hip.h"
 #include "mellin_common.hpp"
@@ -12,6 +13,13 @@
 #include "tile_gemm.hpp"
 
 using namespace mellin;
+
+// Scratch memory of mellin_corr2d_backward_weight_static_f32: one copy per GPU that runs
+// code of this library, held until the process ends.  The name is a host-side handle, not
+// a device address: host code only ever uses the per-device address that
+// static_scratch() obtains from hipGetSymbolAddress.
+#define MELLIN_STATIC_SCRATCH_BYTES (16u << 20)
+static __device__ __align__(256) unsigned char scratch[MELLIN_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -417,6 +425,31 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
                                                (hipStream_t)stream), fn);
 }
 
+// Address of the static scratch array on the current device (nullptr after fail()).  The
+// lookup runs once per device, on the first call made with that device current; it
+// allocates nothing (the array is part of the loaded code object).
+const int kMaxDevices = 64;
+void *g_scratch_addr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+void *static_scratch(const char *fn) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { fail(MELLIN_ERR_RUNTIME, "%s: hipGetDevice: %s", fn, hipGetErrorString(e)); return nullptr; }
+  if (dev < 0 || dev >= kMaxDevices) { fail(MELLIN_ERR_RUNTIME, "%s: device index %d out of range", fn, dev); return nullptr; }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_addr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      fail(MELLIN_ERR_RUNTIME, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_addr[dev] = ptr;
+  }
+  return g_scratch_addr[dev];
+}
+
 // Column ops (mconv.h:1247-1380): x Mellin correlation, y linear correlation.
 template <typename T>
 int col_op(const char *fn, bool to_col, const T *src, i64 c_in, i64 batch, i64 nfx, i64 nfy,
@@ -771,6 +804,20 @@ int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,
                                       size_t workspace_bytes, void *stream) {
   return corr2d_backward_weight<float>(__func__, kind_x, input, grad_out, CORR2D_ARGS,
                                        grad_weight, workspace, workspace_bytes, stream);
+}
+size_t mellin_static_scratch_bytes(void) { return MELLIN_STATIC_SCRATCH_BYTES; }
+int mellin_corr2d_backward_weight_static_f32(int kind_x, const float *input, const float *grad_out,
+                                             MELLIN_CORR2D_DIMS, float *grad_weight, void *stream) {
+  const size_t need = mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS);
+  if (need > MELLIN_STATIC_SCRATCH_BYTES)
+    return fail(MELLIN_ERR_WORKSPACE,
+                "%s: this layer needs %zu bytes of scratch memory, the static array holds %zu; use "
+                "mellin_corr2d_backward_weight_f32 with a workspace", __func__, need,
+                (size_t)MELLIN_STATIC_SCRATCH_BYTES);
+  void *ws = static_scratch(__func__);
+  if (!ws) return MELLIN_ERR_RUNTIME;
+  return corr2d_backward_weight<float>(__func__, kind_x, input, grad_out, CORR2D_ARGS, grad_weight, ws,
+                                       MELLIN_STATIC_SCRATCH_BYTES, stream);
 }
 int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       const double *grad_out, MELLIN_CORR2D_DIMS,

@@ -161,6 +161,26 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
                                       double *grad_weight, void *workspace,
                                       size_t workspace_bytes, void *stream);
 
+/* The weight gradient for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same result, bit for bit, as
+ * mellin_corr2d_backward_weight_f32, but the partial sums live in a static
+ * device array of mellin_static_scratch_bytes() = 16 MiB inside the library
+ * (one copy per GPU the library runs on, held until the process ends) instead
+ * of a caller's workspace: the call allocates and frees nothing.  Layers whose
+ * partial sums need more (mellin_corr2d_backward_weight_workspace() tells) are
+ * rejected with MELLIN_ERR_WORKSPACE.  The array's address is looked up on the
+ * first call made with a device current (not an allocation; make that call
+ * before capturing a graph).  All calls on one GPU share the array: its
+ * contents never need clearing (every word read was written by the same
+ * call), but two calls that overlap in time on one GPU (different streams or
+ * threads) race and give wrong results; serialise them. */
+size_t mellin_static_scratch_bytes(void);
+int mellin_corr2d_backward_weight_static_f32(int kind_x, const float *input,
+                                             const float *grad_out,
+                                             MELLIN_CORR2D_DIMS,
+                                             float *grad_weight, void *stream);
+
 /* forward with the layer's non-linearity applied on the way out: the acoustic
  * model runs every convolution as nonlinearity(conv(x)) (models.py:423-425), and
  * with ReLU, its default, that is out = max(0, bias + correlation) in the same
