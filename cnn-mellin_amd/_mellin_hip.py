@@ -40,6 +40,8 @@ SYMBOLS = {
     "mellin_last_error": (ctypes.c_char_p, []),
     "mellin_last_variant": (ctypes.c_char_p, []),
     "mellin_set_variant": (_int, [ctypes.c_char_p]),
+    "mellin_set_math": (_int, [_int]),
+    "mellin_get_math": (_int, []),
     "mellin_corr2d_backward_weight_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
@@ -89,6 +91,19 @@ def last_variant():
 
 def set_variant(name=None):
     _check(lib.mellin_set_variant((name or "").encode()))
+
+
+MATH_FP32, MATH_BF16X3 = 0, 1
+
+
+def set_math(mode):
+    """MATH_BF16X3 (default): fp32 products as six bf16 products of three-part operands, fp32
+    accumulate; MATH_FP32: the fp32 matrix instructions."""
+    _check(lib.mellin_set_math(int(mode)))
+
+
+def get_math():
+    return lib.mellin_get_math()
 
 
 def _check(code):

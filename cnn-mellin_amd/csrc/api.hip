@@ -27,6 +27,7 @@ thread_local char g_error[512] = "";
 // Process-wide, not per thread: PyTorch runs the backward pass of device tensors on its
 // autograd thread, and a variant forced from the user's thread must hold there too.
 std::atomic<const char *> g_variant{""};
+std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_forced{0};    // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
                                  // and without the row-wise weight gradient
 
@@ -140,6 +141,7 @@ int accumulate_2d(const char *fn, int kind_x, int kind_y, const T *f, const T *g
   pr.g_n = tg ? ng : c_in * ng;   pr.g_c = tg ? batch * ng : ng;
   pr.h_n = th ? nh : c_out * nh;  pr.h_m = th ? batch * nh : nh;
   pr.accumulate = 1;
+  pr.math = g_math;
   return check_hip(run_sepconv<T>(pr, f, g, (const T *)nullptr, h, (hipStream_t)stream), fn);
 }
 
@@ -199,6 +201,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
   pr.g_n = c_in * ng; pr.g_c = ng;
   pr.h_n = c_out * nh; pr.h_m = nh;
   pr.accumulate = 0;
+  pr.math = g_math;
   pr.relu = activation == MELLIN_ACT_RELU;
   if (wrote_half) *wrote_half = false;
   if (half_out && sizeof(T) == 4 && g_forced != 1) {
@@ -264,6 +267,7 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   pr.g_n = c_out * nh; pr.g_c = nh;
   pr.h_n = m2 * nhx * ngy; pr.h_m = nhx * ngy;
   pr.accumulate = 0;
+  pr.math = g_math;
   if (!make_tile_plan(pr, tp.plan, &tp.lds, &tp.mt, &tp.nt)) return false;
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
   tp.fold = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
@@ -370,6 +374,7 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
   pr.g_n = c_out * nh; pr.g_c = nh;
   pr.h_n = c_in * ng; pr.h_m = ng;
   pr.accumulate = 0;
+  pr.math = g_math;
   if (half_out && sizeof(T) == 4 && g_forced != 1) {
     // as in the forward pass: the matrix-core kernel stores half precision itself
     TilePlan pl;
@@ -719,6 +724,14 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
   return log_lift_backward<double>("mellin_log_lift_backward_f64", x, grad_y, eps, tau, flags, outer, t, inner,
                                    grad_x, grad_params, workspace, workspace_bytes, stream);
 }
+
+int mellin_set_math(int mode) {
+  if (mode != MELLIN_MATH_FP32 && mode != MELLIN_MATH_BF16X3)
+    return fail(MELLIN_ERR_ARGUMENT, "mellin_set_math: unknown mode %d", mode);
+  g_math = mode;
+  return MELLIN_OK;
+}
+int mellin_get_math(void) { return g_math; }
 
 int mellin_set_variant(const char *name) {
   if (!name || !*name) { g_forced = 0; return MELLIN_OK; }

@@ -33,7 +33,10 @@ struct SepConv {
   int accumulate;                // 1: h += result (h pre-initialised); 0: h = bias + result
   int relu = 0;                  // with accumulate == 0: h = max(0, bias + result)
   int out_half = 0;              // with accumulate == 0: h is half-precision storage (matrix-core kernel only)
+  int math = 0;                  // MATH_FP32: fp32 matrix instructions; MATH_BF16X3: bf16 ones on three-part operands
 };
+
+enum MathMode : int { MATH_FP32 = 0, MATH_BF16X3 = 1 };
 
 // Reduction form used by the weight gradient:
 // w[m, c, fx, fy] = sum_{n, hx, hy} a[n, m, hx, hy] * g[n, c, tap_x(hx, fx), tap_y(hy, fy)]

@@ -55,8 +55,11 @@ namespace {
 // channels fit in one or two chunks).
 // HOUT: H is half-precision storage (not with ACC): the fp32 results are rounded to
 // nearest even as they are stored.
-template <int MT, int NT, bool ACC, int MB, bool HOUT>
-__global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
+// SPLIT: the products run on the bf16 matrix cores, every fp32 operand as the exact sum of
+// three bf16 parts (tile_stage.hpp); only for layers whose channels are one chunk.  The
+// filter block then lives in LDS as fragments, built once per workgroup.
+template <int MT, int NT, bool ACC, int MB, bool HOUT, bool SPLIT>
+__global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H) {
   // The plan is read where it lies, in the kernel-argument segment (it is the
@@ -70,17 +73,18 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
   ConstPlan *const plan_base = (ConstPlan *)__builtin_amdgcn_kernarg_segment_ptr();
   ConstPlan *plp = plan_base;
 #define pl (*plp)
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   constexpr int M_T = MT * 32;
   constexpr int P = kWaves * NT * 32;
   const int g_words = pl.CC * pl.R * pl.RS;          // one signal buffer
-  const int w_words = M_T * pl.WSS;                  // one filter buffer
+  const int w_words = SPLIT ? 12 * (pl.KC16 >> 3) * M_T : M_T * pl.WSS;   // one filter buffer (SPLIT: 3 parts x 16-byte fragments)
   float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
-  const int ws_word0 = pl.sbuf * g_words;
-  float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS]
-  const bool single_chunk = pl.CC >= pl.C;
+  const int ws_word0 = SPLIT ? (pl.sbuf * g_words + 3) & ~3 : pl.sbuf * g_words;
+  float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS], or the fragments
+  const bool single_chunk = SPLIT || pl.CC >= pl.C;
+  const int n_tapoff = SPLIT ? pl.KC16 : pl.KCp;
   int *tapoff = (int *)(Ws0 + (single_chunk ? 1 : 2) * w_words);   // [KCp]
-  float *Bs = (float *)(tapoff + pl.KCp);            // [M_T] bias (zeros when accumulating)
+  float *Bs = (float *)(tapoff + n_tapoff);          // [M_T] bias (zeros when accumulating)
 
   MELLIN_PROBE_DECL
   const int tid = threadIdx.x;
@@ -177,23 +181,46 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
     // zeros (padding, rows without a tap) survive from the tile's chunk two stages back
     issue_signal<kWaves, kMemo>(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave,
                                &memo, ch == 0, ch < 2);
-    if (!single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
+    if (!SPLIT && !single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
   };
 
   {
     const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
-    for (int k = tid; k < pl.KCp; k += kThreads) {
+    const int k_taps = pl.C * pl.nf;
+    for (int k = tid; k < n_tapoff; k += kThreads) {
       int cl, t, fx, fy;
       by_nf.divmod(k, cl, t);
       by_nfy.divmod(t, fx, fy);
-      tapoff[k] = cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+      // (SPLIT pads the taps to a multiple of 16: a padded tap reads the lane's first word,
+      // always a staged one, and meets a zero weight)
+      tapoff[k] = (SPLIT && k >= k_taps) ? 0 : cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
     }
     for (int m = tid; m < M_T; m += kThreads)
       Bs[m] = (!ACC && bias && m0 + m < pl.M) ? bias[m0 + m] : 0.f;
   }
   MELLIN_STAMP(0);
   if (my_stages > 0) {
-    if (single_chunk) issue_filter(0, pl.C, ws_word0, true);
+    if (SPLIT) {
+      // filter fragments, once: a thread splits the eight taps k = 8 g .. 8 g + 7 of channel m
+      const int groups = pl.KC16 >> 3, k_taps = pl.C * pl.nf;
+      const FastDiv by_groups(groups), by_nf(pl.nf);
+      uintx4 *frag = (uintx4 *)Ws0;
+      for (int idx = tid; idx < groups * M_T; idx += kThreads) {
+        int m, g;
+        by_groups.divmod(idx, m, g);
+        float x[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int k = 8 * g + i;
+          int cl, t;
+          by_nf.divmod(k, cl, t);
+          x[i] = (k < k_taps && m0 + m < pl.M) ? F[(i64)(m0 + m) * pl.f_m + (i64)cl * pl.f_c + t] : 0.f;
+        }
+        store_frag(frag, groups, M_T, g, m, x);
+      }
+    } else if (single_chunk) {
+      issue_filter(0, pl.C, ws_word0, true);
+    }
     issue_stage(0, 0, 0);
   }
   MELLIN_STAMP(1);
@@ -331,6 +358,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
     // ---- matrix-core loop over the tap pairs of this chunk
     {
       const int cc = min(pl.CC, pl.C - ch * pl.CC);
+      if (SPLIT)
+        multiply_taps_split<MT, NT>(acc, (const uintx4 *)Ws0, M_T, tapoff, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words,
+                                    lane_base, pl.KC16, l32, half);
+      else
       multiply_taps<MT, NT>(acc, Ws0 + (single_chunk ? 0 : (st & 1) * w_words) + l32 * pl.WSS + half, 32 * pl.WSS,
                             tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
@@ -341,10 +372,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 4 : 2)) void tile_gemm_kernel(
 #undef pl
 }
 
-template <int MT, int NT, bool ACC, int MB, bool HOUT = false>
+template <int MT, int NT, bool ACC, int MB, bool HOUT = false, bool SPLIT = false>
 hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const float *f,
                           const float *g, const float *bias, float *h, hipStream_t stream) {
-  auto kern = tile_gemm_kernel<MT, NT, ACC, MB, HOUT>;
+  auto kern = tile_gemm_kernel<MT, NT, ACC, MB, HOUT, SPLIT>;
   if (lds_bytes > 64 * 1024) {
     // opt in to more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per CU)
     static thread_local size_t granted = 0;
@@ -363,10 +394,11 @@ hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const
 
 // Workgroups of the forward kernel that a CU holds at once: bounded by LDS and
 // by the registers of the instance (NT == 2 needs more than 128).
-static int workgroups_per_cu(size_t lds_bytes, int mt, int nt) {
+static int workgroups_per_cu(size_t lds_bytes, int mt, int nt, bool split) {
   const int by_lds = (int)((160 * 1024) / (lds_bytes + 512));
   (void)mt;
-  return std::max(1, std::min(by_lds, nt == 2 ? 3 : 4));
+  const int by_regs = split ? (nt == 2 ? 2 : 3) : (nt == 2 ? 3 : 4);
+  return std::max(1, std::min(by_lds, by_regs));
 }
 
 // Fill `pl` for the problem `pr`; returns false when the tiled kernel does not
@@ -411,7 +443,8 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     // full one's rate (measured), so the smaller tile wins when it fills its last round
     // that much better.
     const i64 big = pr.batch * ((Q + 255) / 256) * m_tiles, small = pr.batch * ((Q + 127) / 128) * m_tiles;
-    const i64 slots_big = 256 * 3, slots_small = 256 * 4;
+    const bool want_split = pr.math == MATH_BF16X3;
+    const i64 slots_big = 256 * (want_split ? 2 : 3), slots_small = 256 * (want_split ? 3 : 4);
     const double fill_big = (double)big / (double)(((big + slots_big - 1) / slots_big) * slots_big);
     const double fill_small = (double)small / (double)(((small + slots_small - 1) / slots_small) * slots_small);
     if (0.9 * fill_small > 1.05 * fill_big) *nt = 1;       // only on a clear margin: layers staged in chunks lose more
@@ -505,15 +538,28 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   *lds_bytes = 4 * (2 * (size_t)pl.CC * pl.R * pl.RS + (single ? 1 : 2) * (size_t)M_T * pl.WSS +
                     pl.KCp + M_T);
   if (*lds_bytes > 76 * 1024) return false;
+  // the bf16 matrix cores: when the whole filter is one chunk and its fragments fit
+  pl.split = 0;
+  pl.KC16 = 0;
+  const int kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
+  auto split_lds = [&](int sbuf) {
+    return 4 * ((((size_t)sbuf * pl.CC * pl.R * pl.RS) + 3) & ~(size_t)3) + (size_t)6 * kc16 * M_T +
+           4 * (size_t)(kc16 + M_T);
+  };
+  if (pr.math == MATH_BF16X3 && single && split_lds(2) <= 76 * 1024) {
+    pl.split = 1;
+    pl.KC16 = kc16;
+    *lds_bytes = split_lds(2);
+  }
   // A launch small enough that every tile gets a workgroup of its own once the
   // second signal buffer is dropped (more workgroups fit per CU) runs as one
   // wave of single-stage workgroups: nothing to prefetch, and no second round
   // in which most of the chip idles.
   pl.sbuf = 2;
   if (single) {
-    const size_t one = *lds_bytes - 4 * (size_t)pl.CC * pl.R * pl.RS;
-    const i64 slots2 = 256 * (i64)workgroups_per_cu(*lds_bytes, *mt, *nt);
-    const i64 slots1 = 256 * (i64)workgroups_per_cu(one, *mt, *nt);
+    const size_t one = pl.split ? split_lds(1) : *lds_bytes - 4 * (size_t)pl.CC * pl.R * pl.RS;
+    const i64 slots2 = 256 * (i64)workgroups_per_cu(*lds_bytes, *mt, *nt, pl.split);
+    const i64 slots1 = 256 * (i64)workgroups_per_cu(one, *mt, *nt, pl.split);
     const i64 wgs = (i64)pl.total_tiles * m_tiles;
     if (wgs > slots2 && wgs <= slots1) { pl.sbuf = 1; *lds_bytes = one; }
   }
@@ -526,7 +572,7 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const int M_T = mt * 32;
   // persistent workgroups: as many as fit at once on the 256 CUs
   const int m_tiles = (pl.M + M_T - 1) / M_T;
-  const int per_cu = workgroups_per_cu(lds_bytes, mt, nt);
+  const int per_cu = workgroups_per_cu(lds_bytes, mt, nt, pl.split);
   int gx = std::max(1, (256 * per_cu) / m_tiles);
   gx = std::min(gx, pl.total_tiles);
   if (pl.sbuf == 1 && gx < pl.total_tiles) return hipErrorInvalidValue;   // one buffer: one stage per workgroup
@@ -535,6 +581,11 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
+    if (pl.split) {                                                                          \
+      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream); \
+      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, true>(pl, lds_bytes, grid, f, g, bias, h, stream);   \
+      return launch_variant<MT_, NT_, false, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream);                   \
+    }                                                                                        \
     if (pl.accumulate)                                                                       \
       return memo ? launch_variant<MT_, NT_, true, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)  \
                   : launch_variant<MT_, NT_, true, 0>(pl, lds_bytes, grid, f, g, bias, h, stream); \

@@ -9,6 +9,8 @@
 namespace mellin {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
@@ -380,6 +382,105 @@ __device__ __forceinline__ void multiply_taps(floatx16 (&acc)[MT][NT], const flo
       for (int t = 0; t < NT; ++t)
         acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[t], acc[i][t], 0, 0, 0);
   }
+}
+
+// ---- fp32 products on the bf16 matrix cores ------------------------------------------
+// An fp32 value is the exact sum of three bf16 values (8 + 8 + 8 significant bits):
+// hi = x with its low 16 bits cleared, mid = (x - hi) likewise, lo = x - hi - mid.  A
+// product x * y is then the sum of nine bf16 products, each exact in fp32; the six
+// largest (hi hi, hi mid, mid hi, hi lo, lo hi, mid mid) carry everything down to
+// 2^-24 of |x y|, i.e. what an fp32 multiply-add keeps.  v_mfma_f32_32x32x16_bf16
+// accumulates in fp32 and runs at sixteen times the rate of v_mfma_f32_32x32x2_f32
+// per product, so six of them cost three eighths of the fp32 instruction's time.
+__device__ __forceinline__ bf16x8 as_bf16x8(uintx4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// x[0..8) -> packed hi / mid / lo parts (element i in half i & 1 of word i >> 1)
+__device__ __forceinline__ void split8(const float (&x)[8], uintx4 &hi, uintx4 &mid, uintx4 &lo) {
+  unsigned m[8], l[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float r1 = x[i] - __uint_as_float(__float_as_uint(x[i]) & 0xFFFF0000u);
+    const float r2 = r1 - __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
+    m[i] = __float_as_uint(r1);
+    l[i] = __float_as_uint(r2);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // the upper halves of two words: {a[31:16], b[31:16]} -> word (a high, b low)
+    hi[i] = __builtin_amdgcn_perm(__float_as_uint(x[2 * i + 1]), __float_as_uint(x[2 * i]), 0x07060302u);
+    mid[i] = __builtin_amdgcn_perm(m[2 * i + 1], m[2 * i], 0x07060302u);
+    lo[i] = __builtin_amdgcn_perm(l[2 * i + 1], l[2 * i], 0x07060302u);
+  }
+}
+
+// acc += A * B over 16 values of k, both operands as hi / mid / lo parts; small terms first
+__device__ __forceinline__ void mfma_split6(floatx16 &acc, const uintx4 &ah, const uintx4 &am, const uintx4 &al,
+                                            const uintx4 &bh, const uintx4 &bm, const uintx4 &bl) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(al), as_bf16x8(bh), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ah), as_bf16x8(bl), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(am), as_bf16x8(bm), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(am), as_bf16x8(bh), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ah), as_bf16x8(bm), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ah), as_bf16x8(bh), acc, 0, 0, 0);
+}
+
+// Fragment store of a (rows x K) fp32 operand, K a multiple of 16: the parts of the eight
+// values k = 8 g .. 8 g + 7 of row r are one 16-byte word at
+//   frag[(part * groups + g) * rows + r],   groups = K / 8,
+// so the 32 lanes of a half-wave (rows r .. r + 31, one group) read 512 consecutive bytes.
+__device__ __forceinline__ void store_frag(uintx4 *frag, int groups, int rows, int g, int r, const float (&x)[8]) {
+  uintx4 hi, mid, lo;
+  split8(x, hi, mid, lo);
+  frag[(0 * groups + g) * rows + r] = hi;
+  frag[(1 * groups + g) * rows + r] = mid;
+  frag[(2 * groups + g) * rows + r] = lo;
+}
+
+// The matrix-core loop of multiply_taps on the bf16 cores: the filter block comes as
+// fragments (store_frag: rows = M_T channels, K = KC16 taps, zero past the last tap),
+// the signal words are read as in multiply_taps, eight taps per lane and step (lane half
+// h takes taps 16 s + 8 h ..), and split in registers.  tp[k] is valid for k < KC16.
+template <int MT, int NT>
+__device__ __forceinline__ void multiply_taps_split(floatx16 (&acc)[MT][NT], const uintx4 *frag, int m_rows,
+                                                    const int *tp, const float *Gs, const int (&lane_base)[NT],
+                                                    int KC16, int l32, int half) {
+  const int groups = KC16 >> 3;
+  const int steps = KC16 >> 4;
+  struct Ops { uintx4 ah[MT], am[MT], al[MT], bh[NT], bm[NT], bl[NT]; };
+  auto fetch = [&](int s, Ops &o) {
+    const int g = 2 * s + half;
+    const int4 o0 = *(const int4 *)(tp + 8 * g), o1 = *(const int4 *)(tp + 8 * g + 4);
+    const int off[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = Gs[lane_base[t] + off[i]];
+      split8(x, o.bh[t], o.bm[t], o.bl[t]);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      o.ah[i] = frag[(0 * groups + g) * m_rows + i * 32 + l32];
+      o.am[i] = frag[(1 * groups + g) * m_rows + i * 32 + l32];
+      o.al[i] = frag[(2 * groups + g) * m_rows + i * 32 + l32];
+    }
+  };
+  auto multiply = [&](const Ops &o) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) mfma_split6(acc[i][t], o.ah[i], o.am[i], o.al[i], o.bh[t], o.bm[t], o.bl[t]);
+  };
+  Ops a, b;
+  int s = 0;
+  if (steps > 0) fetch(0, a);
+  for (; s + 1 < steps; s += 2) {
+    fetch(s + 1, b);
+    multiply(a);
+    if (s + 2 < steps) fetch(s + 2, a);
+    multiply(b);
+  }
+  if (s < steps) multiply(a);
 }
 
 }  // namespace mellin

@@ -310,6 +310,21 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
  * (two-pass input gradient). */
 const char *mellin_last_variant(void);
 
+/* How the matrix-core kernels form their fp32 products (process-wide).
+ *   MELLIN_MATH_BF16X3 (default)  every fp32 operand is taken as the exact sum of three
+ *     bf16 values (8 + 8 + 8 significant bits) and a product as the sum of the six largest
+ *     of the nine bf16 cross products, which the bf16 matrix instructions form exactly and
+ *     accumulate in fp32; what is dropped is below 2^-24 of the product, i.e. below the
+ *     rounding of an fp32 multiply-add.  Storage, accumulation and results are fp32.
+ *   MELLIN_MATH_FP32  the fp32 matrix instructions (v_mfma_f32_32x32x2_f32), one sixth of
+ *     the multiply rate.
+ * Kernels that have no bf16 form yet run in fp32 under either setting.  Infinities in
+ * the operands give NaN under MELLIN_MATH_BF16X3 (inf - inf while splitting). */
+#define MELLIN_MATH_FP32 0
+#define MELLIN_MATH_BF16X3 1
+int mellin_set_math(int mode);
+int mellin_get_math(void);
+
 /* Force a variant for subsequent operator-level calls of the process (all threads):
  * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
  * kernels; "two-pass" = automatic choice without the specialised gradient
