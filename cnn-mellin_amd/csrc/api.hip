@@ -172,6 +172,7 @@ SepConv forward_problem(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64
   pr.g_n = c_in * ng; pr.g_c = ng;
   pr.h_n = c_out * nh; pr.h_m = nh;
   pr.accumulate = 0;
+  pr.math = g_math;
   return pr;
 }
 

@@ -57,9 +57,10 @@ struct WgradPlan {
   int CCj;                         // input channels a column block can touch
   int GSS;                         // row stride of the staged grad_out tile (words)
   int S;                           // position shares = persistent workgroups per output block
-  int rows_mode;                   // 1: the row-wise kernel (one output row per wavefront)
+  int rows_mode;                   // 1: the row-wise kernel (one output row per wavefront); 2: its bf16 form
   int nbuf;                        // row-wise kernel: LDS buffers per operand (1 or 2)
   int rpw;                         // row-wise kernel: output rows per wavefront and unit
+  int split;                       // the caller allows the bf16 matrix cores (three-part operands)
   size_t lds_bytes, ws_bytes;
 };
 

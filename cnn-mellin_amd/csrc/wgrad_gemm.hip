@@ -483,6 +483,309 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
   }
 }
 
+// The row-wise weight gradient on the bf16 matrix cores (tile_stage.hpp: every fp32 operand
+// as the exact sum of three bf16 parts, six products each).  Same units and partial-sum
+// scheme as above; what differs is how the operands reach the matrix instructions.
+//
+//   * A step covers 16 positions, two groups of eight consecutive outputs of one row (one
+//     per half-wave); a row of noy outputs is NG = ceil(noy / 8) groups, the last one moved
+//     back to start at noy - 8 so that it is eight whole positions too (the ones it shares
+//     with the group before it meet zeros in the other operand).  The groups of a unit are
+//     numbered row by row and paired into steps regardless of rows; wavefront w takes steps
+//     w, w + 4, ...
+//   * grad_out (95 % of the bytes) never touches LDS: the eight positions of a lane's
+//     channel are 32 consecutive bytes of global memory, loaded straight into registers
+//     two steps ahead and split there.  Every grad_out value is loaded and split once.
+//   * the input words a unit needs are loaded into registers while the unit before it
+//     multiplies, then split once, by all threads, into 16-byte fragments
+//     Bf[part][channel][virtual row][group][fy]: the eight input words that the group's
+//     positions read through filter column fy (zeros for padding and for rows without a
+//     tap).  One thread makes all nfy fragments of a (channel, row, group): it splits the
+//     8 + nfy - 1 words once and assembles the shifted copies from the packed halves.  A
+//     lane (column j = (c, fx, fy)) fetches its operand of a step with three aligned
+//     16-byte LDS reads.
+// Nothing here uses the direct global->LDS loads, so the compiler counts every load in
+// flight and a wait for one never drags in the younger ones.  Needs unit y stride, no y
+// up-sampling and unit y dilation (consecutive filter columns read consecutive words).
+constexpr int kStreamTasks = 2;                    // (channel, row, group) tasks a thread can hold in registers
+template <int MT, int JT>
+__global__ __launch_bounds__(kThreads, (MT == 1 ? 3 : 2)) void wgrad_stream_kernel(
+    WgradPlan wp, const float *__restrict__ A, const float *__restrict__ G,
+    float *__restrict__ ws) {
+  extern __shared__ __align__(16) float lds[];
+  const TilePlan &pl = wp.t;
+  constexpr int M_T = MT * 32, J_T = JT * 32;
+  const int RB = kWaves * wp.rpw;                    // output rows per unit
+  const int NG = (pl.noy + 7) >> 3;                  // groups per row
+  const int tail0 = pl.noy - 8;                      // first position of a row's last group
+  const int tasks_max = wp.CCj * pl.R * NG;          // (channel, virtual row, group) triples
+  const int bf_part = tasks_max * pl.nfy + 1;        // fragments per part; the last word of a part is zeros
+  uintx4 *Bf = (uintx4 *)lds;                        // [3][CCj][R][NG][nfy] (+ the zero word)
+  int2 *step_tab = (int2 *)(Bf + 3 * bf_part);       // [groups of a full unit]: grad_out offset, fragment offset
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, l32 = lane & 31;
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+
+  const int mg = blockIdx.y / wp.j_groups, jg = blockIdx.y - mg * wp.j_groups;
+  const int m0 = mg * M_T, j0 = jg * J_T;
+  const int c_lo = j0 / pl.nf;
+  const int j_last = min(wp.J, j0 + J_T) - 1;
+  const int ccj = j_last / pl.nf - c_lo + 1;
+
+  // fragment word of column j's tap for (unit row 0, group 0)
+  int col_word[JT];
+  {
+    const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
+#pragma unroll
+    for (int t = 0; t < JT; ++t) {
+      const int j = min(j0 + t * 32 + l32, wp.J - 1);   // columns past J are computed but never stored
+      int c, tt, fx, fy;
+      by_nf.divmod(j, c, tt);
+      by_nfy.divmod(tt, fx, fy);
+      col_word[t] = ((c - c_lo) * pl.R + pl.Bx * fx + pl.Cx0) * NG * pl.nfy + fy;
+    }
+  }
+  // this lane's grad_out channel per tile, as a word offset within an image (channels past M
+  // read the last one; their rows of the result are never used)
+  int a_off[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) a_off[i] = min(m0 + i * 32 + l32, pl.M - 1) * (int)wp.a_m;
+
+  const int units_per_image = (pl.nox_eff + RB - 1) / RB;
+  const int total_units = pl.batch * units_per_image;
+  const int share = total_units / (int)gridDim.x, extra = total_units - share * (int)gridDim.x;
+  const int my_units = share + ((int)blockIdx.x < extra ? 1 : 0);
+  const int first_unit = (int)blockIdx.x * share + min((int)blockIdx.x, extra);
+
+  const FastDiv by_ng(NG), by_r(pl.R), by_nfx(pl.nfx);
+  for (int i = tid; i < RB * NG + 1; i += kThreads) {
+    int r, g;
+    by_ng.divmod(i, r, g);                              // group i of the unit: row r, group g of the row
+    step_tab[i] = make_int2(r * pl.noy + (g == NG - 1 ? tail0 : 8 * g), (pl.Ax * r * NG + g) * pl.nfy);
+  }
+  if (tid < 3) Bf[tid * bf_part + bf_part - 1] = uintx4{0u, 0u, 0u, 0u};
+
+  // ---- the input words of a unit, in registers --------------------------------------
+  // task tk = (cl * R + vrow) * NG + g; a thread takes tasks tid, tid + 256, ...  A task loads
+  // the E = 8 + nfy - 1 words its nfy fragments share (up to 16).  What does not change
+  // from unit to unit is worked out once: the task's virtual row (-1: no such task), the
+  // offset of its first word within an image apart from the row, which of its words lie
+  // inside the image, and how many leading positions the group before already covers.
+  const int E = 8 + pl.nfy - 1, n4 = (E + 3) >> 2;
+  struct XRegs { float v[kStreamTasks][16]; };
+  int t_row[kStreamTasks], t_off[kStreamTasks], t_mask[kStreamTasks], t_dead[kStreamTasks];
+#pragma unroll
+  for (int k = 0; k < kStreamTasks; ++k) {
+    const int tk = tid + k * kThreads;
+    int rest, g, cl, vrow;
+    by_ng.divmod(tk, rest, g);
+    by_r.divmod(rest, cl, vrow);
+    const bool tail = g == NG - 1;
+    const int c0 = (tail ? tail0 : 8 * g) + pl.cy;         // signal column of the group's first position, fy = 0
+    int mask = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) mask |= (e < E && c0 + e >= 0 && c0 + e < pl.ngy) ? 1 << e : 0;
+    // the whole run of 4 * n4 words lies inside the row: it can be loaded 16 bytes at a time
+    if (c0 >= 0 && c0 + 4 * n4 <= pl.ngy) mask |= 1 << 16;
+    t_row[k] = (tk < tasks_max && cl < ccj) ? vrow : -1;
+    t_off[k] = cl * (int)pl.g_c + c0;                      // fits: c_in * ngx * ngy < 2^31
+    t_mask[k] = mask;
+    t_dead[k] = tail ? 8 * g - tail0 : 0;
+  }
+  auto load_x = [&](int ui, XRegs &xr) {
+    const int unit = first_unit + ui;
+    const int u = unit / pl.batch, n = unit - u * pl.batch;
+    const int ox_lo = u * RB, rows = min(RB, pl.nox_eff - ox_lo);
+    const int R_tile = mellin_x ? rows * pl.nfx : pl.ax * (rows - 1) + pl.bx_span + 1;
+    const int vx_min = pl.ax * ox_lo + pl.cx + pl.bx_min;
+    const float *Gn = G + (i64)n * pl.g_n + (i64)c_lo * pl.g_c;
+#pragma unroll
+    for (int k = 0; k < kStreamTasks; ++k) {
+      const int vrow = t_row[k];
+      int gx = -1;
+      if (vrow >= 0 && vrow < R_tile) {
+        if (mellin_x) {
+          int oxl, fx;
+          by_nfx.divmod(vrow, oxl, fx);
+          gx = mellin_tap32(pl.kind_x, ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux, pl.mg_p1);
+        } else {
+          const int vx = vx_min + vrow;
+          if (vx >= 0) {
+            if (pl.ux == 1) { if (vx < pl.ngx) gx = vx; }
+            else { const int qx = vx / pl.ux; if (qx * pl.ux == vx && qx < pl.ngx) gx = qx; }
+          }
+        }
+      }
+      const float *src = Gn + (t_off[k] + max(gx, 0) * pl.ngy);
+      const int mask = gx >= 0 ? t_mask[k] : 0;
+      if (mask >> 16) {
+        typedef float4 __attribute__((aligned(4))) float4u;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float4 w = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (q < n4) w = *(const float4u *)(src + 4 * q);
+          xr.v[k][4 * q] = w.x; xr.v[k][4 * q + 1] = w.y; xr.v[k][4 * q + 2] = w.z; xr.v[k][4 * q + 3] = w.w;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) xr.v[k][e] = (mask >> e & 1) ? src[e] : 0.f;
+      }
+    }
+  };
+  auto store_x = [&](const XRegs &xr) {
+#pragma unroll
+    for (int k = 0; k < kStreamTasks; ++k) {
+      const int tk = tid + k * kThreads;
+      if (tk >= tasks_max) continue;
+      // the three parts of every word, packed in pairs: P[part][q] = words 2 q, 2 q + 1
+      unsigned P[3][8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        unsigned h[2], m[2], l[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const float x = xr.v[k][2 * q + b];
+          const float r1 = x - __uint_as_float(__float_as_uint(x) & 0xFFFF0000u);
+          const float r2 = r1 - __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
+          h[b] = __float_as_uint(x); m[b] = __float_as_uint(r1); l[b] = __float_as_uint(r2);
+        }
+        P[0][q] = __builtin_amdgcn_perm(h[1], h[0], 0x07060302u);
+        P[1][q] = __builtin_amdgcn_perm(m[1], m[0], 0x07060302u);
+        P[2][q] = __builtin_amdgcn_perm(l[1], l[0], 0x07060302u);
+      }
+      // positions the group before already covers become zeros (pairs 2 i, 2 i + 1 of the fragment)
+      const int dead = t_dead[k];
+      unsigned keep[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) keep[i] = 2 * i + 1 < dead ? 0u : (2 * i < dead ? 0xFFFF0000u : 0xFFFFFFFFu);
+#pragma unroll
+      for (int fy = 0; fy < 8; ++fy) {
+        if (fy < pl.nfy) {
+#pragma unroll
+          for (int part = 0; part < 3; ++part) {
+            uintx4 w;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              // words fy + 2 i, fy + 2 i + 1
+              const unsigned v = (fy & 1) ? __builtin_amdgcn_alignbit(P[part][(fy + 1) / 2 + i < 8 ? (fy + 1) / 2 + i : 7],
+                                                                       P[part][(fy - 1) / 2 + i], 16)
+                                          : P[part][fy / 2 + i];
+              w[i] = v & keep[i];
+            }
+            Bf[part * bf_part + tk * pl.nfy + fy] = w;
+          }
+        }
+      }
+    }
+  };
+
+  floatx16 acc[MT][JT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
+
+  // ---- steps ----------------------------------------------------------------------------
+  // Operands of step s of the current unit for this lane: the grad_out words come from
+  // global memory (requested two steps ahead), the fragments from LDS.
+  struct AOp { float4 lo[MT], hi[MT]; int bword; };
+  const float *abase = A;                               // grad_out of the unit's image and first row (wave-uniform)
+  int live_groups = 0;                                  // groups of the current unit
+  auto load_a = [&](int s, AOp &o) {
+    int gi = 2 * s + half;
+    const bool live = gi < live_groups;
+    if (!live) gi = 0;                                  // past the last group: any valid words, and zeros on the other side
+    const int2 e = step_tab[gi];
+    o.bword = live ? e.y : -1;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      typedef float4 __attribute__((aligned(4))) float4u;   // a row starts wherever the rows before it end
+      const float *p = abase + (a_off[i] + e.x);
+      o.lo[i] = *(const float4u *)p;
+      o.hi[i] = *(const float4u *)(p + 4);
+    }
+  };
+  auto multiply_step = [&](const AOp &o) {
+    uintx4 bh[JT], bm[JT], bl[JT];
+#pragma unroll
+    for (int t = 0; t < JT; ++t) {
+      const uintx4 *b = Bf + (o.bword >= 0 ? col_word[t] + o.bword : bf_part - 1);
+      bh[t] = b[0]; bm[t] = b[bf_part]; bl[t] = b[2 * bf_part];
+    }
+    uintx4 ah[MT], am[MT], al[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const float x[8] = {o.lo[i].x, o.lo[i].y, o.lo[i].z, o.lo[i].w, o.hi[i].x, o.hi[i].y, o.hi[i].z, o.hi[i].w};
+      split8(x, ah[i], am[i], al[i]);
+    }
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) mfma_split6(acc[i][t], ah[i], am[i], al[i], bh[t], bm[t], bl[t]);
+  };
+
+  XRegs xr;
+  if (my_units > 0) load_x(0, xr);
+  for (int ui = 0; ui < my_units; ++ui) {
+    const int unit = first_unit + ui;
+    const int u = unit / pl.batch, n = unit - u * pl.batch;
+    const int ox_lo = u * RB, rows = min(RB, pl.nox_eff - ox_lo);
+    live_groups = rows * NG;
+    const int steps = (live_groups + 1) >> 1;
+    abase = A + (i64)n * wp.a_n + (i64)ox_lo * pl.noy;
+    __syncthreads();                                     // every wavefront is done with the fragments of the unit before
+    // this wavefront's first two steps: their grad_out words travel while the input is split
+    AOp b0, b1, b2;
+    load_a(min(wave, steps - 1), b0);
+    load_a(min(wave + kWaves, steps - 1), b1);
+    b2 = b1;
+    store_x(xr);
+    __syncthreads();                                     // fragments complete
+    if (ui + 1 < my_units) load_x(ui + 1, xr);           // consumed at the top of the next unit
+    // three operand buffers in rotation, two steps in flight; no copies, so no wait for a
+    // younger load sneaks in
+    for (int s = wave; s < steps; s += 3 * kWaves) {
+      if (s + 2 * kWaves < steps) load_a(s + 2 * kWaves, b2);
+      multiply_step(b0);
+      if (s + kWaves >= steps) break;
+      if (s + 3 * kWaves < steps) load_a(s + 3 * kWaves, b0);
+      multiply_step(b1);
+      if (s + 2 * kWaves >= steps) break;
+      if (s + 4 * kWaves < steps) load_a(s + 4 * kWaves, b1);
+      multiply_step(b2);
+    }
+  }
+
+  // ---- sum the four wavefronts in wave order, then write the partial block ------
+  __syncthreads();
+  float *red = lds;                                   // [M_T][J_T]
+  for (int w = 0; w < kWaves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < JT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float *dst = red + m * J_T + t * 32 + l32;
+            if (w == 0) *dst = acc[i][t][r];
+            else *dst += acc[i][t][r];
+          }
+    }
+    __syncthreads();
+  }
+  float *out = ws + (i64)blockIdx.x * wp.M_pad * wp.J_pad + (i64)m0 * wp.J_pad + j0;
+  for (int e = tid; e < M_T * J_T; e += kThreads) {
+    const int m = e / J_T, jj = e - m * J_T;
+    out[(i64)m * wp.J_pad + jj] = red[e];
+  }
+}
+
 // W[m, j] = sum over the S partial blocks, in index order.  A block of 256
 // threads handles 16 outputs: 16 threads per output add every 16th partial,
 // then thread 0 of each output adds the 16 sums in order.
@@ -549,6 +852,23 @@ hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const flo
   return hipGetLastError();
 }
 
+template <int MT, int JT>
+hipError_t launch_stream(const WgradPlan &wp, dim3 grid, const float *a, const float *g, float *ws,
+                         hipStream_t stream) {
+  auto kern = wgrad_stream_kernel<MT, JT>;
+  if (wp.lds_bytes > 64 * 1024) {
+    static thread_local size_t granted = 0;
+    if (granted < wp.lds_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)wp.lds_bytes);
+      if (e != hipSuccess) return e;
+      granted = wp.lds_bytes;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 // Plan the weight gradient of the layer whose FORWARD problem is `fwd`
@@ -556,8 +876,12 @@ hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const flo
 static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt,
                                int rows_opt_nbuf, int rows_opt_rpw, int jt_max);
 
-bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf,
+bool make_wgrad_plan(const SepConv &fwd_in, WgradPlan &wp, bool g_allow_rows, int rows_opt_mt, int rows_opt_nbuf,
                      int rows_opt_rpw) {
+  // (the forward tiling is only borrowed for its staging geometry: plan it for the fp32 kernel)
+  SepConv fwd = fwd_in;
+  fwd.math = MATH_FP32;
+  wp.split = fwd_in.math == MATH_BF16X3;
   // narrower column blocks touch fewer input channels and so need less LDS
   for (int jt_max = 3; jt_max >= 1; --jt_max)
     if (make_wgrad_plan_jt(fwd, wp, g_allow_rows, rows_opt_mt, rows_opt_nbuf, rows_opt_rpw, jt_max)) return true;
@@ -591,6 +915,46 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
   // (rows of 5 and 7: 12 % and 25 %).  On a Mellin axis its tiles stage a virtual row per
   // (row, filter row) pair for only 128 positions and the row-wise kernel stays ahead.
   const int min_row = mellin_x ? 4 : 8;
+  if (wp.split && !pl.segment && pl.ay == 1 && pl.uy == 1 && pl.by == 1 && pl.nfy <= 8 && pl.noy >= 8 &&
+      pl.nox_eff >= 1 && g_allow_rows && (i64)pl.M * pl.Q < ((i64)1 << 30)) {
+    // The bf16 form (wgrad_stream_kernel): grad_out goes through registers, LDS holds the
+    // fragments of the input rows a unit needs.  The largest unit whose fragment tasks a
+    // workgroup's threads can hold (two each) and that still lets three workgroups share a
+    // CU, else two.  All 64 channels in one workgroup where there are that many: the input
+    // fragments are then made once for twice the products.
+    const int NG = (pl.noy + 7) / 8;
+    const int mt_s = (pl.M > 32 && rows_opt_mt != 1) ? 2 : 1;
+    const int m_groups = (pl.M + mt_s * 32 - 1) / (mt_s * 32);
+    const int ccj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
+    const int blocks_y = m_groups * wp.j_groups;
+    for (int pass = 0; pass < 2 && !wp.rows_mode; ++pass)
+      for (int rpw = rows_opt_rpw > 0 ? rows_opt_rpw : 4; rpw >= 1; --rpw) {
+        const int rb = kWaves * rpw;
+        const i64 Rr = mellin_x ? (i64)rb * pl.nfx : (i64)pl.ax * (rb - 1) + pl.bx_span + 1;
+        const i64 tasks = (i64)ccj * Rr * NG;
+        const size_t bytes = std::max((size_t)48 * (tasks * pl.nfy + 1) + 8 * (size_t)(rb * NG + 2),
+                                      4 * (size_t)mt_s * 32 * J_T);
+        if (Rr > 8192 || tasks > 2 * kThreads) continue;
+        const int cap = mt_s == 2 ? 2 : 3;                 // registers
+        if (bytes > (size_t)(pass == 0 && cap == 3 ? 52 : 78) * 1024) { if (rows_opt_rpw > 0) break; continue; }
+        const int per_cu = std::max(1, std::min((int)((160 * 1024) / (bytes + 512)), cap));
+        const i64 units = (i64)pl.batch * ((pl.nox_eff + rb - 1) / rb);
+        const i64 S = std::min<i64>(std::max<i64>(1, (256 * per_cu) / blocks_y), units);
+        wp.rows_mode = 2;
+        pl.R = (int)Rr;
+        wp.CCj = ccj;
+        wp.lds_bytes = bytes;
+        wp.nbuf = 1;
+        wp.rpw = rpw;
+        wp.mt = mt_s;
+        wp.m_groups = m_groups;
+        wp.M_pad = m_groups * mt_s * 32;
+        wp.S = (int)S;
+        wp.ws_bytes = (size_t)wp.S * wp.M_pad * wp.J_pad * sizeof(float);
+        break;
+      }
+    if (wp.rows_mode) return true;
+  }
   if (!pl.segment && pl.ay == 1 && pl.noy >= min_row && pl.nox_eff >= 1 && g_allow_rows) {
     // Row-wise variant: units of kWaves * rpw output rows, about 300 positions per
     // unit (two rows of 38 per wavefront, sixteen rows of 5).
@@ -681,7 +1045,13 @@ hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float 
                         float *grad_weight, float *workspace, hipStream_t stream) {
   dim3 grid((unsigned)wp.S, (unsigned)(wp.m_groups * wp.j_groups));
   hipError_t e = hipErrorInvalidValue;
-  if (wp.rows_mode) {
+  if (wp.rows_mode == 2) {
+#define MELLIN_STREAM_CASE(MT_, JT_)                                                       \
+  if (wp.mt == MT_ && wp.jt == JT_) e = launch_stream<MT_, JT_>(wp, grid, grad_out, input, workspace, stream);
+    MELLIN_STREAM_CASE(1, 1) MELLIN_STREAM_CASE(1, 2) MELLIN_STREAM_CASE(1, 3)
+    MELLIN_STREAM_CASE(2, 1) MELLIN_STREAM_CASE(2, 2) MELLIN_STREAM_CASE(2, 3)
+#undef MELLIN_STREAM_CASE
+  } else if (wp.rows_mode) {
 #define MELLIN_ROWS_CASE(MT_, JT_)                                                         \
   if (wp.mt == MT_ && wp.jt == JT_) e = launch_rows<MT_, JT_>(wp, grid, grad_out, input, workspace, stream);
     MELLIN_ROWS_CASE(1, 1) MELLIN_ROWS_CASE(1, 2) MELLIN_ROWS_CASE(1, 3)
