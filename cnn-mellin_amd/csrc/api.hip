@@ -295,7 +295,8 @@ int choose_input_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 n
   ips.ws_bytes = 0;
   if (forced == 1) return IN_GATHER;
   if (forced == 0 && make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
-                                     px, py, ux, uy, ips.fused) && ips.fused.ws_bytes <= kMaxWorkspaceBytes) {
+                                     px, py, ux, uy, ips.fused, 0, 0, -1, g_math) &&
+      ips.fused.ws_bytes <= kMaxWorkspaceBytes) {
     ips.ws_bytes = ips.fused.ws_bytes;
     return IN_FUSED;
   }

@@ -446,6 +446,243 @@ hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go,
   return hipGetLastError();
 }
 
+// The same input gradient on the bf16 matrix cores (tile_stage.hpp: every fp32 operand as
+// the exact sum of three bf16 parts, six products each), for layers whose taps fit one
+// 32-row tile per input channel (nf <= 32, at most three input channels).
+//
+// One workgroup of four wavefronts per (image, strip); a wavefront takes a quarter of the
+// strip's rows, 32 * NT positions at a time, and ALL input channels' taps of them:
+//   * grad_out never touches LDS.  For tap products the reduction runs over the output
+//     channels, so a lane's eight values of a step are eight channels of ONE position:
+//     eight loads whose 32 lanes read 128 consecutive bytes.  They are requested one step
+//     ahead and split in registers (every grad_out value is loaded and split once).
+//   * the filter lives in LDS as fragments, built once per workgroup.
+//   * a wavefront folds its products into a private LDS image of the grad_input rows its
+//     positions reach (no other wavefront touches it); at the end the four images are added
+//     up in wave order into the strip's image, which is written out exactly as above.
+template <int MTT, int NT>
+__global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl, const float *__restrict__ W,
+                                                              const float *__restrict__ GO,
+                                                              float *__restrict__ GI, float *__restrict__ WS) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int P = NT * 32, ROWS = MTT * 32;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, l32 = lane & 31;
+  const int n = blockIdx.x / pl.strips, strip = blockIdx.x - n * pl.strips;
+  const int ha = strip * pl.Th, hb = min(ha + pl.Th, pl.H);    // grad_out rows [ha, hb)
+  const int ksteps = (pl.c_out + 15) >> 4, kgroups = 2 * ksteps;
+  const int plane_words = pl.Rp * pl.Wp;                       // the strip's image, one input channel
+  const int Rw = pl.sx * (pl.rw - 1) + pl.dx * (pl.nfx - 1) + 1;
+  const int wplane_words = Rw * pl.Wp;                         // a wavefront's image, one input channel
+  // LDS: filter fragments [3][kgroups][ROWS] (later the strip's image [c_in][Rp][Wp] and the
+  // row table), then the wavefronts' images [4][c_in][Rw][Wp]
+  uintx4 *Af = (uintx4 *)lds;
+  const int af_part = kgroups * ROWS;
+  const int head_words = max(12 * af_part, pl.c_in * plane_words + max(pl.Rp, pl.sx * pl.Th));
+  float *wplanes = lds + ((head_words + 3) & ~3);
+  float *myplane = wplanes + wave * pl.c_in * wplane_words;
+
+  for (int i = tid; i < kWaves * pl.c_in * wplane_words; i += 256) wplanes[i] = 0.f;
+  {
+    // a thread splits the eight output channels k = 8 g .. 8 g + 7 of matrix row `row`
+    // (tap m = row % 32 of input channel row / 32)
+    const FastDiv by_rows(ROWS);
+    for (int idx = tid; idx < kgroups * ROWS; idx += 256) {
+      int g, row;
+      by_rows.divmod(idx, g, row);
+      const int ci = row >> 5, m = row & 31;
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int k = 8 * g + i;
+        x[i] = (k < pl.c_out && ci < pl.c_in && m < pl.nf) ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : 0.f;
+      }
+      store_frag(Af, kgroups, ROWS, g, row, x);
+    }
+  }
+  // accumulator register r of this lane holds tap m(r); its offset in an image (-1: no such tap)
+  int off[16];
+  {
+    const FastDiv by_nfy(pl.nfy);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = (r >> 2) * 8 + half * 4 + (r & 3);
+      int fx, fy;
+      by_nfy.divmod(m, fx, fy);
+      off[r] = m < pl.nf ? pl.dx * fx * pl.Wp + pl.dy * fy : -1;
+    }
+  }
+  // this wavefront's positions [q0, q1) of the image
+  const int r0 = min(ha + wave * pl.rw, hb), r1 = min(r0 + pl.rw, hb);
+  const int q0 = r0 * pl.nhy, q1 = r1 * pl.nhy;
+  const int n_it = (q1 - q0 + P - 1) / P;
+  const int total = n_it * ksteps;
+  const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
+  const FastDiv by_nhy(pl.nhy);
+
+  // step st = (iteration, 16 output channels): this lane's eight channels of NT positions
+  struct BOp { float v[NT][8]; };
+  auto load_b = [&](int st, BOp &o) {
+    const int it = st / ksteps, ks = st - it * ksteps;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int q = min(q0 + it * P + t * 32 + l32, q1 - 1);   // past the range: any valid position, never folded
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int k = min(16 * ks + 8 * half + i, pl.c_out - 1);   // past c_out: the filter fragment is zero
+        o.v[t][i] = GOn[(i64)k * pl.nh + q];
+      }
+    }
+  };
+  floatx16 acc[MTT][NT];
+  auto compute = [&](int st, const BOp &o) {
+    const int it = st / ksteps, ks = st - it * ksteps;
+    if (ks == 0) {
+#pragma unroll
+      for (int a = 0; a < MTT; ++a)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
+    }
+    uintx4 bh[NT], bm[NT], bl[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
+    const int g = 2 * ks + half;
+#pragma unroll
+    for (int a = 0; a < MTT; ++a) {
+      const uintx4 ah = Af[g * ROWS + a * 32 + l32], am = Af[af_part + g * ROWS + a * 32 + l32],
+                   al = Af[2 * af_part + g * ROWS + a * 32 + l32];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
+    }
+    if (ks == ksteps - 1) {
+      // fold: Z[tap, position] joins word base(position) + off(tap) of the input channel's image
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int rel = it * P + t * 32 + l32;              // position counted from q0
+        if (q0 + rel < q1) {
+          int hxr, hy;
+          by_nhy.divmod(rel, hxr, hy);
+          float *dst = myplane + pl.sx * hxr * pl.Wp + pl.sy * hy;
+#pragma unroll
+          for (int a = 0; a < MTT; ++a) {
+            if (a < pl.c_in) {
+#pragma unroll
+              for (int c4 = 0; c4 < 4; ++c4) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  if (off[4 * j + c4] >= 0) v[j] = dst[a * wplane_words + off[4 * j + c4]];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  if (off[4 * j + c4] >= 0) dst[a * wplane_words + off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
+              }
+            }
+          }
+        }
+      }
+    }
+  };
+  __syncthreads();                                       // fragments and zeros are in place
+  {
+    BOp b0, b1;
+    if (total > 0) load_b(0, b0);
+    for (int st = 0; st < total; st += 2) {
+      if (st + 1 < total) load_b(st + 1, b1);
+      compute(st, b0);
+      if (st + 1 >= total) break;
+      if (st + 2 < total) load_b(st + 2, b0);
+      compute(st + 1, b1);
+    }
+  }
+  __syncthreads();                                       // every wavefront's image is complete; the fragments are free
+
+  // the strip's image: row i = grad_input row g0 + i; wavefront w's image starts at row sx * w * rw
+  float *planes = lds;
+  const FastDiv by_plane(plane_words), by_wp(pl.Wp);
+  for (int i = tid; i < pl.c_in * plane_words; i += 256) {
+    int cc, rem, row, col;
+    by_plane.divmod(i, cc, rem);
+    by_wp.divmod(rem, row, col);
+    float v = 0.f;
+    for (int w = 0; w < kWaves; ++w) {
+      const int wr = row - pl.sx * w * pl.rw;
+      if (wr >= 0 && wr < Rw) v += wplanes[(w * pl.c_in + cc) * wplane_words + wr * pl.Wp + col];
+    }
+    planes[i] = v;
+  }
+  const int g0 = pl.sx * ha - pl.px;
+  const int rp_t = max(pl.Rp, pl.sx * pl.Th);
+  int *row_dst = (int *)(planes + pl.c_in * plane_words);
+  const StripMap map(pl);
+  for (int pi = tid; pi < rp_t; pi += 256) {
+    const int gx = g0 + pi;
+    int code = -1;
+    if (gx >= 0 && gx < pl.ngx) {
+      int s_lo, s_hi;
+      map.feeding(gx, s_lo, s_hi);
+      if (s_lo == s_hi) {
+        if (s_lo == strip) code = 2 * gx;
+      } else if (strip == s_lo || strip == s_hi) {
+        const int r = gx - (pl.sx * s_hi * pl.Th - pl.px);
+        code = 2 * (((s_hi - 1) * pl.nshared + r) * 2 + (strip - s_lo)) + 1;
+      }
+    }
+    row_dst[pi] = code;
+  }
+  __syncthreads();
+  {
+    const int row_words = rp_t * pl.ngy;
+    const FastDiv by_ngy(pl.ngy), by_rp(rp_t);
+    const i64 nc0 = (i64)n * pl.c_in;
+    for (int i = tid; i < pl.c_in * row_words; i += 256) {
+      int r2, gy, cc, pi;
+      by_ngy.divmod(i, r2, gy);
+      by_rp.divmod(r2, cc, pi);
+      const int code = row_dst[pi];
+      if (code < 0) continue;
+      float v = 0.f;
+      if (pi < pl.Rp && gy + pl.py < pl.Wp) v = planes[cc * plane_words + pi * pl.Wp + pl.py + gy];
+      if (code & 1)
+        WS[((nc0 + cc) * (pl.strips - 1) * pl.nshared * 2 + (code >> 1)) * pl.ngy + gy] = v;
+      else
+        GI[((nc0 + cc) * pl.ngx + (code >> 1)) * pl.ngy + gy] = v;
+    }
+  }
+  // grad_input rows past the reach of the last grad_out row belong to the last strip: zeros
+  if (strip == pl.strips - 1) {
+    const int z0 = max(0, g0 + rp_t);
+    const int zrows = pl.ngx - z0;
+    if (zrows > 0) {
+      const i64 per_c = (i64)zrows * pl.ngy;
+      for (i64 i = tid; i < pl.c_in * per_c; i += 256) {
+        const i64 cc = i / per_c, w = i - cc * per_c;
+        GI[(((i64)n * pl.c_in + cc) * pl.ngx + z0) * pl.ngy + w] = 0.f;
+      }
+    }
+  }
+}
+
+template <int MTT, int NT>
+hipError_t launch_stream_instance(const IgradPlan &pl, const float *w, const float *go, float *gi,
+                                  float *ws, hipStream_t stream) {
+  auto kern = igrad_stream_kernel<MTT, NT>;
+  if (pl.lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)pl.lds_bytes);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(pl.batch * pl.strips)), dim3(256), pl.lds_bytes, stream, pl, w, go, gi,
+                     ws);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || pl.ws_bytes == 0) return e;
+  hipLaunchKernelGGL(igrad_combine_kernel,
+                     dim3((unsigned)(pl.strips - 1), (unsigned)(pl.batch * pl.c_in)), dim3(256), 0,
+                     stream, pl, ws, gi);
+  return hipGetLastError();
+}
+
 // Tap products for the gather-fold input gradient (any x axis kind):
 //   Z[n, ci, m, q] = sum_co w[co, ci, m] * grad_out[n, co, q]
 // Same operands, staging and work split over wavefronts as above; the
@@ -614,7 +851,7 @@ hipError_t launch_tap_product(const TapProductPlan &pl, const float *weight, con
 
 bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                      i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
-                     i64 ux, i64 uy, IgradPlan &pl, int force_nt, int force_Th, int force_pipe) {
+                     i64 ux, i64 uy, IgradPlan &pl, int force_nt, int force_Th, int force_pipe, int math) {
   if (kind_x != AX_LCORR || ux != 1 || uy != 1) return false;
   if (px < 0 || py < 0) return false;
   const i64 nf = nfx * nfy, nh = nhx * nhy, ng = ngx * ngy;
@@ -665,6 +902,41 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
   i64 Th = std::max<i64>((H + want_strips - 1) / want_strips, std::max<i64>(min_th, 2));
   if (force_Th > 0) Th = std::max<i64>(force_Th, min_th);
   Th = std::min(Th, std::max(H, min_th));
+  pl.stream = 0;
+  pl.rw = 0;
+  if (math == MATH_BF16X3 && mtn == 1 && c_in <= 3 && pl.batched_fold && force_nt == 0 && force_Th == 0 &&
+      force_pipe != 0 && ngx + px + reach + sx < ((i64)1 << 22) && batch * c_in <= 65535 &&
+      (reach - sx + 1) * ngy < ((i64)1 << 22)) {
+    // The bf16 form (igrad_stream_kernel): four wavefronts per (image, strip), rw rows each.
+    // Pick rw for the fewest rounds of workgroups times 64-position passes per wavefront.
+    const i64 kgroups = 2 * ((c_out + 15) / 16), rows = c_in * 32;
+    double best = 0;
+    for (i64 rw = 1; rw <= 32; ++rw) {
+      const i64 Th_s = 4 * rw;
+      if (Th_s < std::max<i64>(min_th, 2)) continue;
+      const i64 Rw = sx * (rw - 1) + reach + 1, Rp = sx * (Th_s - 1) + reach + 1;
+      if ((Th_s + 2) * nhy >= ((i64)1 << 22) || c_in * std::max(Rp, sx * Th_s) * ngy >= ((i64)1 << 22)) break;
+      const i64 head = std::max<i64>(12 * kgroups * rows, c_in * Rp * Wp + std::max(Rp, sx * Th_s));
+      const size_t lds = 4 * (size_t)(((head + 3) & ~(i64)3) + 4 * c_in * Rw * Wp);
+      if (lds > 150 * 1024) break;
+      const i64 per_cu = lds + 512 <= 80 * 1024 ? 2 : 1;
+      const i64 strips = (H + Th_s - 1) / Th_s, wgs = batch * strips;
+      const i64 rounds = (wgs + 256 * per_cu - 1) / (256 * per_cu), passes = (rw * nhy + 63) / 64;
+      // (a workgroup alone on its CU runs at about 0.6 of the rate of two)
+      const double rate = (double)(batch * H * nhy) / ((double)rounds * passes * (per_cu == 2 ? 1.0 : 1.2));
+      if (rate > best * 1.02) {
+        best = rate;
+        pl.stream = 1; pl.rw = (int)rw; pl.nt = 2; pl.jobs = 1;
+        pl.Th = (int)Th_s; pl.H = (int)H; pl.strips = (int)strips;
+        pl.Rp = (int)Rp; pl.Wp = (int)Wp; pl.lds_bytes = lds;
+        pl.nshared = (int)std::max<i64>(0, reach - sx + 1);
+        pl.ws_bytes = pl.strips > 1 && pl.nshared > 0
+                          ? 4 * (size_t)batch * c_in * (pl.strips - 1) * pl.nshared * 2 * ngy : 0;
+      }
+    }
+    if (pl.stream && (i64)pl.batch * pl.strips < ((i64)1 << 31)) return true;
+    pl.stream = 0;
+  }
   // jobs per workgroup: make the wavefront count a multiple of four when that fits
   const int max_waves = pl.ksteps == 64 ? 8 : 12;      // registers: see the launch bounds
   pl.jobs = 1;
@@ -699,6 +971,11 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
 
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
                         float *grad_input, float *workspace, hipStream_t stream) {
+  if (pl.stream) {
+    if (pl.c_in == 1) return launch_stream_instance<1, 2>(pl, weight, grad_out, grad_input, workspace, stream);
+    if (pl.c_in == 2) return launch_stream_instance<2, 2>(pl, weight, grad_out, grad_input, workspace, stream);
+    return launch_stream_instance<3, 2>(pl, weight, grad_out, grad_input, workspace, stream);
+  }
   // the pipelined fold needs batches that cannot collide and no padded matrix rows
   const bool pipe = pl.pipe && pl.nt == 2;
 #define MELLIN_IGRAD_CASE(KS, NT_)                                                       \

@@ -26,6 +26,8 @@ struct IgradPlan {
   int Rp, Wp;                      // accumulator plane: rows and row length (words)
   int pipe;                        // streaming variant (fold overlapped with the multiplies)
   int batched_fold;                // taps with congruent matrix rows never share a word: fold them in batches
+  int stream;                      // the bf16 form: four wavefronts per strip, grad_out through registers
+  int rw;                          // stream: grad_out rows per wavefront (Th = 4 * rw)
   size_t lds_bytes, ws_bytes;      // ws: partial rows at the strip boundaries
 };
 
@@ -35,7 +37,8 @@ struct IgradPlan {
 // too many channels, planes that do not fit in LDS, sizes beyond 32-bit indexing).
 bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                      i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py,
-                     i64 ux, i64 uy, IgradPlan &pl, int force_nt = 0, int force_Th = 0, int force_pipe = -1);
+                     i64 ux, i64 uy, IgradPlan &pl, int force_nt = 0, int force_Th = 0, int force_pipe = -1,
+                     int math = MATH_FP32);
 
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
                         float *grad_input, float *workspace, hipStream_t stream);
