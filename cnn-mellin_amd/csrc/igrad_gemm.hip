@@ -509,7 +509,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       const int m = (r >> 2) * 8 + half * 4 + (r & 3);
       int fx, fy;
       by_nfy.divmod(m, fx, fy);
-      off[r] = m < pl.nf ? pl.dx * fx * pl.Wp + pl.dy * fy : -1;
+      off[r] = pl.dx * fx * pl.Wp + pl.dy * fy;             // (registers of taps past nf are never folded)
     }
   }
   // this wavefront's positions [q0, q1) of the image
@@ -520,21 +520,34 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
   const FastDiv by_nhy(pl.nhy);
 
-  // step st = (iteration, 16 output channels): this lane's eight channels of NT positions
+  // step st = (iteration, 16 output channels): this lane's eight channels of NT positions.
+  // Addresses are 32-bit byte offsets from the image's grad_out (the plan keeps c_out * nh
+  // * 4 below 2^31): one add per load, no 64-bit arithmetic in the loop.
   struct BOp { float v[NT][8]; };
+  // Buffer loads: a lane's byte offset within the image's grad_out is fixed for a tile
+  // (position, and which eight of a step's channels), the channel's offset is wave-uniform
+  // and travels in a scalar register, so a load costs no vector arithmetic; offsets past
+  // the image's c_out * nh words (a last step reaching past c_out) read zeros.
+  const __amdgpu_buffer_rsrc_t go_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)GOn, 0, pl.c_out * pl.nh * 4, 0x00020000);
+  const int nh4 = pl.nh * 4;
   auto load_b = [&](int st, BOp &o) {
     const int it = st / ksteps, ks = st - it * ksteps;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int q = min(q0 + it * P + t * 32 + l32, q1 - 1);   // past the range: any valid position, never folded
+      const int voff = q * 4 + 8 * half * nh4;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = min(16 * ks + 8 * half + i, pl.c_out - 1);   // past c_out: the filter fragment is zero
-        o.v[t][i] = GOn[(i64)k * pl.nh + q];
-      }
+      for (int i = 0; i < 8; ++i)
+        o.v[t][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(go_rsrc, voff, (16 * ks + i) * nh4, 0));
     }
   };
   floatx16 acc[MTT][NT];
+  // taps 4 j .. 4 j + 3 of a lane (registers r = 4 j + c) are filter columns fy0 + c of one filter
+  // row when nfy is a multiple of 4; with dy = 1 they are four consecutive words of the image,
+  // reached with immediate offsets from the first
+  const bool quad = (pl.nfy & 3) == 0 && pl.dy == 1;
+  const int jmax = pl.nf >> 3;                              // (the plan keeps nf a multiple of 8) live register quads
   auto compute = [&](int st, const BOp &o) {
     const int it = st / ksteps, ks = st - it * ksteps;
     if (ks == 0) {
@@ -548,11 +561,10 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     uintx4 bh[NT], bm[NT], bl[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
-    const int g = 2 * ks + half;
+    const uintx4 *af = Af + (2 * ks + half) * ROWS + l32;
 #pragma unroll
     for (int a = 0; a < MTT; ++a) {
-      const uintx4 ah = Af[g * ROWS + a * 32 + l32], am = Af[af_part + g * ROWS + a * 32 + l32],
-                   al = Af[2 * af_part + g * ROWS + a * 32 + l32];
+      const uintx4 ah = af[a * 32], am = af[af_part + a * 32], al = af[2 * af_part + a * 32];
 #pragma unroll
       for (int t = 0; t < NT; ++t) mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
     }
@@ -567,16 +579,33 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
           float *dst = myplane + pl.sx * hxr * pl.Wp + pl.sy * hy;
 #pragma unroll
           for (int a = 0; a < MTT; ++a) {
-            if (a < pl.c_in) {
+            float *pa = dst + a * wplane_words;
+            if (quad) {
+              // (one filter column at a time, as below: neighbouring positions share words across
+              // columns; the four columns of a filter row sit at fixed distances from the first)
+              float *pj[4];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) pj[j] = pa + off[4 * j];
 #pragma unroll
               for (int c4 = 0; c4 < 4; ++c4) {
                 float v[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                  if (off[4 * j + c4] >= 0) v[j] = dst[a * wplane_words + off[4 * j + c4]];
+                  if (j < jmax) v[j] = pj[j][c4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                  if (off[4 * j + c4] >= 0) dst[a * wplane_words + off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
+                  if (j < jmax) pj[j][c4] = v[j] + acc[a][t][4 * j + c4];
+              }
+            } else {
+#pragma unroll
+              for (int c4 = 0; c4 < 4; ++c4) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  if (j < jmax) v[j] = pa[off[4 * j + c4]];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  if (j < jmax) pa[off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
               }
             }
           }
@@ -904,7 +933,8 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
   Th = std::min(Th, std::max(H, min_th));
   pl.stream = 0;
   pl.rw = 0;
-  if (math == MATH_BF16X3 && mtn == 1 && c_in <= 3 && pl.batched_fold && force_nt == 0 && force_Th == 0 &&
+  if (math == MATH_BF16X3 && mtn == 1 && c_in <= 3 && (nf & 7) == 0 && c_out * nh < ((i64)1 << 29) &&
+      pl.batched_fold && force_nt == 0 && force_Th == 0 &&
       force_pipe != 0 && ngx + px + reach + sx < ((i64)1 << 22) && batch * c_in <= 65535 &&
       (reach - sx + 1) * ngy < ((i64)1 << 22)) {
     // The bf16 form (igrad_stream_kernel): four wavefronts per (image, strip), rw rows each.
