@@ -467,18 +467,31 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   extern __shared__ __align__(16) float lds[];
   constexpr int P = NT * 32, ROWS = MTT * 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef EXP_STAMP
+  long long stamp[8]; int nstamp = 0;
+#define STAMP() stamp[nstamp++] = __builtin_readcyclecounter()
+#else
+#define STAMP()
+#endif
+  STAMP();
   const int half = lane >> 5, l32 = lane & 31;
   const int n = blockIdx.x / pl.strips, strip = blockIdx.x - n * pl.strips;
   const int ha = strip * pl.Th, hb = min(ha + pl.Th, pl.H);    // grad_out rows [ha, hb)
-  const int ksteps = (pl.c_out + 15) >> 4, kgroups = 2 * ksteps;
+  // steps of 16 output channels, an even number of them (the two operand buffers alternate;
+  // a step past c_out reads zeros on both sides)
+  const int ksteps = ((pl.c_out + 31) >> 5) * 2, kgroups = 2 * ksteps;
   const int plane_words = pl.Rp * pl.Wp;                       // the strip's image, one input channel
+  // (a wavefront's image has rows for all 32 matrix rows of a tile, also those past the last
+  // tap: their products are exact zeros and are folded like the others, which keeps the
+  // fold free of conditions)
   const int Rw = pl.sx * (pl.rw - 1) + pl.dx * (pl.nfx - 1) + 1;
-  const int wplane_words = Rw * pl.Wp;                         // a wavefront's image, one input channel
+  const int Rw_alloc = pl.sx * (pl.rw - 1) + pl.dx * (31 / pl.nfy) + 1;
+  const int wplane_words = Rw_alloc * pl.Wp;                   // a wavefront's image, one input channel
   // LDS: filter fragments [3][kgroups][ROWS] (later the strip's image [c_in][Rp][Wp] and the
   // row table), then the wavefronts' images [4][c_in][Rw][Wp]
   uintx4 *Af = (uintx4 *)lds;
   const int af_part = kgroups * ROWS;
-  const int head_words = max(12 * af_part, pl.c_in * plane_words + max(pl.Rp, pl.sx * pl.Th));
+  const int head_words = max(12 * af_part, max(pl.Rp, pl.sx * pl.Th));
   float *wplanes = lds + ((head_words + 3) & ~3);
   float *myplane = wplanes + wave * pl.c_in * wplane_words;
 
@@ -487,17 +500,29 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     // a thread splits the eight output channels k = 8 g .. 8 g + 7 of matrix row `row`
     // (tap m = row % 32 of input channel row / 32)
     const FastDiv by_rows(ROWS);
-    for (int idx = tid; idx < kgroups * ROWS; idx += 256) {
-      int g, row;
-      by_rows.divmod(idx, g, row);
-      const int ci = row >> 5, m = row & 31;
-      float x[8];
+    for (int idx0 = tid; idx0 < kgroups * ROWS; idx0 += 4 * 256) {
+      // four tasks at a time: all their loads are requested before the first is split
+      float x[4][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = 8 * g + i;
-        x[i] = (k < pl.c_out && ci < pl.c_in && m < pl.nf) ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : 0.f;
+      for (int u = 0; u < 4; ++u) {
+        const int idx = idx0 + u * 256;
+        int g, row;
+        by_rows.divmod(idx, g, row);
+        const int ci = row >> 5, m = row & 31;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int k = 8 * g + i;
+          x[u][i] = (idx < kgroups * ROWS && k < pl.c_out && ci < pl.c_in && m < pl.nf)
+                        ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : 0.f;
+        }
       }
-      store_frag(Af, kgroups, ROWS, g, row, x);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = idx0 + u * 256;
+        int g, row;
+        by_rows.divmod(idx, g, row);
+        if (idx < kgroups * ROWS) store_frag(Af, kgroups, ROWS, g, row, x[u]);
+      }
     }
   }
   // accumulator register r of this lane holds tap m(r); its offset in an image (-1: no such tap)
@@ -509,7 +534,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       const int m = (r >> 2) * 8 + half * 4 + (r & 3);
       int fx, fy;
       by_nfy.divmod(m, fx, fy);
-      off[r] = pl.dx * fx * pl.Wp + pl.dy * fy;             // (registers of taps past nf are never folded)
+      off[r] = pl.dx * fx * pl.Wp + pl.dy * fy;             // (also for rows past the last tap: see Rw_alloc)
     }
   }
   // this wavefront's positions [q0, q1) of the image
@@ -531,15 +556,18 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   const __amdgpu_buffer_rsrc_t go_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)GOn, 0, pl.c_out * pl.nh * 4, 0x00020000);
   const int nh4 = pl.nh * 4;
-  auto load_b = [&](int st, BOp &o) {
-    const int it = st / ksteps, ks = st - it * ksteps;
+  auto load_b = [&](int it, int ks, BOp &o) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int q = min(q0 + it * P + t * 32 + l32, q1 - 1);   // past the range: any valid position, never folded
       const int voff = q * 4 + 8 * half * nh4;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
+#ifdef EXP_NO_LOAD
+        o.v[t][i] = __int_as_float(voff + i + ks);
+#else
         o.v[t][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(go_rsrc, voff, (16 * ks + i) * nh4, 0));
+#endif
     }
   };
   floatx16 acc[MTT][NT];
@@ -547,28 +575,42 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   // row when nfy is a multiple of 4; with dy = 1 they are four consecutive words of the image,
   // reached with immediate offsets from the first
   const bool quad = (pl.nfy & 3) == 0 && pl.dy == 1;
-  const int jmax = pl.nf >> 3;                              // (the plan keeps nf a multiple of 8) live register quads
-  auto compute = [&](int st, const BOp &o) {
-    const int it = st / ksteps, ks = st - it * ksteps;
-    if (ks == 0) {
-#pragma unroll
-      for (int a = 0; a < MTT; ++a)
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
-    }
+  auto multiply = [&](auto first_tag, int ks, const BOp &o) {
+    constexpr bool kFirst = decltype(first_tag)::value;      // an iteration's first step starts the sums from zero
     uintx4 bh[NT], bm[NT], bl[NT];
 #pragma unroll
+#ifdef EXP_NO_SPLIT
+    for (int t = 0; t < NT; ++t) {
+      bh[t] = uintx4{__float_as_uint(o.v[t][0]), __float_as_uint(o.v[t][1]), __float_as_uint(o.v[t][2]), __float_as_uint(o.v[t][3])};
+      bm[t] = uintx4{__float_as_uint(o.v[t][4]), __float_as_uint(o.v[t][5]), __float_as_uint(o.v[t][6]), __float_as_uint(o.v[t][7])};
+      bl[t] = bh[t] ^ bm[t];
+    }
+#else
     for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
+#endif
     const uintx4 *af = Af + (2 * ks + half) * ROWS + l32;
 #pragma unroll
     for (int a = 0; a < MTT; ++a) {
       const uintx4 ah = af[a * 32], am = af[af_part + a * 32], al = af[2 * af_part + a * 32];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
+      for (int t = 0; t < NT; ++t) {
+        if (kFirst) {
+          const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          acc[a][t] = zero16;
+        }
+#ifdef EXP_ONE_MFMA
+        acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ah ^ am ^ al), as_bf16x8(bh[t] ^ bm[t] ^ bl[t]), acc[a][t], 0, 0, 0);
+#else
+        mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
+#endif
+      }
     }
-    if (ks == ksteps - 1) {
+  };
+  auto fold_tiles = [&](int it) {
+#ifdef EXP_NO_FOLD
+    if (it != 0) return;
+#endif
+    {
       // fold: Z[tap, position] joins word base(position) + off(tap) of the input channel's image
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -590,22 +632,18 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
               for (int c4 = 0; c4 < 4; ++c4) {
                 float v[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                  if (j < jmax) v[j] = pj[j][c4];
+                for (int j = 0; j < 4; ++j) v[j] = pj[j][c4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                  if (j < jmax) pj[j][c4] = v[j] + acc[a][t][4 * j + c4];
+                for (int j = 0; j < 4; ++j) pj[j][c4] = v[j] + acc[a][t][4 * j + c4];
               }
             } else {
 #pragma unroll
               for (int c4 = 0; c4 < 4; ++c4) {
                 float v[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                  if (j < jmax) v[j] = pa[off[4 * j + c4]];
+                for (int j = 0; j < 4; ++j) v[j] = pa[off[4 * j + c4]];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                  if (j < jmax) pa[off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
+                for (int j = 0; j < 4; ++j) pa[off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
               }
             }
           }
@@ -613,37 +651,37 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       }
     }
   };
+  STAMP();
   __syncthreads();                                       // fragments and zeros are in place
+  STAMP();
   {
+    // two operand buffers alternate; the loads of a step are requested one step ahead
     BOp b0, b1;
-    if (total > 0) load_b(0, b0);
-    for (int st = 0; st < total; st += 2) {
-      if (st + 1 < total) load_b(st + 1, b1);
-      compute(st, b0);
-      if (st + 1 >= total) break;
-      if (st + 2 < total) load_b(st + 2, b0);
-      compute(st + 1, b1);
+    if (n_it > 0) load_b(0, 0, b0);
+    for (int it = 0; it < n_it; ++it) {
+      load_b(it, 1, b1);
+      multiply(std::true_type(), 0, b0);
+      for (int ks = 1; ks + 1 < ksteps; ks += 2) {
+        load_b(it, ks + 1, b0);
+        multiply(std::false_type(), ks, b1);
+        load_b(it, ks + 2, b1);
+        multiply(std::false_type(), ks + 1, b0);
+      }
+      if (it + 1 < n_it) load_b(it + 1, 0, b0);
+      multiply(std::false_type(), ksteps - 1, b1);
+      fold_tiles(it);
     }
   }
+  STAMP();
   __syncthreads();                                       // every wavefront's image is complete; the fragments are free
+  STAMP();
 
-  // the strip's image: row i = grad_input row g0 + i; wavefront w's image starts at row sx * w * rw
-  float *planes = lds;
-  const FastDiv by_plane(plane_words), by_wp(pl.Wp);
-  for (int i = tid; i < pl.c_in * plane_words; i += 256) {
-    int cc, rem, row, col;
-    by_plane.divmod(i, cc, rem);
-    by_wp.divmod(rem, row, col);
-    float v = 0.f;
-    for (int w = 0; w < kWaves; ++w) {
-      const int wr = row - pl.sx * w * pl.rw;
-      if (wr >= 0 && wr < Rw) v += wplanes[(w * pl.c_in + cc) * wplane_words + wr * pl.Wp + col];
-    }
-    planes[i] = v;
-  }
+  // Where the rows of the strip's image go: row i is grad_input row g0 + i.  -1 nowhere
+  // (another strip owns it, or it lies outside grad_input), 2 gx straight to grad_input,
+  // 2 (slot index) + 1 a partial row in the workspace.
   const int g0 = pl.sx * ha - pl.px;
   const int rp_t = max(pl.Rp, pl.sx * pl.Th);
-  int *row_dst = (int *)(planes + pl.c_in * plane_words);
+  int *row_dst = (int *)lds;
   const StripMap map(pl);
   for (int pi = tid; pi < rp_t; pi += 256) {
     const int gx = g0 + pi;
@@ -661,23 +699,41 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     row_dst[pi] = code;
   }
   __syncthreads();
+  // A wavefront takes rows wave, wave + 4, ... of every input channel, its lanes the columns:
+  // the row is the sum, in wave order, of the wavefronts' images that reach it (wavefront
+  // w's image starts at row sx * w * rw), written where the row's code says.
   {
-    const int row_words = rp_t * pl.ngy;
-    const FastDiv by_ngy(pl.ngy), by_rp(rp_t);
     const i64 nc0 = (i64)n * pl.c_in;
-    for (int i = tid; i < pl.c_in * row_words; i += 256) {
-      int r2, gy, cc, pi;
-      by_ngy.divmod(i, r2, gy);
-      by_rp.divmod(r2, cc, pi);
-      const int code = row_dst[pi];
-      if (code < 0) continue;
+    auto row_sum = [&](int cc, int pi, int gy) {
       float v = 0.f;
-      if (pi < pl.Rp && gy + pl.py < pl.Wp) v = planes[cc * plane_words + pi * pl.Wp + pl.py + gy];
-      if (code & 1)
-        WS[((nc0 + cc) * (pl.strips - 1) * pl.nshared * 2 + (code >> 1)) * pl.ngy + gy] = v;
-      else
-        GI[((nc0 + cc) * pl.ngx + (code >> 1)) * pl.ngy + gy] = v;
-    }
+      if (pi < pl.Rp && gy + pl.py < pl.Wp) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+          const int wr = pi - pl.sx * w * pl.rw;
+          if (wr >= 0 && wr < Rw) v += wplanes[(w * pl.c_in + cc) * wplane_words + wr * pl.Wp + pl.py + gy];
+        }
+      }
+      return v;
+    };
+    auto row_out = [&](int cc, int code) {
+      return (code & 1) ? WS + ((nc0 + cc) * (pl.strips - 1) * pl.nshared * 2 + (code >> 1)) * pl.ngy
+                        : GI + ((nc0 + cc) * pl.ngx + (code >> 1)) * pl.ngy;
+    };
+    for (int cc = 0; cc < pl.c_in; ++cc)
+      for (int pi = wave; pi < rp_t; pi += 4 * kWaves) {
+        // four rows per trip, so that their LDS reads are in flight together
+        int code[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) code[u] = pi + u * kWaves < rp_t ? row_dst[pi + u * kWaves] : -1;
+        for (int gy = lane; gy < pl.ngy; gy += 64) {
+          float v[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[u] = code[u] >= 0 ? row_sum(cc, pi + u * kWaves, gy) : 0.f;
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (code[u] >= 0) row_out(cc, code[u])[gy] = v[u];
+        }
+      }
   }
   // grad_input rows past the reach of the last grad_out row belong to the last strip: zeros
   if (strip == pl.strips - 1) {
@@ -691,6 +747,12 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       }
     }
   }
+  STAMP();
+#ifdef EXP_STAMP
+  if ((blockIdx.x == 100 || blockIdx.x == 300) && lane == 0)
+    printf("blk %d wave %d n_it %d: prologue %lld barrier %lld main %lld barrier %lld epilogue %lld\n", (int)blockIdx.x, wave, n_it,
+           stamp[1] - stamp[0], stamp[2] - stamp[1], stamp[3] - stamp[2], stamp[4] - stamp[3], stamp[5] - stamp[4]);
+#endif
 }
 
 template <int MTT, int NT>
@@ -939,24 +1001,27 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
       (reach - sx + 1) * ngy < ((i64)1 << 22)) {
     // The bf16 form (igrad_stream_kernel): four wavefronts per (image, strip), rw rows each.
     // Pick rw for the fewest rounds of workgroups times 64-position passes per wavefront.
-    const i64 kgroups = 2 * ((c_out + 15) / 16), rows = c_in * 32;
+    const i64 kgroups = 4 * ((c_out + 31) / 32), rows = c_in * 32;
     double best = 0;
     for (i64 rw = 1; rw <= 32; ++rw) {
       const i64 Th_s = 4 * rw;
       if (Th_s < std::max<i64>(min_th, 2)) continue;
       const i64 Rw = sx * (rw - 1) + reach + 1, Rp = sx * (Th_s - 1) + reach + 1;
       if ((Th_s + 2) * nhy >= ((i64)1 << 22) || c_in * std::max(Rp, sx * Th_s) * ngy >= ((i64)1 << 22)) break;
-      const i64 head = std::max<i64>(12 * kgroups * rows, c_in * Rp * Wp + std::max(Rp, sx * Th_s));
-      const size_t lds = 4 * (size_t)(((head + 3) & ~(i64)3) + 4 * c_in * Rw * Wp);
+      const i64 head = std::max<i64>(12 * kgroups * rows, std::max(Rp, sx * Th_s));
+      const i64 Rw_alloc = sx * (rw - 1) + dx * (31 / nfy) + 1;     // rows for all 32 matrix rows of a tile
+      const size_t lds = 4 * (size_t)(((head + 3) & ~(i64)3) + 4 * c_in * Rw_alloc * Wp);
       if (lds > 150 * 1024) break;
       const i64 per_cu = lds + 512 <= 80 * 1024 ? 2 : 1;
       const i64 strips = (H + Th_s - 1) / Th_s, wgs = batch * strips;
-      const i64 rounds = (wgs + 256 * per_cu - 1) / (256 * per_cu), passes = (rw * nhy + 63) / 64;
+      const i64 tile = c_in == 1 ? 64 : 32;                       // positions per pass (registers)
+      const i64 rounds = (wgs + 256 * per_cu - 1) / (256 * per_cu), passes = (rw * nhy + tile - 1) / tile * tile / 32;
       // (a workgroup alone on its CU runs at about 0.6 of the rate of two)
-      const double rate = (double)(batch * H * nhy) / ((double)rounds * passes * (per_cu == 2 ? 1.0 : 1.2));
+      // (setting up and writing out cost a workgroup about as much as two passes)
+      const double rate = (double)(batch * H * nhy) / ((double)rounds * (passes + 2) * (per_cu == 2 ? 1.0 : 1.2));
       if (rate > best * 1.02) {
         best = rate;
-        pl.stream = 1; pl.rw = (int)rw; pl.nt = 2; pl.jobs = 1;
+        pl.stream = 1; pl.rw = (int)rw; pl.nt = c_in == 1 ? 2 : 1; pl.jobs = 1;
         pl.Th = (int)Th_s; pl.H = (int)H; pl.strips = (int)strips;
         pl.Rp = (int)Rp; pl.Wp = (int)Wp; pl.lds_bytes = lds;
         pl.nshared = (int)std::max<i64>(0, reach - sx + 1);
@@ -1003,8 +1068,8 @@ hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *g
                         float *grad_input, float *workspace, hipStream_t stream) {
   if (pl.stream) {
     if (pl.c_in == 1) return launch_stream_instance<1, 2>(pl, weight, grad_out, grad_input, workspace, stream);
-    if (pl.c_in == 2) return launch_stream_instance<2, 2>(pl, weight, grad_out, grad_input, workspace, stream);
-    return launch_stream_instance<3, 2>(pl, weight, grad_out, grad_input, workspace, stream);
+    if (pl.c_in == 2) return launch_stream_instance<2, 1>(pl, weight, grad_out, grad_input, workspace, stream);
+    return launch_stream_instance<3, 1>(pl, weight, grad_out, grad_input, workspace, stream);
   }
   // the pipelined fold needs batches that cannot collide and no padded matrix rows
   const bool pipe = pl.pipe && pl.nt == 2;
