@@ -676,62 +676,83 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   __syncthreads();                                       // every wavefront's image is complete; the fragments are free
   STAMP();
 
-  // Where the rows of the strip's image go: row i is grad_input row g0 + i.  -1 nowhere
-  // (another strip owns it, or it lies outside grad_input), 2 gx straight to grad_input,
-  // 2 (slot index) + 1 a partial row in the workspace.
+  // Write-out.  Row i of the strip's image is grad_input row g0 + i: the sum, in wave order,
+  // of the rows of the wavefronts' images that reach it (wavefront w's image starts at row
+  // sx * w * rw).  One thread per row first works out everything about the row: where it
+  // goes (-1 nowhere: another strip owns it, or it lies outside grad_input; 0 straight to
+  // grad_input; 1 a partial row in the workspace, upper strip's share first) at which word
+  // of the image's grad_input or workspace slice, which wavefronts' images reach it and
+  // where their rows lie.  Then a wavefront takes rows wave, wave + 4, ... of every input
+  // channel with its lanes on the columns, and everything wave-uniform comes from the table.
   const int g0 = pl.sx * ha - pl.px;
   const int rp_t = max(pl.Rp, pl.sx * pl.Th);
-  int *row_dst = (int *)lds;
-  const StripMap map(pl);
-  for (int pi = tid; pi < rp_t; pi += 256) {
-    const int gx = g0 + pi;
-    int code = -1;
-    if (gx >= 0 && gx < pl.ngx) {
-      int s_lo, s_hi;
-      map.feeding(gx, s_lo, s_hi);
-      if (s_lo == s_hi) {
-        if (s_lo == strip) code = 2 * gx;
-      } else if (strip == s_lo || strip == s_hi) {
-        const int r = gx - (pl.sx * s_hi * pl.Th - pl.px);
-        code = 2 * (((s_hi - 1) * pl.nshared + r) * 2 + (strip - s_lo)) + 1;
-      }
-    }
-    row_dst[pi] = code;
-  }
-  __syncthreads();
-  // A wavefront takes rows wave, wave + 4, ... of every input channel, its lanes the columns:
-  // the row is the sum, in wave order, of the wavefronts' images that reach it (wavefront
-  // w's image starts at row sx * w * rw), written where the row's code says.
+  int4 *row_tab = (int4 *)lds;                           // kind, destination word, first image word, images
+  const int wave_words = pl.c_in * wplane_words;         // from one wavefront's images to the next one's
+  const int wave_step = wave_words - pl.sx * pl.rw * pl.Wp;   // ... to the same image row there
   {
-    const i64 nc0 = (i64)n * pl.c_in;
-    auto row_sum = [&](int cc, int pi, int gy) {
-      float v = 0.f;
-      if (pi < pl.Rp && gy + pl.py < pl.Wp) {
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-          const int wr = pi - pl.sx * w * pl.rw;
-          if (wr >= 0 && wr < Rw) v += wplanes[(w * pl.c_in + cc) * wplane_words + wr * pl.Wp + pl.py + gy];
+    const StripMap map(pl);
+    for (int pi = tid; pi < rp_t; pi += 256) {
+      const int gx = g0 + pi;
+      int kind = -1, dst = 0;
+      if (gx >= 0 && gx < pl.ngx) {
+        int s_lo, s_hi;
+        map.feeding(gx, s_lo, s_hi);
+        if (s_lo == s_hi) {
+          if (s_lo == strip) { kind = 0; dst = gx * pl.ngy; }
+        } else if (strip == s_lo || strip == s_hi) {
+          // boundary s_hi, row number within the boundary's shared rows, upper or lower strip
+          const int r = gx - (pl.sx * s_hi * pl.Th - pl.px);
+          kind = 1;
+          dst = (((s_hi - 1) * pl.nshared + r) * 2 + (strip - s_lo)) * pl.ngy;
         }
       }
-      return v;
-    };
-    auto row_out = [&](int cc, int code) {
-      return (code & 1) ? WS + ((nc0 + cc) * (pl.strips - 1) * pl.nshared * 2 + (code >> 1)) * pl.ngy
-                        : GI + ((nc0 + cc) * pl.ngx + (code >> 1)) * pl.ngy;
-    };
+      // wavefronts w0 .. w0 + nw - 1 have row pi in their images (none: a row past the reach of
+      // the strip's last grad_out row, zeros)
+      int w0 = 0, nw = 0;
+      for (int w = 0; w < kWaves; ++w) {
+        const int wr = pi - pl.sx * w * pl.rw;
+        if (pi < pl.Rp && wr >= 0 && wr < Rw) { if (nw == 0) w0 = w; ++nw; }
+      }
+      row_tab[pi] = make_int4(kind, dst, w0 * wave_words + (pi - pl.sx * w0 * pl.rw) * pl.Wp, nw);
+    }
+  }
+  __syncthreads();
+  {
+    const int gi_c = pl.ngx * pl.ngy, ws_c = (pl.strips - 1) * pl.nshared * 2 * pl.ngy;   // words per input channel
+    float *GIn = GI + (i64)n * pl.c_in * gi_c, *WSn = WS + (i64)n * pl.c_in * ws_c;
+    // four rows per trip: their table entries first, then all their reads, then the stores,
+    // so that the LDS round trips of the four overlap
     for (int cc = 0; cc < pl.c_in; ++cc)
       for (int pi = wave; pi < rp_t; pi += 4 * kWaves) {
-        // four rows per trip, so that their LDS reads are in flight together
-        int code[4];
+        int kind[4], dst[4], src[4], nw[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) code[u] = pi + u * kWaves < rp_t ? row_dst[pi + u * kWaves] : -1;
+        for (int u = 0; u < 4; ++u) {
+          const int4 e = row_tab[min(pi + u * kWaves, rp_t - 1)];
+          kind[u] = pi + u * kWaves < rp_t ? __builtin_amdgcn_readfirstlane(e.x) : -1;
+          dst[u] = __builtin_amdgcn_readfirstlane(e.y);
+          src[u] = __builtin_amdgcn_readfirstlane(e.z);
+          nw[u] = __builtin_amdgcn_readfirstlane(e.w);
+        }
         for (int gy = lane; gy < pl.ngy; gy += 64) {
-          float v[4];
+          // (no branches: all reads are requested together; a wavefront that does not reach the
+          // row, or a column past the image's, re-reads the first word and adds a zero)
+          const bool inside = gy + pl.py < pl.Wp;
+          const int col = inside ? gy : 0;
+          float x[4][kWaves];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) v[u] = code[u] >= 0 ? row_sum(cc, pi + u * kWaves, gy) : 0.f;
+          for (int u = 0; u < 4; ++u) {
+            const float *in = wplanes + src[u] + cc * wplane_words + pl.py;
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (code[u] >= 0) row_out(cc, code[u])[gy] = v[u];
+            for (int k = 0; k < kWaves; ++k) x[u][k] = in[(k < nw[u] ? k * wave_step : 0) + col];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            float v = 0.f;
+#pragma unroll
+            for (int k = 0; k < kWaves; ++k) v += (inside && k < nw[u]) ? x[u][k] : 0.f;
+            float *out = (kind[u] > 0 ? WSn + cc * ws_c : GIn + cc * gi_c) + dst[u];
+            if (kind[u] >= 0) out[gy] = v;
+          }
         }
       }
   }
@@ -750,8 +771,8 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   STAMP();
 #ifdef EXP_STAMP
   if ((blockIdx.x == 100 || blockIdx.x == 300) && lane == 0)
-    printf("blk %d wave %d n_it %d: prologue %lld barrier %lld main %lld barrier %lld epilogue %lld\n", (int)blockIdx.x, wave, n_it,
-           stamp[1] - stamp[0], stamp[2] - stamp[1], stamp[3] - stamp[2], stamp[4] - stamp[3], stamp[5] - stamp[4]);
+    printf("blk %d wave %d n_it %d: prologue %lld barrier %lld main %lld barrier %lld rowtab %lld barrier %lld rows %lld\n", (int)blockIdx.x, wave, n_it,
+           stamp[1] - stamp[0], stamp[2] - stamp[1], stamp[3] - stamp[2], stamp[4] - stamp[3], stamp[5] - stamp[4], stamp[6] - stamp[5], stamp[7] - stamp[6]);
 #endif
 }
 
