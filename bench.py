@@ -10,11 +10,18 @@ s = d = u = 1, p = 0, fp32, inputs resident in HBM before the clock starts.
 Prints one JSON line.  `value` is algorithmic GB/s (each operand read once,
 each result written once) over the whole step; `frames_per_s` counts the
 32 x 512 input frames once per step.  `roofline` describes the pass that takes
-the longest, timed with HIP events on the launch stream: against the fp32
-matrix peak when its arithmetic intensity (algorithmic FLOP per algorithmic
-byte) is above the machine's ridge point, against the HBM peak otherwise, with
-the other figure alongside.  `cpu_baseline` times the CPU checker on the same
-batch on the host cores.
+the longest (median of at least 100 launches, each timed with HIP events on the
+launch stream), against the roof that binds it: the time its algorithmic bytes
+need at the HBM peak against the time its matrix instructions need at their
+peak (bf16 instructions, six per fp32 product, when the kernels ran in the
+library's default bf16x3 mode; fp32 instructions otherwise), with the other
+figure alongside.  `cpu_baseline` times the CPU checker on the same batch on
+the host cores.
+
+Before the clock starts the step is repeated until the GPU has been busy for
+50 ms (`prewarm_ms`; outside the timed region, on top of --warmup): a step
+takes a quarter of a millisecond and a chip that has idled runs its first few
+milliseconds 5-10 % slow.
 """
 import argparse
 import json
@@ -29,21 +36,26 @@ for _p in (ROOT, os.path.join(ROOT, "cnn-mellin_amd")):
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3     # MI355X fp32 matrix (MFMA) = packed vector fp32, published
+BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 matrix (MFMA), published
+PREWARM_MS = 50.0
+MIN_PASS_REPS = 100
 
-# HBM bytes per launch of each pass at this workload, measured with
-#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 3 --warmup 1 --no-cpu
-#   rocprofv3 --pmc WRITE_SIZE -- python3 bench.py --steps 3 --warmup 1 --no-cpu
-# (KiB per dispatch, summed over the kernels of the pass) and scaled by what the same
-# counters read for a plain 256 MiB device copy (--copy-calibration): FETCH_SIZE x 2.0,
-# WRITE_SIZE x 1.0.  The summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    "mconv2d.forward": 35.3e6, "mconv2d.grad_input": 88.3e6, "mconv2d.grad_weight": 47.8e6,
-    "lconv2d.forward": 195.6e6, "lconv2d.grad_input": 190.1e6, "lconv2d.grad_weight": 214.3e6,
-}
-MEASURED_TRAFFIC_VARIANTS = {
-    "mconv2d.forward": "mfma", "mconv2d.grad_input": "mfma-taps+fold", "mconv2d.grad_weight": "mfma-rows",
-    "lconv2d.forward": "mfma", "lconv2d.grad_input": "mfma-fused", "lconv2d.grad_weight": "mfma-rows",
-}
+# HBM bytes per launch of each pass at this workload come from the data file that is written
+# together with the profile summary of the same name under profiles/ (rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters read for a plain
+# 256 MiB device copy).  An entry is used only if the pass ran the variant and the math mode
+# that were profiled.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_cfg3_hbm_bytes.json")
+
+
+def measured_traffic(pass_name, variant, math):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            e = json.load(f)["passes"][pass_name]
+    except (OSError, KeyError, ValueError):
+        return None
+    return e["bytes"] if (e.get("variant"), e.get("math")) == (variant, math) else None
+
 
 CFG = dict(batch=32, c_in=3, c_out=64, ngx=512, ngy=41, nfx=8, nfy=4,
            s=(1, 1), d=(1, 1), p=(0, 0), u=(1, 1))
@@ -129,17 +141,19 @@ class Layer:
 
 
 def time_pass(fn, reps, torch):
-    """Average duration of one call, in microseconds, from HIP events on the launch stream."""
-    for _ in range(3):
+    """Median duration of one call, in microseconds: every call sits between two HIP events
+    on the launch stream (torch's current stream is the stream the library launches on)."""
+    for _ in range(5):
         fn()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(reps):
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    marks[0].record()
+    for i in range(reps):
         fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) * 1e3 / reps
+        marks[i + 1].record()
+    marks[-1].synchronize()
+    times = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(reps))
+    return times[len(times) // 2]
 
 
 def cpu_baseline(layers, slice_n, reps=25):
@@ -164,8 +178,25 @@ def cpu_baseline(layers, slice_n, reps=25):
     med = sorted(times)[len(times) // 2]
     nbytes = sum(3 * (L.bytes_per_pass - L.w.numel() * 4) * slice_n / CFG["batch"] + 3 * L.w.numel() * 4
                  for L in layers)
+    extra = {}
+    if oracle.have_ref():
+        # the reference's own header (compiled from the reference checkout where one was present
+        # at build time) has the Mellin x linear kernels only: the same half of the step through
+        # it and through the port, to show that the port is not the slower of the two
+        L = layers[0]
+        x = np.ascontiguousarray(L.x_cpu.numpy()[:slice_n])
+        go = np.ascontiguousarray(L.go_cpu.numpy()[:slice_n])
+        w, b = L.w_cpu.numpy(), L.b_cpu.numpy()
+        for impl in ("ref", "port"):
+            ts = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                oracle.mcorrlcorr(x, w, b, 1, 1, 0, 1, 0, impl=impl)
+                oracle.mcorrlcorr_backward(x, w, go, 1, 1, 0, 1, impl=impl)
+                ts.append(time.perf_counter() - t0)
+            extra["mconv2d_half_%s_ms" % ("reference" if impl == "ref" else "port")] = round(sorted(ts)[2] * 1e3, 2)
     return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": min(threads, cores),
-            "kind": "port",
+            "kind": "port", **extra,
             "sample": "same step on utterances 0..%d of 32 (%.0f MB algorithmic), median of %d repetitions "
                       "(%.1f s of CPU work in all), %.2f s each; %.0f frames/s"
                       % (slice_n - 1, nbytes / 1e6, reps, sum(times), med, slice_n * CFG["ngx"] / med),
@@ -175,10 +206,10 @@ def cpu_baseline(layers, slice_n, reps=25):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # a step is a third of a millisecond and the first few milliseconds after an idle spell run
-    # 5-8 % slow (measured: 5 warm-up steps 0.358 ms/step, 50 or more 0.335), hence the defaults
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--math", choices=["bf16x3", "fp32"], default="bf16x3",
+                    help="how the matrix kernels form fp32 products (library default: bf16x3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--variant", default=None, help="force a kernel variant (e.g. generic)")
     ap.add_argument("--cpu-slice", type=int, default=32, help="utterances in the CPU baseline sample")
@@ -205,6 +236,7 @@ def main():
                           "launches": 10}))
         return
     hip.set_variant(args.variant)
+    hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
     gen = torch.Generator().manual_seed(2)
     layers = [Layer(hip.AX_MCORR, "mconv2d", gen, dev), Layer(hip.AX_LCORR, "lconv2d", gen, dev)]
 
@@ -214,6 +246,17 @@ def main():
             L.backward_input()
             L.backward_weight()
 
+    # pre-warm: steps until the GPU has worked for PREWARM_MS (disclosed, outside the timed region)
+    pre0, pre1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pre0.record()
+    prewarm_ms, prewarm_steps = 0.0, 0
+    while prewarm_ms < PREWARM_MS:
+        for _ in range(20):
+            step()
+        prewarm_steps += 20
+        pre1.record()
+        pre1.synchronize()
+        prewarm_ms = pre0.elapsed_time(pre1)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -229,32 +272,44 @@ def main():
     frames = CFG["batch"] * CFG["ngx"]
 
     # per-pass durations (one kernel chain per pass) for the roofline of the dominant one
-    per_pass = {}
-    variants = {}
+    per_pass, variants, maths = {}, {}, {}
     for L in layers:
         for pname, fn in L.passes():
-            per_pass["%s.%s" % (L.name, pname)] = time_pass(fn, max(10, args.steps), torch)
-            variants["%s.%s" % (L.name, pname)] = hip.last_variant()
+            key = "%s.%s" % (L.name, pname)
+            per_pass[key] = time_pass(fn, max(MIN_PASS_REPS, args.steps), torch)
+            variants[key] = hip.last_variant()
+            maths[key] = "bf16x3" if hip.last_math() == hip.MATH_BF16X3 else "fp32"
     dom = max(per_pass, key=per_pass.get)
     domL = layers[0] if dom.startswith("mconv2d") else layers[1]
     dom_us = per_pass[dom]
     achieved_gbs = domL.bytes_per_pass / dom_us / 1e3
     dom_tflops = 2 * domL.macs_per_pass / dom_us / 1e6
-    # which roof: arithmetic intensity against the ridge point of the two peaks
-    intensity = 2 * domL.macs_per_pass / domL.bytes_per_pass
-    ridge = FP32_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS
-    traffic = MEASURED_TRAFFIC_BYTES.get(dom) if variants[dom] == MEASURED_TRAFFIC_VARIANTS.get(dom) else None
-    if intensity > ridge:
-        roof = {"bound": "mfma", "achieved": round(dom_tflops, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(dom_tflops / FP32_PEAK_TFLOPS, 4)}
+    # which roof: the time the algorithmic bytes need at the HBM peak against the time the
+    # matrix instructions need at theirs (six bf16 instructions' worth per fp32 product in
+    # bf16x3 mode, where every fp32 operand is the exact sum of three bf16 parts)
+    flops = 2 * domL.macs_per_pass
+    if maths[dom] == "bf16x3":
+        matrix_flops, matrix_peak, matrix_unit = 6 * flops, BF16_PEAK_TFLOPS, "bf16"
+    else:
+        matrix_flops, matrix_peak, matrix_unit = flops, FP32_PEAK_TFLOPS, "fp32"
+    t_hbm_us = domL.bytes_per_pass / HBM_PEAK_GBS / 1e3
+    t_matrix_us = matrix_flops / matrix_peak / 1e6
+    matrix_tflops = matrix_flops / dom_us / 1e6
+    traffic = measured_traffic(dom, variants[dom], maths[dom])
+    if t_matrix_us > t_hbm_us:
+        roof = {"bound": "mfma", "achieved": round(matrix_tflops, 2), "peak": matrix_peak, "unit": "TFLOP/s",
+                "frac": round(matrix_tflops / matrix_peak, 4)}
     else:
         roof = {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved_gbs / HBM_PEAK_GBS, 4)}
-    roof.update({"traffic": traffic, "kernel": dom, "variant": variants[dom], "avg_us": round(dom_us, 2),
-                 "flop_per_byte": round(intensity, 1), "ridge_flop_per_byte": round(ridge, 1),
-                 "algorithmic_bytes": domL.bytes_per_pass, "algorithmic_flops": 2 * domL.macs_per_pass,
+    roof.update({"traffic": traffic, "kernel": dom, "variant": variants[dom], "math": maths[dom],
+                 "median_us": round(dom_us, 2), "reps": max(MIN_PASS_REPS, args.steps),
+                 "algorithmic_bytes": domL.bytes_per_pass, "algorithmic_flops": flops,
+                 "us_at_hbm_peak": round(t_hbm_us, 2), "us_at_matrix_peak": round(t_matrix_us, 2),
+                 "matrix_instructions": matrix_unit, "matrix_flops_executed": matrix_flops,
                  "hbm_GBps": round(achieved_gbs, 1), "hbm_frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-                 "fp32_TFLOPs": round(dom_tflops, 2), "fp32_frac": round(dom_tflops / FP32_PEAK_TFLOPS, 4)})
+                 "matrix_TFLOPs": round(matrix_tflops, 2), "matrix_frac": round(matrix_tflops / matrix_peak, 4),
+                 "fp32_equivalent_TFLOPs": round(dom_tflops, 2)})
 
     line = {
         "metric": "mconv2d+lconv2d fwd+bwd GB/s and frames/sec on 1 MI355X; % HBM roofline",
@@ -268,19 +323,26 @@ def main():
                                "mconv2d (Mellin x linear) and lconv2d (linear x linear), each forward + "
                                "input-gradient + weight-gradient",
                    "algorithmic_MB_per_step": round(step_bytes / 1e6, 3),
-                   "GFLOP_per_step": round(step_flops / 1e9, 3)},
+                   "GFLOP_per_step": round(step_flops / 1e9, 3),
+                   "arithmetic": ("fp32 storage, fp32 accumulation; products of the matrix kernels: every fp32 "
+                                  "operand as the exact sum of three bf16 parts, the six largest of the nine "
+                                  "cross products on the bf16 matrix cores (what is dropped is below 2^-24 of "
+                                  "a product)" if args.math == "bf16x3" else
+                                  "fp32 storage, accumulation and matrix instructions")},
+        "prewarm_ms": round(prewarm_ms, 1), "prewarm_steps": prewarm_steps,
         "frames_per_s": round(frames / (elapsed / args.steps), 1),
         "pct_hbm_roofline": round(100.0 * step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS, 2),
         "tflops": round(step_flops / (elapsed / args.steps) / 1e12, 2),
         "roofline": roof,
         "per_pass_us": {k: round(v, 2) for k, v in per_pass.items()},
         "per_pass_variant": variants,
+        "per_pass_math": maths,
     }
     line["per_pass_roofline"] = {
         k: {"hbm_frac": round((layers[0] if k.startswith("mconv2d") else layers[1]).bytes_per_pass / v / 1e3
                               / HBM_PEAK_GBS, 4),
-            "fp32_frac": round(2 * (layers[0] if k.startswith("mconv2d") else layers[1]).macs_per_pass / v / 1e6
-                               / FP32_PEAK_TFLOPS, 4)}
+            "fp32_equivalent_TFLOPs": round(2 * (layers[0] if k.startswith("mconv2d") else layers[1]).macs_per_pass
+                                            / v / 1e6, 2)}
         for k, v in per_pass.items()}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(layers, args.cpu_slice)

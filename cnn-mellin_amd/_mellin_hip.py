@@ -42,6 +42,7 @@ SYMBOLS = {
     "mellin_set_variant": (_int, [ctypes.c_char_p]),
     "mellin_set_math": (_int, [_int]),
     "mellin_get_math": (_int, []),
+    "mellin_last_math": (_int, []),
     "mellin_corr2d_backward_weight_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
@@ -104,6 +105,11 @@ def set_math(mode):
 
 def get_math():
     return lib.mellin_get_math()
+
+
+def last_math():
+    """The mode the most recent operator-level call's kernels multiplied in."""
+    return lib.mellin_last_math()
 
 
 def _check(code):

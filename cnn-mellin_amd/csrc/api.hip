@@ -28,6 +28,7 @@ thread_local char g_error[512] = "";
 // autograd thread, and a variant forced from the user's thread must hold there too.
 std::atomic<const char *> g_variant{""};
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
+std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
 std::atomic<int> g_forced{0};    // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
                                  // and without the row-wise weight gradient
 
@@ -97,6 +98,7 @@ template <typename T>
 hipError_t run_sepconv(const SepConv &pr, const T *f, const T *g, const T *bias,
                        T *h, hipStream_t stream) {
   g_variant = "generic";
+  g_last_math = MATH_FP32;
   return launch_sepconv_generic<T>(pr, f, g, bias, h, stream);
 }
 
@@ -109,10 +111,12 @@ hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
     int mt = 0, nt = 0;
     if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
       g_variant = "mfma";
+      g_last_math = pl.split ? MATH_BF16X3 : MATH_FP32;
       return launch_tile_gemm(pl, lds, mt, nt, f, g, bias, h, stream);
     }
   }
   g_variant = "generic";
+  g_last_math = MATH_FP32;
   return launch_sepconv_generic<float>(pr, f, g, bias, h, stream);
 }
 
@@ -214,6 +218,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
     pr.out_half = 1;
     if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
       g_variant = "mfma";
+      g_last_math = pl.split ? MATH_BF16X3 : MATH_FP32;
       if (wrote_half) *wrote_half = true;
       return check_hip(launch_tile_gemm(pl, lds, mt, nt, (const float *)weight, (const float *)input,
                                         (const float *)bias, (float *)half_out, (hipStream_t)stream), fn);
@@ -338,12 +343,14 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
                   workspace_bytes);
     if (which == IN_FUSED) {
       g_variant = "mfma-fused";
+      g_last_math = ips.fused.stream ? MATH_BF16X3 : MATH_FP32;
       return check_hip(launch_igrad(ips.fused, (const float *)weight, (const float *)grad_out,
                                     (float *)grad_input, (float *)workspace, (hipStream_t)stream), fn);
     }
     if (which == IN_TAPS) {
       // tap products through the workspace, then a gather (any x axis kind)
       g_variant = "mfma-taps+fold";
+      g_last_math = MATH_FP32;
       hipError_t e = launch_tap_product(ips.taps, (const float *)weight, (const float *)grad_out,
                                         (float *)workspace, (hipStream_t)stream);
       if (e == hipSuccess) {
@@ -357,6 +364,7 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
     if (which == IN_TWO_PASS) {
       const TwoPassInput &tp = ips.two;
       g_variant = "mfma+fold";
+      g_last_math = tp.plan.split ? MATH_BF16X3 : MATH_FP32;
       hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight,
                                       (const float *)grad_out, nullptr, (float *)workspace,
                                       (hipStream_t)stream);
@@ -385,6 +393,7 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
     pr.out_half = 1;
     if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
       g_variant = "mfma";
+      g_last_math = pl.split ? MATH_BF16X3 : MATH_FP32;
       if (wrote_half) *wrote_half = true;
       return check_hip(launch_tile_gemm(pl, lds, mt, nt, (const float *)weight, (const float *)grad_out, nullptr,
                                         (float *)half_out, (hipStream_t)stream), fn);
@@ -417,6 +426,7 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
         return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn,
                     wp.ws_bytes, workspace_bytes);
       g_variant = wp.rows_mode ? "mfma-rows" : "mfma";
+      g_last_math = wp.rows_mode == 2 ? MATH_BF16X3 : MATH_FP32;
       return check_hip(launch_wgrad(wp, (const float *)grad_out, (const float *)input,
                                     (float *)grad_weight, (float *)workspace,
                                     (hipStream_t)stream), fn);
@@ -428,6 +438,7 @@ int corr2d_backward_weight(const char *fn, int kind_x, const T *input,
   if (batch * ng * nh == 0) pr.x.nh_eff = 0;
   pr.batch = batch; pr.c_out = c_out; pr.c_in = c_in;
   g_variant = "generic";
+  g_last_math = MATH_FP32;
   return check_hip(launch_sepreduce_generic<T>(pr, grad_out, input, grad_weight,
                                                (hipStream_t)stream), fn);
 }
@@ -734,6 +745,7 @@ int mellin_set_math(int mode) {
   return MELLIN_OK;
 }
 int mellin_get_math(void) { return g_math; }
+int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
   if (!name || !*name) { g_forced = 0; return MELLIN_OK; }

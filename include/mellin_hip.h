@@ -324,6 +324,9 @@ const char *mellin_last_variant(void);
 #define MELLIN_MATH_BF16X3 1
 int mellin_set_math(int mode);
 int mellin_get_math(void);
+/* The mode the matrix kernels of the most recent operator-level call actually ran in
+ * (MELLIN_MATH_FP32 also for the kernels that use no matrix instructions). */
+int mellin_last_math(void);
 
 /* Force a variant for subsequent operator-level calls of the process (all threads):
  * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
