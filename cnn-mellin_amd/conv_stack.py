@@ -19,7 +19,7 @@ import torch
 
 import mconv
 
-__all__ = ["ConvStackParams", "ConvStack", "layer_plan", "pack_windows"]
+__all__ = ["ConvStackParams", "ConvStack", "FrameClassifier", "layer_plan", "pack_windows"]
 
 
 class ConvStackParams:
@@ -145,3 +145,23 @@ class ConvStack(torch.nn.Module):
             if lay["pool"]:
                 x = torch.nn.functional.max_pool2d(x, (1, 2))
         return x
+
+
+class FrameClassifier(torch.nn.Module):
+    """Convolution stack, then a linear projection of every frame's features to log-probabilities.
+
+    The output stage of the reference's acoustic model without its recurrent layers
+    (models.py:437-454: the convolutional features of a frame, channels x bins flattened, go
+    through ``torch.nn.Linear`` to ``target_dim`` scores): ``x (N, C_in, T, F) ->
+    (N, T', n_out)`` log-probabilities.  The projection is PyTorch's; only the convolutions
+    run in this package's kernels."""
+
+    def __init__(self, stack: ConvStack, n_out: int = 62):
+        super().__init__()
+        self.stack = stack
+        self.out = torch.nn.Linear(stack.out_channels * stack.out_size[1], n_out)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        h = self.stack(x)                                   # (N, C, T', F')
+        h = h.permute(0, 2, 1, 3).flatten(2)                # (N, T', C * F')
+        return torch.nn.functional.log_softmax(self.out(h), dim=-1)

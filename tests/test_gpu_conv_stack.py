@@ -5,20 +5,26 @@
 * parity: forward output and every gradient of a reduced stack against the same
   stack evaluated with the CPU checker in float64 (checker ops wrapped in
   torch.autograd.Function, ReLU / max-pool by torch on the CPU);
-* the full-size 10-layer stack (3 -> 256 channels, 4x4 kernels, batch 32,
-  780 x 41) runs forward + backward, is finite and run-to-run identical.
+* the full-size 10-layer stacks of BASELINE config 5 (3 -> 256 channels, 4x4
+  kernels, ReLU, frequency pools, batch 32, 780 x 41, Linear -> 62
+  log-probabilities), Mellin and linear: one forward + backward of the whole
+  model, then EVERY layer's forward output, input gradient and weight gradient
+  of that run against the CPU checker on the layer's own captured input and
+  upstream gradient (utterance and channel slices), at the operator tolerance
+  rtol 1e-5 / atol 1e-5 * sqrt(fan_in);
+* the full-size Mellin stack is finite and run-to-run identical.
 
-Tolerance: the stack compounds ten layers, so outputs and gradients are held to
-rtol 1e-4 of the largest magnitude of the tensor compared (per-layer tolerance
-is checked by the operator tests).
+Tolerance of the end-to-end comparison of the reduced stack: it compounds five
+layers, so outputs and gradients are held to 1e-4 of the largest magnitude of
+the tensor compared; per-layer comparisons use the operator tolerance.
 """
 import numpy as np
 import pytest
 import torch
 
 import mconv
-from conv_stack import ConvStack, ConvStackParams, layer_plan
-from _gpu import to_gpu, to_np
+from conv_stack import ConvStack, ConvStackParams, FrameClassifier, layer_plan
+from _gpu import assert_close, f64, to_gpu, to_np
 from oracle import oracle
 
 pytestmark = pytest.mark.gpu
@@ -105,6 +111,109 @@ def test_reduced_stack_matches_checker(mellin):
     for no, (conv, (w, b)) in enumerate(zip(stack.convs, params64), 1):
         _close(conv.weight.grad, w.grad, "grad_weight layer %d" % no)
         _close(conv.bias.grad, b.grad, "grad_bias layer %d" % no)
+
+
+def _cfg5_params(mellin):
+    return ConvStackParams(layers=10, mellin=mellin, kernel_time=4, kernel_freq=4, initial_channels=32,
+                           factor_schedule=3, channel_factor=2, time_factor=1, freq_factor=1, in_channels=3,
+                           freq_pool_after=(3, 6, 9), seed=4)
+
+
+def _unit(a, b):
+    """1 / (rms(a) * rms(b)): the scale at which sums of products of a and b meet the
+    tolerance's assumption of unit-scale operands (atol 1e-5 * sqrt(fan_in))."""
+    ra = float(np.sqrt(np.mean(np.square(a, dtype=np.float64))))
+    rb = float(np.sqrt(np.mean(np.square(b, dtype=np.float64))))
+    return 1.0 / max(ra * rb, 1e-30)
+
+
+def _cfg5_batch():
+    gen = torch.Generator().manual_seed(4)
+    lens = torch.randint(100, 781, (32,), generator=gen)
+    x = torch.randn(32, 3, 780, 41, generator=gen)
+    x = x * (torch.arange(780)[None, :] < lens[:, None])[:, None, :, None]     # zero past each length
+    targets = torch.randint(0, 62, (32, 780), generator=gen)
+    return x, lens, targets
+
+
+@pytest.mark.parametrize("mellin", [True, False], ids=["mellin", "linear"])
+def test_full_size_model_every_layer_matches_checker(mellin):
+    """BASELINE config 5 as stated: ten layers 3 -> 256 channels, 4 x 4 kernels, ReLU, frequency
+    max-pool 2 after layers 3, 6 and 9, linear projection to 62 log-probabilities, batch 32 of
+    up to 780 frames x 41 bins, seed 4.  One forward + backward of the model at full size;
+    then each layer of THAT run is checked on its own: its captured input and the captured
+    gradient of its output go through the checker, on two utterances (forward: all output
+    channels of narrow layers, sixteen spread ones of wide layers; input gradient: all
+    channels) and, for the weight gradient, on a spread of channel pairs over all 32
+    utterances (float64 checker: the sums run over up to a million terms).  Activations and
+    gradients deep in the model are far from unit scale, so every comparison is made after
+    scaling by 1 / (rms of the one operand x rms of the other), the scale the tolerance
+    rtol 1e-5 / atol 1e-5 * sqrt(fan_in) is stated for."""
+    stack = ConvStack(780, 41, _cfg5_params(mellin)).cuda()
+    assert [lay["out_channels"] for lay in stack.plan] == [32, 32, 64, 64, 64, 128, 128, 128, 256, 256]
+    model = FrameClassifier(stack, 62).cuda()
+    x, lens, targets = _cfg5_batch()
+    seen = {}
+
+    def keep(no):
+        def hook(module, inputs, output):
+            seen[no] = dict(x=inputs[0], out=output)
+            output.register_hook(lambda g, no=no: seen[no].__setitem__("g_out", g))
+            if inputs[0].requires_grad:
+                inputs[0].register_hook(lambda g, no=no: seen[no].__setitem__("g_in", g))
+        return hook
+
+    for no, conv in enumerate(stack.convs):
+        conv.register_forward_hook(keep(no))
+    xg = x.cuda().requires_grad_(True)
+    logp = model(xg)
+    t_out = stack.out_size[0]
+    assert tuple(logp.shape) == (32, t_out, 62)
+    torch.testing.assert_close(logp.exp().sum(-1), torch.ones(32, t_out, device="cuda"), rtol=1e-4, atol=1e-4)
+    frame_ok = (torch.arange(t_out)[None, :] < lens[:, None]).cuda()
+    loss = -(logp.gather(2, targets[:, :t_out, None].cuda()).squeeze(2) * frame_ok).sum() / frame_ok.sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(loss)) and bool(torch.isfinite(xg.grad).all())
+
+    nb = [1, 22]
+    for no, (lay, conv) in enumerate(zip(stack.plan, stack.convs)):
+        rec = seen[no]
+        fwd = oracle.mcorrlcorr if lay["kind"] == "mcorrlcorr" else oracle.lcorrlcorr
+        bwd = oracle.mcorrlcorr_backward if lay["kind"] == "mcorrlcorr" else oracle.lcorrlcorr_backward
+        s, d, p, r = lay["s"], lay["d"], lay["p"], lay["r"]
+        c_in, c_out = lay["in_channels"], lay["out_channels"]
+        w, b = to_np(conv.weight), to_np(conv.bias)
+        xin = to_np(rec["x"][nb])
+        out = rec["out"]                                             # after the fused ReLU
+        assert tuple(out.shape[:2]) == (32, c_out) and float((out == 0).float().mean()) > 0.05
+        what = "%s layer %d (%d -> %d, %s)" % (lay["kind"], no + 1, c_in, c_out, tuple(out.shape[2:]))
+        # forward, ReLU included
+        co = list(range(c_out)) if c_out <= 64 else list(range(3, c_out, c_out // 16))
+        exp = np.maximum(fwd(xin, w[co], b[co], s, d, p, 1, r), 0)
+        k = _unit(xin, w)
+        assert_close(out[nb][:, co] * k, exp * k, c_in * 16, what + " forward")
+        # the gradient that reaches the correlation: zero where the ReLU clamped
+        g_pre = rec["g_out"] * (out > 0)
+        # input gradient of the two utterances, every input channel
+        if "g_in" in rec or no == 0:
+            got = xg.grad if no == 0 else rec["g_in"]
+            gn = to_np(g_pre[nb])
+            gi, _, _ = bwd(xin, w, gn, s, d, p, 1)
+            k = _unit(w, gn)
+            assert_close(got[nb] * k, gi * k, c_out * 16, what + " grad_input")
+        # weight gradient over the whole batch, a spread of channel pairs
+        cos = sorted({0, c_out // 3, c_out - 1})
+        cis = sorted({0, c_in // 2, c_in - 1})
+        xs = np.ascontiguousarray(to_np(rec["x"][:, cis]))
+        gs = np.ascontiguousarray(to_np(g_pre[:, cos]))
+        _, gw, gb = bwd(*f64(xs, w[cos][:, cis], gs), s, d, p, 1)
+        positions = 32 * out.shape[2] * out.shape[3]
+        k = _unit(xs, gs)
+        assert_close(conv.weight.grad[cos][:, cis] * k, gw * k, positions, what + " grad_weight")
+        k = _unit(gs, np.ones(1))
+        assert_close(conv.bias.grad[cos] * k, gb * k, positions, what + " grad_bias")
+        del rec["x"], rec["out"], rec["g_out"]
 
 
 def test_full_size_stack_runs_and_is_deterministic():
