@@ -467,13 +467,6 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   extern __shared__ __align__(16) float lds[];
   constexpr int P = NT * 32, ROWS = MTT * 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#ifdef EXP_STAMP
-  long long stamp[8]; int nstamp = 0;
-#define STAMP() stamp[nstamp++] = __builtin_readcyclecounter()
-#else
-#define STAMP()
-#endif
-  STAMP();
   const int half = lane >> 5, l32 = lane & 31;
   const int n = blockIdx.x / pl.strips, strip = blockIdx.x - n * pl.strips;
   const int ha = strip * pl.Th, hb = min(ha + pl.Th, pl.H);    // grad_out rows [ha, hb)
@@ -563,11 +556,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       const int voff = q * 4 + 8 * half * nh4;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-#ifdef EXP_NO_LOAD
-        o.v[t][i] = __int_as_float(voff + i + ks);
-#else
         o.v[t][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(go_rsrc, voff, (16 * ks + i) * nh4, 0));
-#endif
     }
   };
   floatx16 acc[MTT][NT];
@@ -579,15 +568,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     constexpr bool kFirst = decltype(first_tag)::value;      // an iteration's first step starts the sums from zero
     uintx4 bh[NT], bm[NT], bl[NT];
 #pragma unroll
-#ifdef EXP_NO_SPLIT
-    for (int t = 0; t < NT; ++t) {
-      bh[t] = uintx4{__float_as_uint(o.v[t][0]), __float_as_uint(o.v[t][1]), __float_as_uint(o.v[t][2]), __float_as_uint(o.v[t][3])};
-      bm[t] = uintx4{__float_as_uint(o.v[t][4]), __float_as_uint(o.v[t][5]), __float_as_uint(o.v[t][6]), __float_as_uint(o.v[t][7])};
-      bl[t] = bh[t] ^ bm[t];
-    }
-#else
     for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
-#endif
     const uintx4 *af = Af + (2 * ks + half) * ROWS + l32;
 #pragma unroll
     for (int a = 0; a < MTT; ++a) {
@@ -598,18 +579,11 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
           const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           acc[a][t] = zero16;
         }
-#ifdef EXP_ONE_MFMA
-        acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ah ^ am ^ al), as_bf16x8(bh[t] ^ bm[t] ^ bl[t]), acc[a][t], 0, 0, 0);
-#else
         mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
-#endif
       }
     }
   };
   auto fold_tiles = [&](int it) {
-#ifdef EXP_NO_FOLD
-    if (it != 0) return;
-#endif
     {
       // fold: Z[tap, position] joins word base(position) + off(tap) of the input channel's image
 #pragma unroll
@@ -651,9 +625,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       }
     }
   };
-  STAMP();
   __syncthreads();                                       // fragments and zeros are in place
-  STAMP();
   {
     // two operand buffers alternate; the loads of a step are requested one step ahead
     BOp b0, b1;
@@ -672,9 +644,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       fold_tiles(it);
     }
   }
-  STAMP();
   __syncthreads();                                       // every wavefront's image is complete; the fragments are free
-  STAMP();
 
   // Write-out.  Row i of the strip's image is grad_input row g0 + i: the sum, in wave order,
   // of the rows of the wavefronts' images that reach it (wavefront w's image starts at row
@@ -768,12 +738,6 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       }
     }
   }
-  STAMP();
-#ifdef EXP_STAMP
-  if ((blockIdx.x == 100 || blockIdx.x == 300) && lane == 0)
-    printf("blk %d wave %d n_it %d: prologue %lld barrier %lld main %lld barrier %lld rowtab %lld barrier %lld rows %lld\n", (int)blockIdx.x, wave, n_it,
-           stamp[1] - stamp[0], stamp[2] - stamp[1], stamp[3] - stamp[2], stamp[4] - stamp[3], stamp[5] - stamp[4], stamp[6] - stamp[5], stamp[7] - stamp[6]);
-#endif
 }
 
 template <int MTT, int NT>

@@ -45,11 +45,6 @@ namespace mellin {
 
 namespace {
 
-#ifndef MELLIN_STAMP
-#define MELLIN_STAMP(i)
-#define MELLIN_PROBE_DECL
-#endif
-
 // MB: 64-word blocks per wave whose staging sources are kept from a tile's first
 // chunk for its other chunks (0: nothing kept; the instance for layers whose
 // channels fit in one or two chunks).
@@ -86,7 +81,6 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   int *tapoff = (int *)(Ws0 + (single_chunk ? 1 : 2) * w_words);   // [KCp]
   float *Bs = (float *)(tapoff + n_tapoff);          // [M_T] bias (zeros when accumulating)
 
-  MELLIN_PROBE_DECL
   const int tid = threadIdx.x;
   // the wave index is wave-uniform: say so, and everything derived from it (row
   // loops, base addresses) is computed on the scalar unit
@@ -198,7 +192,6 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     for (int m = tid; m < M_T; m += kThreads)
       Bs[m] = (!ACC && bias && m0 + m < pl.M) ? bias[m0 + m] : 0.f;
   }
-  MELLIN_STAMP(0);
   if (my_stages > 0) {
     if (SPLIT) {
       // filter fragments, once: a thread splits the eight taps k = 8 g .. 8 g + 7 of channel m
@@ -223,7 +216,6 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     }
     issue_stage(0, 0, 0);
   }
-  MELLIN_STAMP(1);
 
   const FastDiv by_noy(pl.noy);
   floatx16 acc[MT][NT];
@@ -311,23 +303,17 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     // every wave's loads for this stage have landed, and every wave is done
     // reading the buffer the next stage will fill
     wait_all_memory();
-    MELLIN_STAMP(2);
     __syncthreads();
-    MELLIN_STAMP(3);
     if (st + 1 < my_stages) {
-      MELLIN_STAMP(7);
       // (at raised priority: a staging wavefront otherwise gets an issue slot only now and
       // then between the matrix instructions of its SIMD's other wavefronts)
       __builtin_amdgcn_s_setprio(3);
       issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
       __builtin_amdgcn_s_setprio(0);
-      MELLIN_STAMP(8);
     }
-    MELLIN_STAMP(4);
 
     if (ch == 0) {
       if (st > 0) epilogue();                             // the tile finished one stage ago
-      MELLIN_STAMP(5);
       tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
       // position -> LDS word of its (fx = 0, fy = 0) tap
 #pragma unroll
@@ -365,10 +351,8 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       multiply_taps<MT, NT>(acc, Ws0 + (single_chunk ? 0 : (st & 1) * w_words) + l32 * pl.WSS + half, 32 * pl.WSS,
                             tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
-    MELLIN_STAMP(6);
   }
   if (my_stages > 0) epilogue();
-  MELLIN_STAMP(9);
 #undef pl
 }
 

@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
 """Per-pass timings on one MI355X of the layer shapes beside the benchmark's own.
 
-    python cnn-mellin_amd/time_layers.py cfg4            # wide 2-D layer, linear and Mellin x axis
-    python cnn-mellin_amd/time_layers.py cfg2            # 1-D layers over the (s, d, p) grid
-    python cnn-mellin_amd/time_layers.py stack           # the 10-layer 3 -> 256 stacks, layer by layer
+    python time_layers.py cfg4            # wide 2-D layer, linear and Mellin x axis
+    python time_layers.py cfg2            # 1-D layers over the (s, d, p) grid
+    python time_layers.py stack           # the 10-layer 3 -> 256 stacks, layer by layer
 
 Every pass is one call of the C ABI on pre-allocated tensors, timed with HIP events
 on the launch stream.  One JSON object per line: the layer, its output extent, and
@@ -16,7 +16,7 @@ import json
 import os
 import sys
 
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "cnn-mellin_amd"))
 
 
 def tap_pairs(kind, nf, ng, nh, s, d, p, u=1):
@@ -66,7 +66,9 @@ def time_layer(tag, kind_x, x, w, b, s, d, p, r, reps, activation=None):
                      ("grad_input", lambda: hip.corr2d_backward_input(kind_x, w, go, gi, dims)),
                      ("grad_weight", lambda: hip.corr2d_backward_weight(kind_x, x, go, gw, dims))):
         us = event_us(fn, reps)
-        rec[name] = {"us": round(us, 1), "variant": hip.last_variant(), "tflops": round(2 * macs / us / 1e6, 1)}
+        rec[name] = {"us": round(us, 1), "variant": hip.last_variant(),
+                     "math": "bf16x3" if hip.last_math() == hip.MATH_BF16X3 else "fp32",
+                     "tflops": round(2 * macs / us / 1e6, 1)}
     return rec, out
 
 
@@ -104,16 +106,18 @@ def run_stack(reps):
     import time
     import torch
     import _mellin_hip as hip
-    from conv_stack import ConvStack, ConvStackParams
+    from conv_stack import ConvStack, ConvStackParams, FrameClassifier
     for mellin in (True, False):
         params = ConvStackParams(layers=10, mellin=mellin, kernel_time=4, kernel_freq=4, initial_channels=32,
                                  factor_schedule=3, channel_factor=2, time_factor=1, freq_factor=1,
                                  in_channels=3, freq_pool_after=(3, 6, 9), seed=4)
-        stack = ConvStack(780, 41, params).cuda()
+        model = FrameClassifier(ConvStack(780, 41, params), 62).cuda()
+        stack = model.stack
         x = torch.randn(32, 3, 780, 41, device="cuda", requires_grad=True)
 
         def step():
-            stack(x).square().mean().backward()
+            # the conv stack and its Linear -> 62 log-softmax head, summed over frames
+            model(x).square().mean().backward()
         for _ in range(3):
             step()
         torch.cuda.synchronize()
