@@ -215,6 +215,10 @@ def main():
     ap.add_argument("--cpu-slice", type=int, default=32, help="utterances in the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain device copy of known size (to scale profiler byte counters)")
+    ap.add_argument("--only-pass", default=None, metavar="LAYER.PASS",
+                    help="only launch one pass --launches times, e.g. lconv2d.grad_input (for profiler "
+                         "runs: every kernel in the trace then belongs to that pass)")
+    ap.add_argument("--launches", type=int, default=10)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (got --gpus %d)" % args.gpus)
@@ -239,6 +243,17 @@ def main():
     hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
     gen = torch.Generator().manual_seed(2)
     layers = [Layer(hip.AX_MCORR, "mconv2d", gen, dev), Layer(hip.AX_LCORR, "lconv2d", gen, dev)]
+
+    if args.only_pass:
+        fns = {"%s.%s" % (L.name, pname): fn for L in layers for pname, fn in L.passes()}
+        if args.only_pass not in fns:
+            sys.exit("--only-pass: one of %s" % ", ".join(fns))
+        for _ in range(args.launches):
+            fns[args.only_pass]()
+        torch.cuda.synchronize()
+        print(json.dumps({"pass": args.only_pass, "launches": args.launches, "variant": hip.last_variant(),
+                          "math": "bf16x3" if hip.last_math() == hip.MATH_BF16X3 else "fp32"}))
+        return
 
     def step():
         for L in layers:

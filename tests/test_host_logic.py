@@ -176,3 +176,29 @@ def test_workspace_queries_are_bounded_and_overflow_safe():
     dims = hip._dims(1 << 21, 1, 1, (1, 1), (4, 4), (4, 4), (1, 1), (1, 1), (0, 0), (1, 1))
     code = hip.lib.mellin_corr2d_forward_f32(hip.AX_LCORR, None, None, None, *dims, None, None)
     assert code == 1 and "2^20" in hip.last_error()
+
+
+def test_traffic_data_file_agrees_with_the_profile_summary():
+    """bench.py's roofline.traffic comes from profiles/bench_cfg3_hbm_bytes.json; every total in it is
+    a row of the committed profiler summary it names, to the summary's 0.1 MB, with the same kernel
+    variant and math mode."""
+    import json
+    import bench
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(bench.TRAFFIC_FILE) as f:
+        data = json.load(f)
+    rows = {}
+    with open(os.path.join(root, data["source"])) as f:
+        for line in f:
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) > 8 and cells[1] in data["passes"] and cells[4].count("kernel"):
+                rows[cells[1]] = cells
+    assert set(rows) == set(data["passes"]) and len(rows) == 6
+    for name, e in data["passes"].items():
+        cells = rows[name]
+        assert (cells[2], cells[3]) == (e["variant"], e["math"])
+        assert abs(float(cells[5]) - e["read_bytes"] / 1e6) <= 0.11
+        assert abs(float(cells[6]) - e["written_bytes"] / 1e6) <= 0.11
+        assert abs(float(cells[7]) - e["bytes"] / 1e6) <= 0.21
+        assert bench.measured_traffic(name, e["variant"], e["math"]) == e["bytes"]
+        assert bench.measured_traffic(name, "generic", e["math"]) is None
