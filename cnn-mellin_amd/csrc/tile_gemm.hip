@@ -51,8 +51,10 @@ namespace {
 // HOUT: H is half-precision storage (not with ACC): the fp32 results are rounded to
 // nearest even as they are stored.
 // SPLIT: the products run on the bf16 matrix cores, every fp32 operand as the exact sum of
-// three bf16 parts (tile_stage.hpp); only for layers whose channels are one chunk.  The
-// filter block then lives in LDS as fragments, built once per workgroup.
+// three bf16 parts (tile_stage.hpp).  The filter block then lives in LDS as fragments:
+// built once per workgroup when the channels are one chunk, otherwise per stage (the next
+// chunk's filter words are requested into registers before a stage's multiplies and split
+// into the other fragment buffer after them).
 template <int MT, int NT, bool ACC, int MB, bool HOUT, bool SPLIT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
@@ -76,8 +78,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
   const int ws_word0 = SPLIT ? (pl.sbuf * g_words + 3) & ~3 : pl.sbuf * g_words;
   float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS], or the fragments
-  const bool single_chunk = SPLIT || pl.CC >= pl.C;
-  const int n_tapoff = SPLIT ? pl.KC16 : pl.KCp;
+  const bool single_chunk = pl.CC >= pl.C;
+  // SPLIT keeps four tables of KC16 words: signal offset of tap k of a whole chunk and of
+  // the last (shorter) chunk, and the same two for the filter word's byte offset
+  const int n_tapoff = SPLIT ? 4 * pl.KC16 : pl.KCp;
   int *tapoff = (int *)(Ws0 + (single_chunk ? 1 : 2) * w_words);   // [KCp]
   float *Bs = (float *)(tapoff + n_tapoff);          // [M_T] bias (zeros when accumulating)
 
@@ -178,38 +182,82 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     if (!SPLIT && !single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
   };
 
+  // ---- SPLIT: the filter block as fragments ----------------------------------------
+  // Item idx = m * groups + g is the eight taps k = 8 g .. 8 g + 7 of output channel m;
+  // a thread takes items first + tid and first + tid + 256.  Words come through buffer loads whose
+  // offset is (channel's row) + (table entry of the tap): taps past the chunk and
+  // channels past M carry an offset beyond the filter and read as zeros.
+  constexpr int kFilterItems = 2;
+  constexpr unsigned kDeadOffset = 0x40000000u;
+  struct FilterWords { float x[kFilterItems][8]; };
+  const int f_groups = SPLIT ? pl.KC16 >> 3 : 1;
+  const int cc_last = pl.C - (chunks - 1) * pl.CC;
+  __amdgpu_buffer_rsrc_t f_rsrc;
+  if (SPLIT) f_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)F, 0, (int)pl.f_bytes, 0x00020000);
+  auto load_filter = [&](int ch, int first, FilterWords &fw) {
+    const int *ko = tapoff + (ch + 1 == chunks ? 3 : 2) * pl.KC16;
+    const int soff = (int)((unsigned)(ch * pl.CC) * (unsigned)pl.f_c * 4u);
+    const FastDiv by_groups(f_groups);
+#pragma unroll
+    for (int j = 0; j < kFilterItems; ++j) {
+      const int idx = first + tid + j * kThreads;
+      if (idx < f_groups * M_T) {
+        int m, g;
+        by_groups.divmod(idx, m, g);
+        const unsigned row = m0 + m < pl.M ? (unsigned)(m0 + m) * (unsigned)pl.f_m * 4u : kDeadOffset;
+        const int4 k0 = *(const int4 *)(ko + 8 * g), k1 = *(const int4 *)(ko + 8 * g + 4);
+        const int off[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          fw.x[j][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(f_rsrc, (int)(row + (unsigned)off[i]), soff, 0));
+      }
+    }
+  };
+  auto store_filter = [&](const FilterWords &fw, int first, float *buffer) {
+    const FastDiv by_groups(f_groups);
+#pragma unroll
+    for (int j = 0; j < kFilterItems; ++j) {
+      const int idx = first + tid + j * kThreads;
+      if (idx < f_groups * M_T) {
+        int m, g;
+        by_groups.divmod(idx, m, g);
+        store_frag((uintx4 *)buffer, f_groups, M_T, g, m, fw.x[j]);
+      }
+    }
+  };
+
   {
     const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
-    const int k_taps = pl.C * pl.nf;
-    for (int k = tid; k < n_tapoff; k += kThreads) {
+    for (int k = tid; k < (SPLIT ? pl.KC16 : pl.KCp); k += kThreads) {
       int cl, t, fx, fy;
       by_nf.divmod(k, cl, t);
       by_nfy.divmod(t, fx, fy);
-      // (SPLIT pads the taps to a multiple of 16: a padded tap reads the lane's first word,
-      // always a staged one, and meets a zero weight)
-      tapoff[k] = (SPLIT && k >= k_taps) ? 0 : cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+      const int off = cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+      if (SPLIT) {
+        // (the taps are padded to a multiple of 16, and the last chunk may have fewer
+        // channels: such a tap reads the lane's first word, always a staged one, and
+        // meets a zero weight)
+        const bool whole = k < pl.CC * pl.nf, last = k < cc_last * pl.nf;
+        const int fo = (cl * pl.f_c + t) * 4;
+        tapoff[k] = whole ? off : 0;
+        tapoff[pl.KC16 + k] = last ? off : 0;
+        tapoff[2 * pl.KC16 + k] = whole ? fo : (int)kDeadOffset;
+        tapoff[3 * pl.KC16 + k] = last ? fo : (int)kDeadOffset;
+      } else {
+        tapoff[k] = off;
+      }
     }
     for (int m = tid; m < M_T; m += kThreads)
       Bs[m] = (!ACC && bias && m0 + m < pl.M) ? bias[m0 + m] : 0.f;
   }
   if (my_stages > 0) {
     if (SPLIT) {
-      // filter fragments, once: a thread splits the eight taps k = 8 g .. 8 g + 7 of channel m
-      const int groups = pl.KC16 >> 3, k_taps = pl.C * pl.nf;
-      const FastDiv by_groups(groups), by_nf(pl.nf);
-      uintx4 *frag = (uintx4 *)Ws0;
-      for (int idx = tid; idx < groups * M_T; idx += kThreads) {
-        int m, g;
-        by_groups.divmod(idx, m, g);
-        float x[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int k = 8 * g + i;
-          int cl, t;
-          by_nf.divmod(k, cl, t);
-          x[i] = (k < k_taps && m0 + m < pl.M) ? F[(i64)(m0 + m) * pl.f_m + (i64)cl * pl.f_c + t] : 0.f;
-        }
-        store_frag(frag, groups, M_T, g, m, x);
+      __syncthreads();                                    // the offset tables
+      // (a filter that is one chunk may have more items than one round of the threads)
+      for (int first = 0; first < f_groups * M_T; first += kFilterItems * kThreads) {
+        FilterWords fw;
+        load_filter(0, first, fw);
+        store_filter(fw, first, Ws0);
       }
     } else if (single_chunk) {
       issue_filter(0, pl.C, ws_word0, true);
@@ -293,6 +341,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     if (full_m) write_tile(std::true_type());
     else write_tile(std::false_type());
   };
+  FilterWords next_filter;
   for (int st = 0, ti = 0, ch = 0; st < my_stages; ++st, ti += (ch + 1 == chunks), ch = (ch + 1 == chunks) ? 0 : ch + 1) {
     {
       unsigned zero;                                      // a zero the compiler cannot see through
@@ -309,6 +358,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       // then between the matrix instructions of its SIMD's other wavefronts)
       __builtin_amdgcn_s_setprio(3);
       issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
+      if (SPLIT && !single_chunk) load_filter(ch + 1 == chunks ? 0 : ch + 1, 0, next_filter);
       __builtin_amdgcn_s_setprio(0);
     }
 
@@ -345,12 +395,16 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     {
       const int cc = min(pl.CC, pl.C - ch * pl.CC);
       if (SPLIT)
-        multiply_taps_split<MT, NT>(acc, (const uintx4 *)Ws0, M_T, tapoff, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words,
-                                    lane_base, pl.KC16, l32, half);
+        multiply_taps_split<MT, NT>(acc, (const uintx4 *)(Ws0 + (single_chunk ? 0 : (st & 1) * w_words)), M_T,
+                                    tapoff + (ch + 1 == chunks ? pl.KC16 : 0),
+                                    Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, pl.KC16,
+                                    (cc * pl.nf + 15) >> 4, l32, half);
       else
       multiply_taps<MT, NT>(acc, Ws0 + (single_chunk ? 0 : (st & 1) * w_words) + l32 * pl.WSS + half, 32 * pl.WSS,
                             tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
+    // the next stage's fragments: its buffer was last read two stages ago
+    if (SPLIT && !single_chunk && st + 1 < my_stages) store_filter(next_filter, 0, Ws0 + ((st + 1) & 1) * w_words);
   }
   if (my_stages > 0) epilogue();
 #undef pl
@@ -522,18 +576,54 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   *lds_bytes = 4 * (2 * (size_t)pl.CC * pl.R * pl.RS + (single ? 1 : 2) * (size_t)M_T * pl.WSS +
                     pl.KCp + M_T);
   if (*lds_bytes > 76 * 1024) return false;
-  // the bf16 matrix cores: when the whole filter is one chunk and its fragments fit
+  // the bf16 matrix cores: the filter block as fragments (6 bytes per word, taps padded to
+  // a multiple of 16), built by 256 threads of two 8-tap items each
   pl.split = 0;
   pl.KC16 = 0;
-  const int kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
-  auto split_lds = [&](int sbuf) {
-    return 4 * ((((size_t)sbuf * pl.CC * pl.R * pl.RS) + 3) & ~(size_t)3) + (size_t)6 * kc16 * M_T +
-           4 * (size_t)(kc16 + M_T);
+  pl.f_bytes = 0;
+  const i64 f_extent = 4 * ((pr.c_out - 1) * pr.f_m + (pr.c_in - 1) * pr.f_c + nf);
+  auto split_lds = [&](int sbuf, i64 ccs, bool one_chunk) {
+    const size_t kc16 = (size_t)((ccs * pl.nf + 15) / 16) * 16;
+    return 4 * ((((size_t)sbuf * ccs * pl.R * pl.RS) + 3) & ~(size_t)3) + (one_chunk ? 1 : 2) * 6 * kc16 * M_T +
+           4 * (4 * kc16 + M_T);
   };
-  if (pr.math == MATH_BF16X3 && single && split_lds(2) <= 76 * 1024) {
-    pl.split = 1;
-    pl.KC16 = kc16;
-    *lds_bytes = split_lds(2);
+  if (pr.math == MATH_BF16X3 && f_extent <= ((i64)1 << 30)) {
+    const i64 item_cap = (2 * kThreads * 8) / M_T;         // taps per chunk the two items per thread cover
+    if (single) {
+      const i64 kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
+      if (split_lds(2, pl.C, true) <= 76 * 1024) {
+        pl.split = 1;
+        pl.KC16 = (int)kc16;
+        *lds_bytes = split_lds(2, pl.C, true);
+      }
+    } else {
+      // chunks: the largest that fits the LDS of a workgroup (two to a CU with two position
+      // tiles per wavefront, else three), preferring among the top few the one whose taps
+      // fill their multiple of 16 best
+      const size_t budget = *nt == 2 ? 79 * 1024 : 52 * 1024;
+      i64 best = 0;
+      double best_fill = 0;
+      for (i64 c = std::min<i64>(pl.C, 64); c >= 1; --c) {
+        const i64 kc16 = ((c * pl.nf + 15) / 16) * 16;
+        if (kc16 > item_cap || split_lds(2, c, false) > budget) continue;
+        if (best && c < best - 3) break;
+        const i64 n_chunks = (pl.C + c - 1) / c;
+        const i64 last = pl.C - (n_chunks - 1) * c;
+        // matrix steps executed per channel against 1/16 per tap
+        const double fill = (double)(pl.C * pl.nf) /
+                            (double)((n_chunks - 1) * kc16 + ((last * pl.nf + 15) / 16) * 16);
+        if (!best || fill > best_fill + 1e-9) { best = c; best_fill = fill; }
+      }
+      if (best >= 2 && best * pl.R < ((i64)1 << 22)) {
+        pl.split = 1;
+        pl.CC = (int)best;
+        pl.KC16 = (int)(((best * pl.nf + 15) / 16) * 16);
+        pl.KCp = ((pl.CC * pl.nf + 1) / 2) * 2;
+        pl.WSS = pl.KCp + 1;
+        *lds_bytes = split_lds(2, best, pl.CC >= pl.C);
+      }
+    }
+    if (pl.split) pl.f_bytes = (unsigned)f_extent;
   }
   // A launch small enough that every tile gets a workgroup of its own once the
   // second signal buffer is dropped (more workgroups fit per CU) runs as one
@@ -541,7 +631,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // in which most of the chip idles.
   pl.sbuf = 2;
   if (single) {
-    const size_t one = pl.split ? split_lds(1) : *lds_bytes - 4 * (size_t)pl.CC * pl.R * pl.RS;
+    const size_t one = pl.split ? split_lds(1, pl.C, true) : *lds_bytes - 4 * (size_t)pl.CC * pl.R * pl.RS;
     const i64 slots2 = 256 * (i64)workgroups_per_cu(*lds_bytes, *mt, *nt, pl.split);
     const i64 slots1 = 256 * (i64)workgroups_per_cu(one, *mt, *nt, pl.split);
     const i64 wgs = (i64)pl.total_tiles * m_tiles;

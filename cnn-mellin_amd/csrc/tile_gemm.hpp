@@ -35,7 +35,8 @@ struct TilePlan {
   int KCp;                         // CC * nf rounded up to even
   int WSS;                         // stride of the K-major filter block (words)
   int split;                       // products on the bf16 matrix cores, operands as three bf16 parts each
-  int KC16;                        // split: C * nf rounded up to a multiple of 16
+  int KC16;                        // split: CC * nf rounded up to a multiple of 16
+  unsigned f_bytes;                // split: bytes from the filter's first word to its last one's end
 };
 
 // force_nt: 0 lets the plan pick the number of 32-position tiles per wavefront

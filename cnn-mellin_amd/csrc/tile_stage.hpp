@@ -439,13 +439,13 @@ __device__ __forceinline__ void store_frag(uintx4 *frag, int groups, int rows, i
 // The matrix-core loop of multiply_taps on the bf16 cores: the filter block comes as
 // fragments (store_frag: rows = M_T channels, K = KC16 taps, zero past the last tap),
 // the signal words are read as in multiply_taps, eight taps per lane and step (lane half
-// h takes taps 16 s + 8 h ..), and split in registers.  tp[k] is valid for k < KC16.
+// h takes taps 16 s + 8 h ..), and split in registers.  tp[k] is valid for k < KC16;
+// `steps` steps of 16 taps are multiplied (KC16 / 16, or fewer for a shorter chunk).
 template <int MT, int NT>
 __device__ __forceinline__ void multiply_taps_split(floatx16 (&acc)[MT][NT], const uintx4 *frag, int m_rows,
                                                     const int *tp, const float *Gs, const int (&lane_base)[NT],
-                                                    int KC16, int l32, int half) {
+                                                    int KC16, int steps, int l32, int half) {
   const int groups = KC16 >> 3;
-  const int steps = KC16 >> 4;
   struct Ops { uintx4 ah[MT], am[MT], al[MT], bh[NT], bm[NT], bl[NT]; };
   auto fetch = [&](int s, Ops &o) {
     const int g = 2 * s + half;
