@@ -112,6 +112,9 @@ class Layer:
         self.out = torch.empty_like(self.go)
         self.gi = torch.empty_like(self.x)
         self.gw = torch.empty_like(self.w)
+        nbytes = hip.lib.mellin_corr2d_forward_workspace(kind_x, 4, *self.dims)
+        self.ws_fwd = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        self.ws_fwd_bytes = nbytes
         nbytes = hip.lib.mellin_corr2d_backward_weight_workspace(kind_x, 4, *self.dims)
         self.ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
         self.ws_bytes = nbytes
@@ -123,7 +126,8 @@ class Layer:
 
     def forward(self):
         import _mellin_hip as hip
-        hip.corr2d_forward(self.kind_x, self.x, self.w, self.b, self.out, self.dims)
+        hip.corr2d_forward(self.kind_x, self.x, self.w, self.b, self.out, self.dims,
+                           workspace=self.ws_fwd, workspace_bytes=self.ws_fwd_bytes)
 
     def backward_input(self):
         import _mellin_hip as hip

@@ -47,6 +47,8 @@ SYMBOLS = {
     "mellin_corr2d_backward_input_workspace": (_size_t, [_int, _int] + _DIMS),
     "mellin_log_lift_backward_workspace": (_size_t, [_int, _i64, _i64, _i64]),
 }
+SYMBOLS["mellin_corr2d_forward_workspace"] = (_size_t, [_int, _int] + _DIMS)
+SYMBOLS["mellin_corr2d_forward_ws_f32"] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
 SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
@@ -218,7 +220,10 @@ def _same_dtype(*tensors):
 ACT_NONE, ACT_RELU = 0, 1
 
 
-def corr2d_forward(kind_x, input, weight, bias, out, dims, activation=ACT_NONE):
+def corr2d_forward(kind_x, input, weight, bias, out, dims, activation=ACT_NONE, workspace=None,
+                   workspace_bytes=None):
+    """Forward pass; float32 scratch memory (the filter's bf16 fragments of wide layers) comes
+    from `workspace` or, if None, from torch's caching allocator on the launch stream."""
     dev = require_device(input, weight, bias, out)
     _same_dtype(input, weight, bias, out)
     with torch.cuda.device(dev):
@@ -227,6 +232,13 @@ def corr2d_forward(kind_x, input, weight, bias, out, dims, activation=ACT_NONE):
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
             _check(lib.mellin_corr2d_forward_act_f16(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims,
                                                      _dp(out), _ptr(ws.data_ptr()), need, _stream(dev)))
+        elif out.dtype == torch.float32:
+            if workspace is None:
+                workspace_bytes = lib.mellin_corr2d_forward_workspace(kind_x, 4, *dims)
+                workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=dev)
+                             if workspace_bytes else None)
+            _check(lib.mellin_corr2d_forward_ws_f32(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims,
+                                                    _dp(out), _dp(workspace), workspace_bytes or 0, _stream(dev)))
         else:
             fn = getattr(lib, "mellin_corr2d_forward_act_" + suffix(out.dtype))
             _check(fn(kind_x, activation, _dp(input), _dp(weight), _dp(bias), *dims, _dp(out), _stream(dev)))

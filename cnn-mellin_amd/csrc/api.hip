@@ -96,7 +96,8 @@ int check_counts(const char *fn, double a, double b, double c) {
 // sizes within its plan limits), otherwise one thread per output.
 template <typename T>
 hipError_t run_sepconv(const SepConv &pr, const T *f, const T *g, const T *bias,
-                       T *h, hipStream_t stream) {
+                       T *h, hipStream_t stream, void *frag_ws = nullptr, size_t frag_bytes = 0) {
+  (void)frag_ws; (void)frag_bytes;
   g_variant = "generic";
   g_last_math = MATH_FP32;
   return launch_sepconv_generic<T>(pr, f, g, bias, h, stream);
@@ -104,7 +105,8 @@ hipError_t run_sepconv(const SepConv &pr, const T *f, const T *g, const T *bias,
 
 template <>
 hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
-                              const float *bias, float *h, hipStream_t stream) {
+                              const float *bias, float *h, hipStream_t stream, void *frag_ws,
+                              size_t frag_bytes) {
   if (g_forced != 1) {
     TilePlan pl;
     size_t lds = 0;
@@ -112,7 +114,9 @@ hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
     if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
       g_variant = "mfma";
       g_last_math = pl.split ? MATH_BF16X3 : MATH_FP32;
-      return launch_tile_gemm(pl, lds, mt, nt, f, g, bias, h, stream);
+      // scratch memory for the filter's bf16 fragments, when the caller brought enough
+      const bool use_ws = frag_ws && ((uintptr_t)frag_ws & 15) == 0 && frag_bytes >= tile_fragment_bytes(pl, mt);
+      return launch_tile_gemm(pl, lds, mt, nt, f, g, bias, h, stream, use_ws ? (float *)frag_ws : nullptr);
     }
   }
   g_variant = "generic";
@@ -180,13 +184,24 @@ SepConv forward_problem(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64
   return pr;
 }
 
+// Scratch bytes with which the tiled kernel keeps the filter of problem `pr` as bf16
+// fragments (0: it would not use any).
+size_t fragment_bytes(const SepConv &pr) {
+  if (g_forced == 1) return 0;
+  TilePlan pl;
+  size_t lds = 0;
+  int mt = 0, nt = 0;
+  if (!make_tile_plan(pr, pl, &lds, &mt, &nt)) return 0;
+  return tile_fragment_bytes(pl, mt);
+}
+
 template <typename T>
 int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
                    const T *bias, i64 batch, i64 c_in, i64 c_out, i64 nfx,
                    i64 nfy, i64 ngx, i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy,
                    i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, T *out,
                    void *stream, int activation = MELLIN_ACT_NONE, void *half_out = nullptr,
-                   bool *wrote_half = nullptr) {
+                   bool *wrote_half = nullptr, void *workspace = nullptr, size_t workspace_bytes = 0) {
   int rc = check_corr2d(fn, kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx,
                         nhy, sx, sy, dx, dy, px, py, ux, uy);
   if (rc) return rc;
@@ -225,7 +240,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
     }
     pr.out_half = 0;
   }
-  return check_hip(run_sepconv<T>(pr, weight, input, bias, out, (hipStream_t)stream), fn);
+  return check_hip(run_sepconv<T>(pr, weight, input, bias, out, (hipStream_t)stream, workspace, workspace_bytes), fn);
 }
 
 // grad_input[n, ci, gx, gy] = sum_{co, fx, fy} weight[co, ci, fx, fy] *
@@ -244,6 +259,7 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
 struct TwoPassInput {
   TilePlan plan;
   size_t lds, ws_bytes;
+  size_t frag_off, frag_bytes;     // the first pass's filter fragments, behind Y in the workspace
   int mt, nt;
   Axis fold;
 };
@@ -278,6 +294,9 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
   tp.fold = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
   tp.ws_bytes = (size_t)(batch * m2 * nhx * ngy) * sizeof(float);
+  tp.frag_bytes = tile_fragment_bytes(tp.plan, tp.mt);
+  tp.frag_off = (tp.ws_bytes + 255) & ~(size_t)255;
+  if (tp.frag_bytes) tp.ws_bytes = tp.frag_off + tp.frag_bytes;
   return true;
 }
 
@@ -287,6 +306,25 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
 // kMaxWorkspaceBytes is not taken, and the gather form (tiled or one thread per output),
 // which needs none, is the last resort.
 enum InputForm { IN_GATHER = 0, IN_FUSED, IN_TAPS, IN_TWO_PASS };
+
+// The gather form: the convolution with the roles of signal and output exchanged,
+// "signal" = grad_out (length nh), "output" = grad_input (length ng), weight read transposed.
+SepConv input_gather_problem(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx, i64 ngy,
+                             i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy) {
+  const i64 nf = nfx * nfy, ng = ngx * ngy, nh = nhx * nhy;
+  const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
+  SepConv pr;
+  pr.x = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
+  pr.y = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
+  if (c_out * nf * nh == 0) pr.x.nh_eff = 0;
+  pr.batch = batch; pr.c_out = c_in; pr.c_in = c_out;
+  pr.f_m = nf; pr.f_c = c_in * nf;
+  pr.g_n = c_out * nh; pr.g_c = nh;
+  pr.h_n = c_in * ng; pr.h_m = ng;
+  pr.accumulate = 0;
+  pr.math = g_math;
+  return pr;
+}
 struct InputPlans {
   IgradPlan fused;
   TapProductPlan taps;
@@ -315,6 +353,9 @@ int choose_input_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 n
     ips.ws_bytes = ips.two.ws_bytes;
     return IN_TWO_PASS;
   }
+  // (optional for the gather form: without it the kernel splits the filter itself)
+  ips.ws_bytes = fragment_bytes(input_gather_problem(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy,
+                                                     sx, sy, dx, dy, px, py, ux, uy));
   return IN_GATHER;
 }
 
@@ -367,24 +408,16 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
       g_last_math = tp.plan.split ? MATH_BF16X3 : MATH_FP32;
       hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight,
                                       (const float *)grad_out, nullptr, (float *)workspace,
-                                      (hipStream_t)stream);
+                                      (hipStream_t)stream,
+                                      tp.frag_bytes ? (float *)((char *)workspace + tp.frag_off) : nullptr);
       if (e == hipSuccess)
         e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)workspace,
                           (float *)grad_input, (hipStream_t)stream);
       return check_hip(e, fn);
     }
   }
-  SepConv pr;
-  // roles: "signal" = grad_out (length nh), "output" = grad_input (length ng)
-  pr.x = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
-  pr.y = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
-  if (c_out * nf * nh == 0) pr.x.nh_eff = 0;
-  pr.batch = batch; pr.c_out = c_in; pr.c_in = c_out;
-  pr.f_m = nf; pr.f_c = c_in * nf;                              // weight read transposed
-  pr.g_n = c_out * nh; pr.g_c = nh;
-  pr.h_n = c_in * ng; pr.h_m = ng;
-  pr.accumulate = 0;
-  pr.math = g_math;
+  SepConv pr = input_gather_problem(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy,
+                                    px, py, ux, uy);
   if (half_out && sizeof(T) == 4 && g_forced != 1) {
     // as in the forward pass: the matrix-core kernel stores half precision itself
     TilePlan pl;
@@ -401,7 +434,7 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
     pr.out_half = 0;
   }
   return check_hip(run_sepconv<T>(pr, weight, grad_out, (const T *)nullptr, grad_input,
-                                  (hipStream_t)stream), fn);
+                                  (hipStream_t)stream, workspace, workspace_bytes), fn);
 }
 
 template <typename T>
@@ -792,6 +825,24 @@ int mellin_corr2d_forward_f64(int kind_x, const double *input, const double *wei
                               const double *bias, MELLIN_CORR2D_DIMS, double *out,
                               void *stream) {
   return corr2d_forward<double>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream);
+}
+size_t mellin_corr2d_forward_workspace(int kind_x, int elem_bytes, MELLIN_CORR2D_DIMS) {
+  if (elem_bytes != 4) return 0;
+  if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
+  if (!batch || !c_in || !c_out || !nfx || !nfy || !ngx || !ngy || !nhx || !nhy) return 0;
+  return fragment_bytes(forward_problem(kind_x, CORR2D_ARGS));
+}
+int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input, const float *weight,
+                                 const float *bias, MELLIN_CORR2D_DIMS, float *out, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  const size_t need = mellin_corr2d_forward_workspace(kind_x, 4, CORR2D_ARGS);
+  if (need && (!workspace || workspace_bytes < need))
+    return fail(MELLIN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", __func__, need,
+                workspace_bytes);
+  if (need && ((uintptr_t)workspace & 15))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: the workspace must be 16-byte aligned", __func__);
+  return corr2d_forward<float>(__func__, kind_x, input, weight, bias, CORR2D_ARGS, out, stream, activation, nullptr,
+                               nullptr, workspace, workspace_bytes);
 }
 size_t mellin_corr2d_backward_input_workspace(int kind_x, int elem_bytes,
                                               MELLIN_CORR2D_DIMS) {

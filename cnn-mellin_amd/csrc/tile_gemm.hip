@@ -54,11 +54,12 @@ namespace {
 // three bf16 parts (tile_stage.hpp).  The filter block then lives in LDS as fragments:
 // built once per workgroup when the channels are one chunk, otherwise per stage (the next
 // chunk's filter words are requested into registers before a stage's multiplies and split
-// into the other fragment buffer after them).
+// into the other fragment buffer after them), or, when AF holds the whole filter as
+// fragments already (filter_fragments_kernel), copied from there by direct loads.
 template <int MT, int NT, bool ACC, int MB, bool HOUT, bool SPLIT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
-    const float *__restrict__ bias, float *__restrict__ H) {
+    const float *__restrict__ bias, float *__restrict__ H, const float *__restrict__ AF) {
   // The plan is read where it lies, in the kernel-argument segment (it is the
   // first argument), through a pointer the compiler must treat as new in every
   // iteration of the stage loop: fields are then re-read by scalar loads where
@@ -160,6 +161,15 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     }
   };
 
+  // (SPLIT) the fragments of chunk ch of this block's channels, ready-made in AF
+  auto copy_fragments = [&](int ch, int ws_word) {
+    const float *src = AF + ((i64)blockIdx.y * chunks + ch) * w_words;
+    const int bytes = 4 * w_words;                       // a multiple of 16
+    for (int at = wave_id * 1024; at < bytes; at += kWaves * 1024)
+      if (at + 16 * lane < bytes)
+        load16_to_lds_at(src, (unsigned)(at + 16 * lane), lds_base + 4u * (unsigned)ws_word + (unsigned)at);
+  };
+
   // ---- stages owned by this workgroup ------------------------------------------
   // tiles blockIdx.x, blockIdx.x + gridDim.x, ...; each tile has `chunks` stages
   const int my_tiles = (int)blockIdx.x < pl.total_tiles
@@ -180,6 +190,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     issue_signal<kWaves, kMemo>(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave,
                                &memo, ch == 0, ch < 2);
     if (!SPLIT && !single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
+    if (SPLIT && !single_chunk && AF) copy_fragments(ch, ws_word0 + (st & 1) * w_words);
   };
 
   // ---- SPLIT: the filter block as fragments ----------------------------------------
@@ -254,7 +265,8 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     if (SPLIT) {
       __syncthreads();                                    // the offset tables
       // (a filter that is one chunk may have more items than one round of the threads)
-      for (int first = 0; first < f_groups * M_T; first += kFilterItems * kThreads) {
+      if (!single_chunk && AF) copy_fragments(0, ws_word0);
+      else for (int first = 0; first < f_groups * M_T; first += kFilterItems * kThreads) {
         FilterWords fw;
         load_filter(0, first, fw);
         store_filter(fw, first, Ws0);
@@ -276,6 +288,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   constexpr int ES = HOUT ? 2 : 4;                      // bytes per stored element
   const i64 hm1 = pl.h_m * ES, hm2 = 2 * hm1, hm3 = 3 * hm1, hm8 = 8 * hm1;
   const bool full_m = m0 + M_T <= pl.M;
+  const bool buffer_stores = (i64)(M_T + 8) * hm1 < ((i64)1 << 31);    // 32-bit offsets inside a block's channels
   const int m_left = pl.M - m0 - half * 4;              // channels from this lane's first row on
   // They run one stage late, after the next stage's loads are issued and before
   // its multiplies, so that they drain behind the next matrix loop.
@@ -292,6 +305,26 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
         live = live && ox < pl.nox_eff && oy < pl.noy_eff;
       }
       if (!live) continue;
+      if (FULL && !ACC && !HOUT && buffer_stores) {
+        // One descriptor for the block's channels of this image; a lane's offset is its
+        // position plus whole groups of eight channels, the four channels inside a group
+        // are scalar offsets: a store and a quarter of a 32-bit add per word, against a
+        // store and a 64-bit add with pointers.
+        const __amdgpu_buffer_rsrc_t h_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void *)Himg, 0, (int)(M_T * hm1), 0x00020000);
+        int voff = (half * 4) * (int)hm1 + lane_q[t] * 4;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 0]), h_rsrc, voff, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 1]), h_rsrc, voff, (int)hm1, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 2]), h_rsrc, voff, (int)hm2, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 3]), h_rsrc, voff, (int)hm3, 0);
+            voff += (int)hm8;
+          }
+        continue;
+      }
       char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * ES;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
@@ -358,10 +391,9 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       // then between the matrix instructions of its SIMD's other wavefronts)
       __builtin_amdgcn_s_setprio(3);
       issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
-      if (SPLIT && !single_chunk) load_filter(ch + 1 == chunks ? 0 : ch + 1, 0, next_filter);
+      if (SPLIT && !single_chunk && !AF) load_filter(ch + 1 == chunks ? 0 : ch + 1, 0, next_filter);
       __builtin_amdgcn_s_setprio(0);
     }
-
     if (ch == 0) {
       if (st > 0) epilogue();                             // the tile finished one stage ago
       tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
@@ -404,15 +436,40 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
                             tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
     // the next stage's fragments: its buffer was last read two stages ago
-    if (SPLIT && !single_chunk && st + 1 < my_stages) store_filter(next_filter, 0, Ws0 + ((st + 1) & 1) * w_words);
+    if (SPLIT && !single_chunk && !AF && st + 1 < my_stages) store_filter(next_filter, 0, Ws0 + ((st + 1) & 1) * w_words);
   }
   if (my_stages > 0) epilogue();
 #undef pl
 }
 
+// The whole filter as fragments, once per launch, in the order the stages of the SPLIT
+// kernel copy them: AF[m_tile][chunk][part][group][row] (16-byte words).  One thread per
+// (m_tile, chunk, group, row): eight taps of one output channel, split, three stores.
+__global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int M_T, int chunks,
+                                                               const float *__restrict__ F,
+                                                               uintx4 *__restrict__ AF) {
+  const int groups = pl.KC16 >> 3;
+  const int per_block = groups * M_T;
+  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 blocks = (i64)((pl.M + M_T - 1) / M_T) * chunks;
+  if (idx >= blocks * per_block) return;
+  const int blk = (int)(idx / per_block), within = (int)(idx - (i64)blk * per_block);
+  const int m_tile = blk / chunks, ch = blk - m_tile * chunks;
+  const int m = within / groups, g = within - m * groups;
+  const int cc = min(pl.CC, pl.C - ch * pl.CC), row = m_tile * M_T + m;
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int k = 8 * g + i, cl = k / pl.nf, t = k - cl * pl.nf;
+    x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + t] : 0.f;
+  }
+  store_frag(AF + (i64)blk * 3 * per_block, groups, M_T, g, m, x);
+}
+
 template <int MT, int NT, bool ACC, int MB, bool HOUT = false, bool SPLIT = false>
 hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const float *f,
-                          const float *g, const float *bias, float *h, hipStream_t stream) {
+                          const float *g, const float *bias, float *h, hipStream_t stream,
+                          const float *af = nullptr) {
   auto kern = tile_gemm_kernel<MT, NT, ACC, MB, HOUT, SPLIT>;
   if (lds_bytes > 64 * 1024) {
     // opt in to more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per CU)
@@ -424,7 +481,7 @@ hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const
       granted = lds_bytes;
     }
   }
-  hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, pl, f, g, bias, h);
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, pl, f, g, bias, h, af);
   return hipGetLastError();
 }
 
@@ -640,10 +697,27 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   return true;
 }
 
+size_t tile_fragment_bytes(const TilePlan &pl, int mt) {
+  const int chunks = (pl.C + pl.CC - 1) / pl.CC;
+  if (!pl.split || chunks < 2) return 0;
+  const size_t m_tiles = (size_t)((pl.M + mt * 32 - 1) / (mt * 32));
+  return m_tiles * chunks * 3 * (size_t)(pl.KC16 >> 3) * (mt * 32) * 16;
+}
+
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
-                            float *h, hipStream_t stream) {
+                            float *h, hipStream_t stream, float *frag_ws) {
   const int M_T = mt * 32;
+  const float *af = nullptr;
+  if (frag_ws && tile_fragment_bytes(pl, mt)) {
+    const int chunks = (pl.C + pl.CC - 1) / pl.CC;
+    const i64 items = (i64)tile_fragment_bytes(pl, mt) / 48;
+    hipLaunchKernelGGL(filter_fragments_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pl, M_T,
+                       chunks, f, (uintx4 *)frag_ws);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    af = frag_ws;
+  }
   // persistent workgroups: as many as fit at once on the 256 CUs
   const int m_tiles = (pl.M + M_T - 1) / M_T;
   const int per_cu = workgroups_per_cu(lds_bytes, mt, nt, pl.split);
@@ -656,9 +730,9 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
     if (pl.split) {                                                                          \
-      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream); \
-      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, true>(pl, lds_bytes, grid, f, g, bias, h, stream);   \
-      return launch_variant<MT_, NT_, false, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream);                   \
+      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \
+      return launch_variant<MT_, NT_, false, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
     }                                                                                        \
     if (pl.accumulate)                                                                       \
       return memo ? launch_variant<MT_, NT_, true, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)  \

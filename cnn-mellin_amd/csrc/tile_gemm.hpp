@@ -43,9 +43,16 @@ struct TilePlan {
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt,
                     int force_nt = 0);
 
+// Bytes of scratch memory in which a launch keeps the filter as bf16 fragments, block by
+// block as the stages read them (0: the layer does not run on the bf16 matrix cores, or
+// its filter is one block, which every workgroup builds for itself).  Without that
+// scratch every workgroup splits each block again in every tile.
+size_t tile_fragment_bytes(const TilePlan &pl, int mt);
+
+// frag_ws: tile_fragment_bytes() of device memory, 16-byte aligned, or null
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
-                            float *h, hipStream_t stream);
+                            float *h, hipStream_t stream, float *frag_ws = nullptr);
 
 // Weight gradient (wgrad_gemm.hip): position tiling and signal staging of the
 // forward problem in `t`, plus the blocking of the (c_out) x (c_in * taps) output.

@@ -915,7 +915,10 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
   // (rows of 5 and 7: 12 % and 25 %).  On a Mellin axis its tiles stage a virtual row per
   // (row, filter row) pair for only 128 positions and the row-wise kernel stays ahead.
   const int min_row = mellin_x ? 4 : 8;
-  if (wp.split && !pl.segment && pl.ay == 1 && pl.uy == 1 && pl.by == 1 && pl.nfy <= 8 && pl.noy >= 8 &&
+  // (Linear x axis only: on a Mellin axis a unit's fragments cover a virtual row per (row,
+  // filter row) pair, most of them without a tap, and the fp32 row-wise kernel measured
+  // 10-65 % faster on the 64..256-channel layers of the 10-layer stack.)
+  if (wp.split && !mellin_x && !pl.segment && pl.ay == 1 && pl.uy == 1 && pl.by == 1 && pl.nfy <= 8 && pl.noy >= 8 &&
       pl.nox_eff >= 1 && g_allow_rows && (i64)pl.M * pl.Q < ((i64)1 << 30)) {
     // The bf16 form (wgrad_stream_kernel): grad_out goes through registers, LDS holds the
     // fragments of the input rows a unit needs.  The largest unit whose fragment tasks a

@@ -195,6 +195,20 @@ int mellin_corr2d_forward_act_f64(int kind_x, int activation, const double *inpu
                                   const double *weight, const double *bias,
                                   MELLIN_CORR2D_DIMS, double *out, void *stream);
 
+/* The same forward pass with scratch memory.  Layers whose input channels are staged
+ * in several chunks multiply on the bf16 matrix cores from a copy of the filter cut
+ * into bf16 parts (MELLIN_MATH_BF16X3); with `workspace` that copy is made once per
+ * call, without it every workgroup makes its own for every tile (same result bit for
+ * bit, up to 20 % slower on wide layers).  mellin_corr2d_forward_workspace() gives the
+ * bytes (0 for layers that need none; the buffer 16-byte aligned); the entry points
+ * without a workspace argument stay valid.  Replaces, like them, the adapter call
+ * ext/torch_cuda.cu:144-177. */
+size_t mellin_corr2d_forward_workspace(int kind_x, int elem_bytes, MELLIN_CORR2D_DIMS);
+int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input,
+                                 const float *weight, const float *bias,
+                                 MELLIN_CORR2D_DIMS, float *out, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+
 /* Half precision (the data type the reference's Autocast registration casts to,
  * ext/torch.cpp:407-430, before it calls the CUDA kernels instantiated for
  * c10::Half, ext/torch_cuda.cu:45-177): tensors hold IEEE binary16 values in

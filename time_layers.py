@@ -144,11 +144,15 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("config", choices=["cfg2", "cfg4", "stack"])
     ap.add_argument("--reps", type=int, default=10, help="timed calls per pass")
+    ap.add_argument("--math", choices=["bf16x3", "fp32"], default="bf16x3",
+                    help="how the matrix kernels form fp32 products (library default: bf16x3)")
     args = ap.parse_args()
     import torch
     if not torch.cuda.is_available():
         sys.exit("time_layers.py needs a GPU")
     torch.cuda.set_device(0)
+    import _mellin_hip as hip
+    hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
     {"cfg2": run_cfg2, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps)
 
 
