@@ -96,12 +96,13 @@ def set_variant(name=None):
     _check(lib.mellin_set_variant((name or "").encode()))
 
 
-MATH_FP32, MATH_BF16X3 = 0, 1
+MATH_FP32, MATH_BF16X3, MATH_BF16X3_ALWAYS = 0, 1, 2
 
 
 def set_math(mode):
     """MATH_BF16X3 (default): fp32 products as six bf16 products of three-part operands, fp32
-    accumulate; MATH_FP32: the fp32 matrix instructions."""
+    accumulate; MATH_FP32: the fp32 matrix instructions; MATH_BF16X3_ALWAYS: the bf16 form also
+    for layers so small that the default leaves them on the fp32 instructions."""
     _check(lib.mellin_set_math(int(mode)))
 
 

@@ -772,7 +772,7 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
 }
 
 int mellin_set_math(int mode) {
-  if (mode != MELLIN_MATH_FP32 && mode != MELLIN_MATH_BF16X3)
+  if (mode != MELLIN_MATH_FP32 && mode != MELLIN_MATH_BF16X3 && mode != MELLIN_MATH_BF16X3_ALWAYS)
     return fail(MELLIN_ERR_ARGUMENT, "mellin_set_math: unknown mode %d", mode);
   g_math = mode;
   return MELLIN_OK;

@@ -980,7 +980,7 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
   Th = std::min(Th, std::max(H, min_th));
   pl.stream = 0;
   pl.rw = 0;
-  if (math == MATH_BF16X3 && mtn == 1 && c_in <= 3 && (nf & 7) == 0 && c_out * nh < ((i64)1 << 29) &&
+  if (math != MATH_FP32 && mtn == 1 && c_in <= 3 && (nf & 7) == 0 && c_out * nh < ((i64)1 << 29) &&
       pl.batched_fold && force_nt == 0 && force_Th == 0 &&
       force_pipe != 0 && ngx + px + reach + sx < ((i64)1 << 22) && batch * c_in <= 65535 &&
       (reach - sx + 1) * ngy < ((i64)1 << 22)) {

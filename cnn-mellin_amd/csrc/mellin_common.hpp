@@ -36,7 +36,7 @@ struct SepConv {
   int math = 0;                  // MATH_FP32: fp32 matrix instructions; MATH_BF16X3: bf16 ones on three-part operands
 };
 
-enum MathMode : int { MATH_FP32 = 0, MATH_BF16X3 = 1 };
+enum MathMode : int { MATH_FP32 = 0, MATH_BF16X3 = 1, MATH_BF16X3_ALWAYS = 2 };   // ALWAYS: no size heuristics
 
 // Reduction form used by the weight gradient:
 // w[m, c, fx, fy] = sum_{n, hx, hy} a[n, m, hx, hy] * g[n, c, tap_x(hx, fx), tap_y(hy, fy)]

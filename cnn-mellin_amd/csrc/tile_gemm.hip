@@ -538,7 +538,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     // full one's rate (measured), so the smaller tile wins when it fills its last round
     // that much better.
     const i64 big = pr.batch * ((Q + 255) / 256) * m_tiles, small = pr.batch * ((Q + 127) / 128) * m_tiles;
-    const bool want_split = pr.math == MATH_BF16X3;
+    const bool want_split = pr.math != MATH_FP32;
     const i64 slots_big = 256 * (want_split ? 2 : 3), slots_small = 256 * (want_split ? 3 : 4);
     const double fill_big = (double)big / (double)(((big + slots_big - 1) / slots_big) * slots_big);
     const double fill_small = (double)small / (double)(((small + slots_small - 1) / slots_small) * slots_small);
@@ -644,7 +644,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     return 4 * ((((size_t)sbuf * ccs * pl.R * pl.RS) + 3) & ~(size_t)3) + (one_chunk ? 1 : 2) * 6 * kc16 * M_T +
            4 * (4 * kc16 + M_T);
   };
-  if (pr.math == MATH_BF16X3 && f_extent <= ((i64)1 << 30)) {
+  if (pr.math != MATH_FP32 && f_extent <= ((i64)1 << 30)) {
     const i64 item_cap = (2 * kThreads * 8) / M_T;         // taps per chunk the two items per thread cover
     if (single) {
       const i64 kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
@@ -653,7 +653,10 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
         pl.KC16 = (int)kc16;
         *lds_bytes = split_lds(2, pl.C, true);
       }
-    } else {
+    } else if (pr.math == MATH_BF16X3_ALWAYS ||
+               (double)pr.batch * (double)Q * (double)pr.c_out * (double)pr.c_in * (double)nf >= 8e8) {
+      // (layers under 0.8 GMAC (virtual rows counted) stay on the fp32 instructions: config 2's 1-D Mellin layers,
+      // 0.12-0.52 GMAC, measured 25-60 % slower with fragments staged per chunk)
       // chunks: the largest that fits the LDS of a workgroup (two to a CU with two position
       // tiles per wavefront, else three), preferring among the top few the one whose taps
       // fill their multiple of 16 best

@@ -881,7 +881,7 @@ bool make_wgrad_plan(const SepConv &fwd_in, WgradPlan &wp, bool g_allow_rows, in
   // (the forward tiling is only borrowed for its staging geometry: plan it for the fp32 kernel)
   SepConv fwd = fwd_in;
   fwd.math = MATH_FP32;
-  wp.split = fwd_in.math == MATH_BF16X3;
+  wp.split = fwd_in.math != MATH_FP32;
   // narrower column blocks touch fewer input channels and so need less LDS
   for (int jt_max = 3; jt_max >= 1; --jt_max)
     if (make_wgrad_plan_jt(fwd, wp, g_allow_rows, rows_opt_mt, rows_opt_nbuf, rows_opt_rpw, jt_max)) return true;

@@ -332,10 +332,14 @@ const char *mellin_last_variant(void);
  *     rounding of an fp32 multiply-add.  Storage, accumulation and results are fp32.
  *   MELLIN_MATH_FP32  the fp32 matrix instructions (v_mfma_f32_32x32x2_f32), one sixth of
  *     the multiply rate.
- * Kernels that have no bf16 form yet run in fp32 under either setting.  Infinities in
- * the operands give NaN under MELLIN_MATH_BF16X3 (inf - inf while splitting). */
+ *   MELLIN_MATH_BF16X3_ALWAYS  as MELLIN_MATH_BF16X3, also for layers so small that the
+ *     default leaves them on the fp32 instructions because those are faster there (layers
+ *     staged in chunks of channels under 0.8 GMAC): for tests and comparisons.
+ * Kernels that have no bf16 form yet run in fp32 under any setting.  Infinities in
+ * the operands give NaN under the bf16 modes (inf - inf while splitting). */
 #define MELLIN_MATH_FP32 0
 #define MELLIN_MATH_BF16X3 1
+#define MELLIN_MATH_BF16X3_ALWAYS 2
 int mellin_set_math(int mode);
 int mellin_get_math(void);
 /* The mode the matrix kernels of the most recent operator-level call actually ran in

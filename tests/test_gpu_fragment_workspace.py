@@ -15,11 +15,12 @@ from oracle import oracle
 pytestmark = pytest.mark.gpu
 
 CASES = [
-    # (kind, n, c_in, c_out, nf, ng, s, d, p)
-    (hip.AX_LCORR, 2, 160, 70, (3, 3), (33, 30), (1, 1), (2, 1), (2, 1)),     # tail chunk, 70 of 96 channels
-    (hip.AX_LCORR, 3, 96, 128, (4, 4), (40, 12), (1, 1), (1, 1), (1, 1)),
-    (hip.AX_MCORR, 2, 100, 40, (4, 4), (40, 9), (1, 1), (1, 1), (1, 1)),
-    (hip.AX_MCORR, 2, 64, 64, (3, 4), (60, 24), (2, 1), (1, 1), (1, 2)),      # wide Mellin: two-pass input gradient
+    # (kind, n, c_in, c_out, nf, ng, s, d, p): each above the size from which layers staged in chunks
+    # take the bf16 cores (0.8 GMAC)
+    (hip.AX_LCORR, 4, 160, 96, (3, 3), (40, 41), (1, 1), (2, 1), (2, 1)),     # a short last chunk
+    (hip.AX_LCORR, 6, 96, 128, (4, 4), (48, 20), (1, 1), (1, 1), (1, 1)),
+    (hip.AX_MCORR, 8, 128, 128, (4, 4), (120, 14), (1, 1), (1, 1), (1, 1)),   # wide Mellin: two-pass input gradient
+    (hip.AX_MCORR, 6, 96, 128, (3, 4), (200, 24), (2, 1), (1, 1), (1, 2)),
 ]
 
 

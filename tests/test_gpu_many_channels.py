@@ -58,8 +58,18 @@ def _run(kind_x, x, w, b, go, s, d, p, u):
     return out, gi, gw, (v_out, v_gi, v_gw)
 
 
+@pytest.fixture(params=["default", "bf16x3-always"])
+def math_mode(request):
+    """The default math mode leaves layers this small on the fp32 matrix instructions;
+    MATH_BF16X3_ALWAYS sends them through the bf16 form of the chunked kernel as well
+    (per-stage filter fragments, a short last chunk, padded taps)."""
+    hip.set_math(hip.MATH_BF16X3_ALWAYS if request.param == "bf16x3-always" else hip.MATH_BF16X3)
+    yield request.param
+    hip.set_math(hip.MATH_BF16X3)
+
+
 @pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
-def test_chunked_layers_match_checker(case):
+def test_chunked_layers_match_checker(case, math_mode):
     op, n, c_in, c_out, nf, ng, s, d, p, u, r = case
     kind_x, fwd, bwd = OPS[op]
     rng = np.random.default_rng(2000 + CASES.index(case))
@@ -73,6 +83,10 @@ def test_chunked_layers_match_checker(case):
     egi, egw, _ = bwd(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64), s, d, p, u)
     out, gi, gw, variants = _run(kind_x, x, w, b, go, s, d, p, u)
     assert all(v.startswith("mfma") for v in variants), variants
+    if math_mode == "bf16x3-always":
+        hip.corr2d_forward(kind_x, to_gpu(x), to_gpu(w), to_gpu(b), torch.empty_like(out), hip._dims(
+            n, c_in, c_out, nf, ng, tuple(nh), s, d, p, u))
+        assert hip.last_math() == hip.MATH_BF16X3
     assert_close(out, exp, c_in * nf[0] * nf[1], "out %s" % (case,))
     assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
     assert_close(gw, egw, n * nh[0] * nh[1], "grad_weight %s" % (case,))
@@ -109,7 +123,7 @@ SHORT_RUN_CASES = [
 
 
 @pytest.mark.parametrize("case", SHORT_RUN_CASES, ids=[str(i) for i in range(len(SHORT_RUN_CASES))])
-def test_block_copies_of_under_four_words(case):
+def test_block_copies_of_under_four_words(case, math_mode):
     op, n, c_in, c_out, nf, ng, s, d, p, u, r = case
     kind_x, fwd, bwd = OPS[op]
     rng = np.random.default_rng(3000 + SHORT_RUN_CASES.index(case))
