@@ -50,13 +50,14 @@ namespace {
 // channels fit in one or two chunks).
 // HOUT: H is half-precision storage (not with ACC): the fp32 results are rounded to
 // nearest even as they are stored.
-// SPLIT: the products run on the bf16 matrix cores, every fp32 operand as the exact sum of
+// SPLIT (1: the channels are one chunk, 2: several): the products run on the bf16 matrix
+// cores, every fp32 operand as the exact sum of
 // three bf16 parts (tile_stage.hpp).  The filter block then lives in LDS as fragments:
 // built once per workgroup when the channels are one chunk, otherwise per stage (the next
 // chunk's filter words are requested into registers before a stage's multiplies and split
 // into the other fragment buffer after them), or, when AF holds the whole filter as
 // fragments already (filter_fragments_kernel), copied from there by direct loads.
-template <int MT, int NT, bool ACC, int MB, bool HOUT, bool SPLIT>
+template <int MT, int NT, bool ACC, int MB, bool HOUT, int SPLIT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H, const float *__restrict__ AF) {
@@ -79,7 +80,9 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
   const int ws_word0 = SPLIT ? (pl.sbuf * g_words + 3) & ~3 : pl.sbuf * g_words;
   float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS], or the fragments
-  const bool single_chunk = pl.CC >= pl.C;
+  // (a constant for the bf16 instances: the code that builds fragments per stage costs the
+  // one-chunk kernel 24 registers and 6 % of its time when it is merely compiled in)
+  const bool single_chunk = SPLIT ? SPLIT == 1 : pl.CC >= pl.C;
   // SPLIT keeps four tables of KC16 words: signal offset of tap k of a whole chunk and of
   // the last (shorter) chunk, and the same two for the filter word's byte offset
   const int n_tapoff = SPLIT ? 4 * pl.KC16 : pl.KCp;
@@ -466,7 +469,7 @@ __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int 
   store_frag(AF + (i64)blk * 3 * per_block, groups, M_T, g, m, x);
 }
 
-template <int MT, int NT, bool ACC, int MB, bool HOUT = false, bool SPLIT = false>
+template <int MT, int NT, bool ACC, int MB, bool HOUT = false, int SPLIT = 0>
 hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const float *f,
                           const float *g, const float *bias, float *h, hipStream_t stream,
                           const float *af = nullptr) {
@@ -648,7 +651,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     const i64 item_cap = (2 * kThreads * 8) / M_T;         // taps per chunk the two items per thread cover
     if (single) {
       const i64 kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
-      if (split_lds(2, pl.C, true) <= 76 * 1024) {
+      if (split_lds(2, pl.C, true) <= 79 * 1024) {
         pl.split = 1;
         pl.KC16 = (int)kc16;
         *lds_bytes = split_lds(2, pl.C, true);
@@ -732,10 +735,15 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
+    if (pl.split && pl.CC >= pl.C) {                                                         \
+      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \
+      return launch_variant<MT_, NT_, false, 0, false, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+    }                                                                                        \
     if (pl.split) {                                                                          \
-      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
-      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \
-      return launch_variant<MT_, NT_, false, 0, false, true>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+      if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, 2>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, 2>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \
+      return launch_variant<MT_, NT_, false, 0, false, 2>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
     }                                                                                        \
     if (pl.accumulate)                                                                       \
       return memo ? launch_variant<MT_, NT_, true, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)  \
