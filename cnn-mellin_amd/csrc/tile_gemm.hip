@@ -629,6 +629,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     if (cc > 64) cc = 64;
   }
   if (cc * pl.R >= ((i64)1 << 22)) return false;
+  if (cc * ng >= lim) return false;                               // 32-bit byte offsets across a chunk's channels
   pl.CC = (int)cc;
   pl.KCp = ((pl.CC * pl.nf + 1) / 2) * 2;
   pl.WSS = pl.KCp + 1;                                             // odd: 32 channels -> 32 banks
@@ -677,7 +678,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
                             (double)((n_chunks - 1) * kc16 + ((last * pl.nf + 15) / 16) * 16);
         if (!best || fill > best_fill + 1e-9) { best = c; best_fill = fill; }
       }
-      if (best >= 2 && best * pl.R < ((i64)1 << 22)) {
+      if (best >= 2 && best * pl.R < ((i64)1 << 22) && best * ng < lim) {
         pl.split = 1;
         pl.CC = (int)best;
         pl.KC16 = (int)(((best * pl.nf + 15) / 16) * 16);

@@ -151,10 +151,33 @@ struct StageMemo {
 // further on and lands cl planes further on.
 __device__ __forceinline__ void load_channels(const float *base, int g_c, unsigned voff, unsigned lds_addr,
                                               unsigned plane_bytes, int cc) {
-  for (int cl = 0; cl < cc; ++cl) {
-    load_to_lds_at(base, voff, lds_addr);
-    base += g_c;
-    lds_addr += plane_bytes;
+  // One instruction slot is all a staging wavefront gets between the matrix instructions of
+  // its SIMD's other wavefront, so the loop is cut to what it needs: the LDS target goes to
+  // M0, the lane's byte offset moves on by a channel (which also fills the wait state that
+  // M0 wants before the load), the load.  (Offsets stay below 2^32: callers check
+  // cc * g_c < 2^30.)
+  const unsigned long long b = (unsigned long long)base;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  const unsigned step = __builtin_amdgcn_readfirstlane(4u * (unsigned)g_c);
+  const unsigned pb = __builtin_amdgcn_readfirstlane(plane_bytes);
+  unsigned v = voff - step;
+  unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  cc = __builtin_amdgcn_readfirstlane(cc);           // wave-uniform: say so, or the loop's scalars end up in vector registers
+  int cl = 0;
+  for (; cl + 4 <= cc; cl += 4) {                    // four channels per block of straight-line code
+    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3"
+                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase), "s"(pb) : "memory", "scc");
+    m0v = __builtin_amdgcn_readfirstlane(m0v + 4u * pb);
+  }
+  for (; cl < cc; ++cl) {
+    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3"
+                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase) : "memory");
+    m0v = __builtin_amdgcn_readfirstlane(m0v + pb);
   }
 }
 __device__ __forceinline__ void zero_channels(float *at, int plane, int cc) {
