@@ -171,11 +171,12 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
 // ---- half <-> float copies (the half-precision entry points compute in fp32) ------
 namespace {
 
-// eight elements per thread where the run allows 16-byte accesses, singly otherwise
+// eight elements per thread where the run and the pointers (vec) allow 16-byte accesses,
+// singly otherwise
 __global__ __launch_bounds__(kPwThreads) void half_to_float_kernel(const _Float16 *__restrict__ src,
-                                                                   float *__restrict__ dst, i64 n) {
+                                                                   float *__restrict__ dst, i64 n, bool vec) {
   const i64 i0 = ((i64)blockIdx.x * kPwThreads + threadIdx.x) * 8;
-  if (i0 + 8 <= n) {
+  if (vec && i0 + 8 <= n) {
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
     const half8 v = *(const half8 *)(src + i0);
     float4 a = make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
@@ -183,14 +184,14 @@ __global__ __launch_bounds__(kPwThreads) void half_to_float_kernel(const _Float1
     *(float4 *)(dst + i0) = a;
     *(float4 *)(dst + i0 + 4) = b;
   } else {
-    for (i64 i = i0; i < n; ++i) dst[i] = (float)src[i];
+    for (i64 i = i0; i < min(i0 + 8, n); ++i) dst[i] = (float)src[i];
   }
 }
 
 __global__ __launch_bounds__(kPwThreads) void float_to_half_kernel(const float *__restrict__ src,
-                                                                   _Float16 *__restrict__ dst, i64 n) {
+                                                                   _Float16 *__restrict__ dst, i64 n, bool vec) {
   const i64 i0 = ((i64)blockIdx.x * kPwThreads + threadIdx.x) * 8;
-  if (i0 + 8 <= n) {
+  if (vec && i0 + 8 <= n) {
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
     const float4 a = *(const float4 *)(src + i0), b = *(const float4 *)(src + i0 + 4);
     half8 v;
@@ -198,27 +199,29 @@ __global__ __launch_bounds__(kPwThreads) void float_to_half_kernel(const float *
     v[4] = (_Float16)b.x; v[5] = (_Float16)b.y; v[6] = (_Float16)b.z; v[7] = (_Float16)b.w;
     *(half8 *)(dst + i0) = v;
   } else {
-    for (i64 i = i0; i < n; ++i) dst[i] = (_Float16)src[i];
+    for (i64 i = i0; i < min(i0 + 8, n); ++i) dst[i] = (_Float16)src[i];
   }
 }
 
 }  // namespace
 
-// src and dst must be 16-byte aligned (torch allocations and 256-byte aligned
-// workspace regions are)
+// 16-byte accesses when both pointers are 16-byte aligned (torch allocations and the
+// workspace regions are; a view into a half tensor may start at any even address)
 hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   const i64 blocks = (n + 8 * kPwThreads - 1) / (8 * kPwThreads);
+  const bool vec = (((uintptr_t)src | (uintptr_t)dst) & 15) == 0;
   hipLaunchKernelGGL(half_to_float_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream,
-                     (const _Float16 *)src, dst, n);
+                     (const _Float16 *)src, dst, n, vec);
   return hipGetLastError();
 }
 
 hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   const i64 blocks = (n + 8 * kPwThreads - 1) / (8 * kPwThreads);
+  const bool vec = (((uintptr_t)src | (uintptr_t)dst) & 15) == 0;
   hipLaunchKernelGGL(float_to_half_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, src,
-                     (_Float16 *)dst, n);
+                     (_Float16 *)dst, n, vec);
   return hipGetLastError();
 }
 

@@ -171,3 +171,40 @@ def test_half_results_are_the_fp32_results_rounded_once(shape):
     gi16 = torch.empty_like(x)
     hip.corr2d_backward_input(kind_x, w, go, gi16, dims)
     assert torch.equal(gi16, gi32.half())
+
+
+def test_half_views_at_odd_offsets():
+    """Half tensors that start at any even address (a slice of a flat buffer, a cat gradient):
+    the copies between half and fp32 then go element by element instead of 16 bytes at a time.
+    All three passes must give bit for bit what the same operands give from aligned storage."""
+    kind, n, c_in, c_out, nf, ng, s, d, p, u, r = CASES[1]
+    rng = np.random.default_rng(42)
+    x = torch.from_numpy(rng.standard_normal((n, c_in) + ng).astype(np.float16))
+    w = torch.from_numpy((rng.standard_normal((c_out, c_in) + nf) * 0.1).astype(np.float16))
+    b = torch.from_numpy(rng.standard_normal(c_out).astype(np.float16))
+    nh = (mconv.lcorr_valid_size(nf[0], ng[0]), mconv.lcorr_valid_size(nf[1], ng[1]))
+    go = torch.from_numpy(rng.standard_normal((n, c_out) + nh).astype(np.float16))
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, u)
+
+    def shifted(t, off):
+        """the same values in storage that starts `off` halves past a 256-byte boundary"""
+        flat = torch.empty(t.numel() + 8, dtype=torch.float16, device="cuda")
+        view = flat[off:off + t.numel()].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == (2 * off) % 16
+        return view
+
+    def run(off):
+        xg, wg, bg, gog = (shifted(t, off) for t in (x, w, b, go))
+        out = shifted(torch.zeros((n, c_out) + nh, dtype=torch.float16), off)
+        gi = shifted(torch.zeros_like(x), off)
+        gw = shifted(torch.zeros_like(w), off)
+        hip.corr2d_forward(hip.AX_LCORR, xg, wg, bg, out, dims)
+        hip.corr2d_backward_input(hip.AX_LCORR, wg, gog, gi, dims)
+        hip.corr2d_backward_weight(hip.AX_LCORR, xg, gog, gw, dims)
+        return out.clone(), gi.clone(), gw.clone()
+
+    aligned = run(0)
+    for off in (1, 3):
+        for a, c in zip(aligned, run(off)):
+            assert torch.equal(a, c)
