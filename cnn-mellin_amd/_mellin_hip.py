@@ -71,6 +71,9 @@ for _t in ("f32", "f64"):
     SYMBOLS["mellin_log_lift_forward_" + _t] = (_int, [_ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr])
     SYMBOLS["mellin_log_lift_backward_" + _t] = (
         _int, [_ptr, _ptr, _dbl, _dbl, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
+    SYMBOLS["mellin_log_lift_forward_dev_" + _t] = (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr])
+    SYMBOLS["mellin_log_lift_backward_dev_" + _t] = (
+        _int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
     SYMBOLS["mellin_corr2d_forward_act_" + _t] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_forward_" + _t] = (_int, [_int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
     SYMBOLS["mellin_corr2d_backward_input_" + _t] = (
@@ -193,6 +196,28 @@ def log_lift_forward(x, eps, tau, flags, outer, t, inner, y):
     with torch.cuda.device(dev):
         _check(fn(_dp(x), float(eps), float(tau), flags, outer, t, inner, _dp(y), _stream(dev)))
     return y
+
+
+def log_lift_forward_dev(x, params, flags, outer, t, inner, y):
+    """As log_lift_forward with params = (eps, tau) in a device tensor of x's type: no copy to the host."""
+    dev = require_device(x, params, y)
+    _same_dtype(x, params, y)
+    fn = getattr(lib, "mellin_log_lift_forward_dev_" + suffix(y.dtype, half_ok=False))
+    with torch.cuda.device(dev):
+        _check(fn(_dp(x), _dp(params), flags, outer, t, inner, _dp(y), _stream(dev)))
+    return y
+
+
+def log_lift_backward_dev(x, grad_y, params, flags, outer, t, inner, grad_x, grad_params):
+    dev = require_device(x, grad_y, params, grad_x, grad_params)
+    _same_dtype(x, grad_y, params, grad_x, grad_params)
+    fn = getattr(lib, "mellin_log_lift_backward_dev_" + suffix(grad_x.dtype, half_ok=False))
+    need = lib.mellin_log_lift_backward_workspace(grad_x.element_size(), outer, t, inner)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(fn(_dp(x), _dp(grad_y), _dp(params), flags, outer, t, inner, _dp(grad_x),
+                  _ptr(grad_params.data_ptr()), _ptr(ws.data_ptr()), need, _stream(dev)))
+    return grad_x, grad_params
 
 
 def log_lift_backward(x, grad_y, eps, tau, flags, outer, t, inner, grad_x, grad_params):

@@ -569,13 +569,13 @@ int check_log_lift(const char *fn, double eps, int flags, i64 outer, i64 t, i64 
 
 template <typename T>
 int log_lift_forward(const char *fn, const T *x, double eps, double tau, int flags, i64 outer, i64 t, i64 inner,
-                     T *y, void *stream) {
+                     T *y, void *stream, const T *params = nullptr) {
   int rc;
   if ((rc = check_log_lift(fn, eps, flags, outer, t, inner))) return rc;
   if (outer * t * inner == 0) return MELLIN_OK;
   if (!x || !y) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
   hipError_t e = launch_log_lift_forward<T>(x, (T)eps, (T)tau, flags & MELLIN_PW_LOG, flags & MELLIN_PW_LIFT,
-                                            outer, t, inner, y, (hipStream_t)stream);
+                                            outer, t, inner, y, (hipStream_t)stream, params);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
   return MELLIN_OK;
 }
@@ -583,7 +583,7 @@ int log_lift_forward(const char *fn, const T *x, double eps, double tau, int fla
 template <typename T>
 int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, double tau, int flags, i64 outer,
                       i64 t, i64 inner, T *gx, T *grad_params, void *workspace, size_t workspace_bytes,
-                      void *stream) {
+                      void *stream, const T *params = nullptr) {
   int rc;
   if ((rc = check_log_lift(fn, eps, flags, outer, t, inner))) return rc;
   if (!grad_params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
@@ -593,7 +593,7 @@ int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, doubl
     return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, need, workspace_bytes);
   hipError_t e = launch_log_lift_backward<T>(x, gy, (T)eps, (T)tau, flags & MELLIN_PW_LOG, flags & MELLIN_PW_LIFT,
                                              outer, t, inner, gx, grad_params, (T *)workspace,
-                                             (hipStream_t)stream);
+                                             (hipStream_t)stream, params);
   if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
   return MELLIN_OK;
 }
@@ -754,6 +754,31 @@ int mellin_log_lift_forward_f32(const float *x, double eps, double tau, int flag
 int mellin_log_lift_forward_f64(const double *x, double eps, double tau, int flags, int64_t outer, int64_t t,
                                 int64_t inner, double *y, void *stream) {
   return log_lift_forward<double>("mellin_log_lift_forward_f64", x, eps, tau, flags, outer, t, inner, y, stream);
+}
+// eps and tau on the device: params = {eps, tau}
+int mellin_log_lift_forward_dev_f32(const float *x, const float *params, int flags, int64_t outer, int64_t t,
+                                    int64_t inner, float *y, void *stream) {
+  if (!params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  return log_lift_forward<float>(__func__, x, 1.0, 0.0, flags, outer, t, inner, y, stream, params);
+}
+int mellin_log_lift_forward_dev_f64(const double *x, const double *params, int flags, int64_t outer, int64_t t,
+                                    int64_t inner, double *y, void *stream) {
+  if (!params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  return log_lift_forward<double>(__func__, x, 1.0, 0.0, flags, outer, t, inner, y, stream, params);
+}
+int mellin_log_lift_backward_dev_f32(const float *x, const float *grad_y, const float *params, int flags,
+                                     int64_t outer, int64_t t, int64_t inner, float *grad_x, float *grad_params,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+  if (!params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  return log_lift_backward<float>(__func__, x, grad_y, 1.0, 0.0, flags, outer, t, inner, grad_x, grad_params,
+                                  workspace, workspace_bytes, stream, params);
+}
+int mellin_log_lift_backward_dev_f64(const double *x, const double *grad_y, const double *params, int flags,
+                                     int64_t outer, int64_t t, int64_t inner, double *grad_x, double *grad_params,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+  if (!params) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+  return log_lift_backward<double>(__func__, x, grad_y, 1.0, 0.0, flags, outer, t, inner, grad_x, grad_params,
+                                   workspace, workspace_bytes, stream, params);
 }
 size_t mellin_log_lift_backward_workspace(int elem_bytes, int64_t outer, int64_t t, int64_t inner) {
   return log_lift_workspace_bytes(outer, t, inner, (size_t)elem_bytes);

@@ -136,17 +136,18 @@ bool launch_col2spec_padded(const Axis &x, const Axis &y, i64 pairs, i64 taps_pa
 hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pad, const float *Z,
                           float *grad_input, hipStream_t stream);
 
-// pointwise.hip: log compression and dilation lift over x viewed as (outer, t, inner)
+// pointwise.hip: log compression and dilation lift over x viewed as (outer, t, inner).
+// params (device memory, or null): {eps, tau} read by the kernels instead of the arguments
 size_t log_lift_workspace_bytes(i64 outer, i64 t, i64 inner, size_t elem);
 template <typename T>
 hipError_t launch_log_lift_forward(const T *x, T eps, T tau, bool with_log, bool with_lift, i64 outer, i64 t,
-                                   i64 inner, T *y, hipStream_t stream);
+                                   i64 inner, T *y, hipStream_t stream, const T *params = nullptr);
 template <typename T>
 hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool with_log, bool with_lift,
                                     i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
-                                    hipStream_t stream);
+                                    hipStream_t stream, const T *params = nullptr);
 
-// half <-> float copies of n elements (16-byte aligned buffers)
+// half <-> float copies of n elements (16 bytes at a time when both buffers are 16-byte aligned)
 hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream);
 hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream);
 

@@ -27,10 +27,11 @@ template <typename T> __device__ __forceinline__ T sign_of(T v) { return v > T(0
 
 template <typename T, bool LOG, bool LIFT>
 __global__ __launch_bounds__(kPwThreads) void log_lift_forward_kernel(
-    const T *__restrict__ x, T eps, T tau, i64 outer, i64 plane, i64 inner, i64 rows_per_block,
-    T *__restrict__ y) {
+    const T *__restrict__ x, T eps, T tau, const T *__restrict__ params, i64 outer, i64 plane, i64 inner,
+    i64 rows_per_block, T *__restrict__ y) {
   const i64 col = (i64)blockIdx.x * kPwThreads + threadIdx.x;      // t * inner + i
   if (col >= plane) return;
+  if (params) { eps = params[0]; tau = params[1]; }               // the values live on the device
   T p = T(1);
   if (LIFT) p = pow((T)(col / inner + 1), tau);
   const i64 n0 = (i64)blockIdx.y * rows_per_block, n1 = min(outer, n0 + rows_per_block);
@@ -44,9 +45,10 @@ __global__ __launch_bounds__(kPwThreads) void log_lift_forward_kernel(
 // grad_x, and partial sums of d/d eps and d/d tau per block (two values per block)
 template <typename T, bool LOG, bool LIFT>
 __global__ __launch_bounds__(kPwThreads) void log_lift_backward_kernel(
-    const T *__restrict__ x, const T *__restrict__ gy, T eps, T tau, i64 outer, i64 plane, i64 inner,
-    i64 rows_per_block, T *__restrict__ gx, T *__restrict__ partial) {
+    const T *__restrict__ x, const T *__restrict__ gy, T eps, T tau, const T *__restrict__ params, i64 outer,
+    i64 plane, i64 inner, i64 rows_per_block, T *__restrict__ gx, T *__restrict__ partial) {
   __shared__ T red[2][kPwThreads / 64];
+  if (params) { eps = params[0]; tau = params[1]; }
   const i64 col = (i64)blockIdx.x * kPwThreads + threadIdx.x;
   T s_eps = T(0), s_tau = T(0);
   if (col < plane) {
@@ -128,14 +130,14 @@ size_t log_lift_workspace_bytes(i64 outer, i64 t, i64 inner, size_t elem) {
 
 template <typename T>
 hipError_t launch_log_lift_forward(const T *x, T eps, T tau, bool with_log, bool with_lift, i64 outer, i64 t,
-                                   i64 inner, T *y, hipStream_t stream) {
+                                   i64 inner, T *y, hipStream_t stream, const T *params) {
   if (outer <= 0 || t <= 0 || inner <= 0) return hipSuccess;
   dim3 grid;
   i64 rpb;
   shape_grid(outer, t * inner, grid, rpb);
 #define MELLIN_PW_FWD(L_, F_)                                                                    \
   hipLaunchKernelGGL((log_lift_forward_kernel<T, L_, F_>), grid, dim3(kPwThreads), 0, stream, x, \
-                     eps, tau, outer, t * inner, inner, rpb, y)
+                     eps, tau, params, outer, t * inner, inner, rpb, y)
   if (with_log && with_lift) MELLIN_PW_FWD(true, true);
   else if (with_log) MELLIN_PW_FWD(true, false);
   else MELLIN_PW_FWD(false, true);
@@ -146,7 +148,7 @@ hipError_t launch_log_lift_forward(const T *x, T eps, T tau, bool with_log, bool
 template <typename T>
 hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool with_log, bool with_lift,
                                     i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
-                                    hipStream_t stream) {
+                                    hipStream_t stream, const T *params) {
   if (outer <= 0 || t <= 0 || inner <= 0) {
     hipLaunchKernelGGL((log_lift_reduce_kernel<T>), dim3(1), dim3(64), 0, stream, workspace, (i64)0, grad_params);
     return hipGetLastError();
@@ -156,7 +158,7 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
   shape_grid(outer, t * inner, grid, rpb);
 #define MELLIN_PW_BWD(L_, F_)                                                                     \
   hipLaunchKernelGGL((log_lift_backward_kernel<T, L_, F_>), grid, dim3(kPwThreads), 0, stream, x, \
-                     gy, eps, tau, outer, t * inner, inner, rpb, gx, workspace)
+                     gy, eps, tau, params, outer, t * inner, inner, rpb, gx, workspace)
   if (with_log && with_lift) MELLIN_PW_BWD(true, true);
   else if (with_log) MELLIN_PW_BWD(true, false);
   else MELLIN_PW_BWD(false, true);
@@ -226,12 +228,13 @@ hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t 
 }
 
 template hipError_t launch_log_lift_forward<float>(const float *, float, float, bool, bool, i64, i64, i64,
-                                                   float *, hipStream_t);
+                                                   float *, hipStream_t, const float *);
 template hipError_t launch_log_lift_forward<double>(const double *, double, double, bool, bool, i64, i64, i64,
-                                                    double *, hipStream_t);
+                                                    double *, hipStream_t, const double *);
 template hipError_t launch_log_lift_backward<float>(const float *, const float *, float, float, bool, bool, i64,
-                                                    i64, i64, float *, float *, float *, hipStream_t);
+                                                    i64, i64, float *, float *, float *, hipStream_t, const float *);
 template hipError_t launch_log_lift_backward<double>(const double *, const double *, double, double, bool, bool,
-                                                     i64, i64, i64, double *, double *, double *, hipStream_t);
+                                                     i64, i64, i64, double *, double *, double *, hipStream_t,
+                                                     const double *);
 
 }  // namespace mellin

@@ -48,22 +48,26 @@ class _LogLiftFunction(torch.autograd.Function):
         for v in shape[dim + 1:]:
             inner *= v
         t = shape[dim] if x.dim() else 1
-        eps_v = float(eps) if eps is not None else 1.0
-        tau_v = float(tau) if tau is not None else 0.0
+        # eps and tau are device values (exp of the modules' parameters): they go to the
+        # kernels as a two-element device tensor, not through float(), which would wait
+        # for the device and cannot be captured in a graph
+        one, zero = x.new_ones(()), x.new_zeros(())
+        params = torch.stack([eps.detach().to(device=x.device, dtype=x.dtype).reshape(()) if eps is not None else one,
+                              tau.detach().to(device=x.device, dtype=x.dtype).reshape(()) if tau is not None else zero])
         y = torch.empty_like(x)
-        _hip.log_lift_forward(x, eps_v, tau_v, flags, outer, t, inner, y)
-        ctx.save_for_backward(x, eps if isinstance(eps, torch.Tensor) else None,
+        _hip.log_lift_forward_dev(x, params, flags, outer, t, inner, y)
+        ctx.save_for_backward(x, params, eps if isinstance(eps, torch.Tensor) else None,
                               tau if isinstance(tau, torch.Tensor) else None)
-        ctx.geometry = (eps_v, tau_v, flags, outer, t, inner)
+        ctx.geometry = (flags, outer, t, inner)
         return y
 
     @staticmethod
     def backward(ctx, grad_y):
-        x, eps, tau = ctx.saved_tensors
-        eps_v, tau_v, flags, outer, t, inner = ctx.geometry
+        x, params, eps, tau = ctx.saved_tensors
+        flags, outer, t, inner = ctx.geometry
         grad_x = torch.empty_like(x)
         grad_params = torch.empty(2, dtype=x.dtype, device=x.device)
-        _hip.log_lift_backward(x, grad_y.contiguous(), eps_v, tau_v, flags, outer, t, inner, grad_x, grad_params)
+        _hip.log_lift_backward_dev(x, grad_y.contiguous(), params, flags, outer, t, inner, grad_x, grad_params)
         g_eps = grad_params[0].to(eps.dtype).reshape(eps.shape) if eps is not None and ctx.needs_input_grad[1] else None
         g_tau = grad_params[1].to(tau.dtype).reshape(tau.shape) if tau is not None and ctx.needs_input_grad[2] else None
         return grad_x, g_eps, g_tau, None, None

@@ -315,6 +315,27 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
                                  void *workspace, size_t workspace_bytes,
                                  void *stream);
 
+/* The same with eps and tau in DEVICE memory, params = {eps, tau} in the tensors' type
+ * (an unused one is ignored): for values that are themselves results of device work --
+ * the reference modules' exp(log_eps), exp(log_tau) -- so that a call needs no copy to
+ * the host and can be captured in a graph.  eps > 0 is not checked then. */
+int mellin_log_lift_forward_dev_f32(const float *x, const float *params, int flags,
+                                    int64_t outer, int64_t t, int64_t inner,
+                                    float *y, void *stream);
+int mellin_log_lift_forward_dev_f64(const double *x, const double *params, int flags,
+                                    int64_t outer, int64_t t, int64_t inner,
+                                    double *y, void *stream);
+int mellin_log_lift_backward_dev_f32(const float *x, const float *grad_y,
+                                     const float *params, int flags, int64_t outer,
+                                     int64_t t, int64_t inner, float *grad_x,
+                                     float *grad_params, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+int mellin_log_lift_backward_dev_f64(const double *x, const double *grad_y,
+                                     const double *params, int flags, int64_t outer,
+                                     int64_t t, int64_t inner, double *grad_x,
+                                     double *grad_params, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
 /* Name of the kernel variant the most recent operator-level call of the
  * process (on any thread: PyTorch runs backward passes on a thread of its own)
  * dispatched to (for tests and profiling): "generic", "mfma" (tiled

@@ -50,3 +50,47 @@ def test_forward_and_both_gradients_replay_identically(kind):
         x2 = torch.randn_like(x)                          # unrelated eager work between replays
         hip.corr2d_forward(kind, x2, w, b, torch.empty_like(out), dims)
         torch.cuda.synchronize()
+
+
+def test_pointwise_layers_are_capturable():
+    """log compression + dilation lift with eps = exp(log_eps), tau = exp(log_tau) computed on the
+    device: the values reach the kernels through device memory, so neither the forward nor the
+    backward pass waits for the device, and both can be recorded and replayed."""
+    import layers
+    torch.manual_seed(3)
+    x = torch.randn(6, 3, 50, 17, device="cuda")
+    gy = torch.randn_like(x)
+    log_eps = torch.tensor(-1.0, device="cuda", requires_grad=True)
+    log_tau = torch.tensor(0.3, device="cuda", requires_grad=True)
+    y, gx = torch.empty_like(x), torch.empty_like(x)
+    g_eps, g_tau = torch.empty((), device="cuda"), torch.empty((), device="cuda")
+
+    def step():
+        xi = x.detach().requires_grad_(True)
+        out = layers.log_compression_lift(xi, log_eps.exp(), log_tau.exp(), 2)
+        a, b, c = torch.autograd.grad(out, (xi, log_eps, log_tau), gy)
+        y.copy_(out.detach()); gx.copy_(a); g_eps.copy_(b); g_tau.copy_(c)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                        # warm-up off the default stream, as capture requires
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    ref = [t.clone() for t in (y, gx, g_eps, g_tau)]
+    eps, tau = float(log_eps.detach().exp()), float(log_tau.detach().exp())
+    t = torch.arange(1, 51, device="cuda", dtype=torch.float32).view(1, 1, 50, 1)
+    torch.testing.assert_close(ref[0], t ** tau * torch.log(eps + x.abs()), rtol=1e-5, atol=1e-5)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for buf in (y, gx, g_eps, g_tau):
+            buf.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, exp in zip((y, gx, g_eps, g_tau), ref):
+            assert torch.equal(got, exp), "replay %d differs" % rep
+        layers.log_compression(torch.randn_like(x), torch.tensor(0.5, device="cuda"))   # eager work in between
+        torch.cuda.synchronize()
