@@ -49,6 +49,8 @@ SYMBOLS = {
 }
 SYMBOLS["mellin_corr2d_forward_workspace"] = (_size_t, [_int, _int] + _DIMS)
 SYMBOLS["mellin_corr2d_forward_ws_f32"] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
+SYMBOLS["mellin_bias_grad_workspace"] = (_size_t, [_i64, _i64, _i64])
+SYMBOLS["mellin_bias_grad_f32"] = (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
 SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
@@ -230,6 +232,23 @@ def log_lift_backward(x, grad_y, eps, tau, flags, outer, t, inner, grad_x, grad_
         _check(fn(_dp(x), _dp(grad_y), float(eps), float(tau), flags, outer, t, inner, _dp(grad_x),
                   _ptr(grad_params.data_ptr()), _ptr(ws.data_ptr()), need, _stream(dev)))
     return grad_x, grad_params
+
+
+def bias_grad(grad_out, out=None):
+    """(g, grad_bias) for a dense float32 grad_out (N, C, ...): grad_bias = per-channel sums of g, with
+    g = grad_out, or grad_out where `out` > 0 (the backward of a ReLU fused into the forward pass)."""
+    dev = require_device(grad_out, out)
+    _same_dtype(grad_out, out)
+    n, c = grad_out.shape[0], grad_out.shape[1]
+    plane = grad_out[0, 0].numel() if n and c else 0
+    g = torch.empty_like(grad_out) if out is not None else grad_out
+    grad_bias = torch.empty(c, dtype=grad_out.dtype, device=dev)
+    need = lib.mellin_bias_grad_workspace(n, c, plane)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.mellin_bias_grad_f32(_dp(grad_out), _dp(out), n, c, plane, _dp(g) if out is not None else None,
+                                        _dp(grad_bias), _ptr(ws.data_ptr()), need, _stream(dev)))
+    return g, grad_bias
 
 
 def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):

@@ -796,6 +796,31 @@ int mellin_log_lift_backward_f64(const double *x, const double *grad_y, double e
                                    grad_x, grad_params, workspace, workspace_bytes, stream);
 }
 
+size_t mellin_bias_grad_workspace(int64_t batch, int64_t channels, int64_t plane) {
+  if (batch < 0 || channels < 0 || plane < 0 || batch > 65535 || channels > 65535 || plane > ((int64_t)1 << 40)) return 0;
+  return bias_grad_workspace_bytes(batch, channels, plane);
+}
+int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch, int64_t channels, int64_t plane,
+                         float *grad_masked, float *grad_bias, void *workspace, size_t workspace_bytes,
+                         void *stream) {
+  const char *fn = __func__;
+  if (batch < 0 || channels < 0 || plane < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: negative extent", fn);
+  if (batch > 65535 || channels > 65535 || plane > ((int64_t)1 << 40))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: at most 65535 images and channels (got %lld, %lld)", fn, (long long)batch,
+                (long long)channels);
+  if (channels == 0) return MELLIN_OK;
+  if (!grad_bias) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  const size_t need = bias_grad_workspace_bytes(batch, channels, plane);
+  if (need && (!grad_out || (out && !grad_masked))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  if (need && (!workspace || workspace_bytes < need))
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, need, workspace_bytes);
+  hipError_t e = launch_bias_grad(grad_out, out, batch, channels, plane, grad_masked, grad_bias, (float *)workspace,
+                                  (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
 int mellin_set_math(int mode) {
   if (mode != MELLIN_MATH_FP32 && mode != MELLIN_MATH_BF16X3 && mode != MELLIN_MATH_BF16X3_ALWAYS)
     return fail(MELLIN_ERR_ARGUMENT, "mellin_set_math: unknown mode %d", mode);

@@ -147,6 +147,12 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
                                     i64 outer, i64 t, i64 inner, T *gx, T *grad_params, T *workspace,
                                     hipStream_t stream, const T *params = nullptr);
 
+// pointwise.hip: per-channel sums of grad_out (N, C, plane), optionally masked by out > 0 (the masked
+// gradient is then written to grad_masked); workspace of bias_grad_workspace_bytes()
+size_t bias_grad_workspace_bytes(i64 batch, i64 channels, i64 plane);
+hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, i64 channels, i64 plane,
+                            float *grad_masked, float *grad_bias, float *workspace, hipStream_t stream);
+
 // half <-> float copies of n elements (16 bytes at a time when both buffers are 16-byte aligned)
 hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream);
 hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream);

@@ -170,6 +170,88 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
   return hipGetLastError();
 }
 
+// ---- bias gradient, with the backward of a fused ReLU ---------------------------------
+// grad_bias[c] = sum over images and positions of g[n, c, :], where g = grad_out or, when
+// the layer's ReLU was applied by the forward kernel, grad_out where out > 0 and zero
+// elsewhere (g is then also written: it is what the gradient kernels take).  One pass over
+// the operands; sums in a fixed order: a block adds up 4096 consecutive elements of one
+// (image, channel) plane (lanes strided, a shuffle tree per wavefront, the wavefronts in
+// order), a second kernel adds a channel's blocks in index order.
+namespace {
+
+constexpr int kBiasChunk = 4096;
+
+template <bool MASK>
+__global__ __launch_bounds__(kPwThreads) void bias_grad_kernel(const float *__restrict__ go,
+                                                               const float *__restrict__ out,
+                                                               float *__restrict__ gm, float *__restrict__ partial,
+                                                               i64 plane, int chunks) {
+  __shared__ float red[kPwThreads / 64];
+  const int chunk = blockIdx.x, c = blockIdx.y, n = blockIdx.z, C = gridDim.y, N = gridDim.z;
+  const i64 base = ((i64)n * C + c) * plane + (i64)chunk * kBiasChunk;
+  const int len = (int)min((i64)kBiasChunk, plane - (i64)chunk * kBiasChunk);
+  float s = 0.f;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < len; i += kPwThreads) {
+    float v = go[base + i];
+    if (MASK) {
+      v = out[base + i] > 0.f ? v : 0.f;
+      gm[base + i] = v;
+    }
+    s += v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_down(s, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float a = 0.f;
+    for (int w = 0; w < kPwThreads / 64; ++w) a += red[w];
+    partial[((i64)c * N + n) * chunks + chunk] = a;
+  }
+}
+
+__global__ __launch_bounds__(64) void bias_reduce_kernel(const float *__restrict__ partial, i64 per_channel,
+                                                         float *__restrict__ grad_bias) {
+  const float *p = partial + (i64)blockIdx.x * per_channel;
+  float a = 0.f;
+  for (i64 i = threadIdx.x; i < per_channel; i += 64) a += p[i];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) a += __shfl_down(a, o);
+  if (threadIdx.x == 0) grad_bias[blockIdx.x] = a;
+}
+
+}  // namespace
+
+size_t bias_grad_workspace_bytes(i64 batch, i64 channels, i64 plane) {
+  if (batch <= 0 || channels <= 0 || plane <= 0) return 0;
+  const i64 chunks = (plane + kBiasChunk - 1) / kBiasChunk;
+  return (size_t)(batch * channels * chunks) * sizeof(float);
+}
+
+hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, i64 channels, i64 plane,
+                            float *grad_masked, float *grad_bias, float *workspace, hipStream_t stream) {
+  if (channels <= 0) return hipSuccess;
+  if (batch <= 0 || plane <= 0) {                       // empty sums
+    hipLaunchKernelGGL(bias_reduce_kernel, dim3((unsigned)channels), dim3(64), 0, stream, workspace, (i64)0,
+                       grad_bias);
+    return hipGetLastError();
+  }
+  const i64 chunks = (plane + kBiasChunk - 1) / kBiasChunk;
+  const dim3 grid((unsigned)chunks, (unsigned)channels, (unsigned)batch);
+  if (out)
+    hipLaunchKernelGGL(bias_grad_kernel<true>, grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
+                       workspace, plane, (int)chunks);
+  else
+    hipLaunchKernelGGL(bias_grad_kernel<false>, grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
+                       workspace, plane, (int)chunks);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(bias_reduce_kernel, dim3((unsigned)channels), dim3(64), 0, stream, workspace, batch * chunks,
+                     grad_bias);
+  return hipGetLastError();
+}
+
 // ---- half <-> float copies (the half-precision entry points compute in fp32) ------
 namespace {
 

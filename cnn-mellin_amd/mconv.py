@@ -227,18 +227,28 @@ class _Corr2dFunction(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         input, weight = ctx.saved_tensors[:2]
-        if len(ctx.saved_tensors) == 3:                     # through the fused ReLU: pass where out > 0
-            grad_out = grad_out * (ctx.saved_tensors[2] > 0)
+        out = ctx.saved_tensors[2] if len(ctx.saved_tensors) == 3 else None
         grad_out = grad_out.contiguous()
-        grad_input = grad_weight = grad_bias = None
+        grad_bias = None
+        want_bias = ctx.has_bias and ctx.needs_input_grad[2]
+        if grad_out.dtype == torch.float32 and grad_out.shape[0] <= 65535 and grad_out.shape[1] <= 65535 and \
+                (out is not None or want_bias):
+            # one pass: the backward of the fused ReLU (pass where out > 0) and the bias gradient
+            grad_out, grad_bias = _hip.bias_grad(grad_out, out)
+            if not want_bias:
+                grad_bias = None
+        else:
+            if out is not None:                             # through the fused ReLU: pass where out > 0
+                grad_out = grad_out * (out > 0)
+            if want_bias:
+                grad_bias = grad_out.sum((0, 2, 3))
+        grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
             grad_input = _hip.corr2d_backward_input(
                 ctx.kind_x, weight, grad_out, torch.empty_like(input), ctx.dims)
         if ctx.needs_input_grad[1]:
             grad_weight = _hip.corr2d_backward_weight(
                 ctx.kind_x, input, grad_out, torch.empty_like(weight), ctx.dims)
-        if ctx.has_bias and ctx.needs_input_grad[2]:
-            grad_bias = grad_out.sum((0, 2, 3))
         return grad_input, grad_weight, grad_bias, None, None, None, None, None, None, None, None
 
 

@@ -336,6 +336,20 @@ int mellin_log_lift_backward_dev_f64(const double *x, const double *grad_y,
                                      double *grad_params, void *workspace,
                                      size_t workspace_bytes, void *stream);
 
+/* Bias gradient of a layer, grad_bias[c] = sum over images and positions of
+ * g[n, c, :] for grad_out (batch, channels, plane) -- the reference leaves this to
+ * grad_out.sum(...) (ext/torch.cpp:231,300) -- in one pass together with the backward of
+ * a ReLU that the forward kernel applied (MELLIN_ACT_RELU): with `out` (the layer's
+ * output) given, g = grad_out where out > 0 and 0 elsewhere, and g is written to
+ * grad_masked, the gradient that the backward_input / backward_weight calls then take;
+ * with out == NULL, g = grad_out and grad_masked is not touched.  Sums run in a fixed
+ * order.  At most 65535 images and channels.  Scratch: mellin_bias_grad_workspace(). */
+size_t mellin_bias_grad_workspace(int64_t batch, int64_t channels, int64_t plane);
+int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch,
+                         int64_t channels, int64_t plane, float *grad_masked,
+                         float *grad_bias, void *workspace, size_t workspace_bytes,
+                         void *stream);
+
 /* Name of the kernel variant the most recent operator-level call of the
  * process (on any thread: PyTorch runs backward passes on a thread of its own)
  * dispatched to (for tests and profiling): "generic", "mfma" (tiled

@@ -1,0 +1,65 @@
+"""Bias gradient and the backward of a fused ReLU in one pass (mellin_bias_grad_f32): the masked
+gradient must be grad_out where out > 0 and zero elsewhere, exactly; the per-channel sums are
+compared with float64 sums of the same values at rtol 1e-5 / atol 1e-5 * sqrt(terms) and must not
+change from run to run.  The reference computes both in PyTorch (ext/torch.cpp:231,300 and the
+model's ReLU, models.py:423-425)."""
+import numpy as np
+import pytest
+import torch
+
+import _mellin_hip as hip
+import mconv
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(32, 64, 505, 38), (3, 5, 7, 11), (2, 33, 4097, 1), (1, 1, 1, 1), (5, 7, 4096, 1), (4, 130, 60, 33)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=["x".join(map(str, s)) for s in SHAPES])
+@pytest.mark.parametrize("masked", [True, False], ids=["relu", "plain"])
+def test_bias_grad_matches_float64_sums(shape, masked):
+    torch.manual_seed(sum(shape))
+    go = torch.randn(*shape, device="cuda")
+    out = torch.relu(torch.randn(*shape, device="cuda")) if masked else None
+    g, gb = hip.bias_grad(go, out)
+    exp_g = go * (out > 0) if masked else go
+    assert torch.equal(g, exp_g)
+    if not masked:
+        assert g.data_ptr() == go.data_ptr()                # nothing is copied
+    exp = exp_g.double().sum((0, 2, 3))
+    terms = shape[0] * shape[2] * shape[3]
+    np.testing.assert_allclose(gb.cpu().numpy(), exp.cpu().numpy(), rtol=1e-5, atol=1e-5 * terms ** 0.5)
+    g2, gb2 = hip.bias_grad(go, out)
+    assert torch.equal(gb, gb2) and torch.equal(g, g2)
+
+
+def test_bias_grad_edge_cases():
+    empty = torch.empty(0, 4, 3, 2, device="cuda")
+    g, gb = hip.bias_grad(empty, None)
+    assert gb.shape == (4,) and float(gb.abs().sum()) == 0.0
+    go = torch.randn(2, 3, 5, 5, device="cuda")
+    need = hip.lib.mellin_bias_grad_workspace(2, 3, 25)
+    assert need == 2 * 3 * 4
+    gb = torch.empty(3, device="cuda")
+    rc = hip.lib.mellin_bias_grad_f32(hip._dp(go), None, 2, 3, 25, None, hip._dp(gb), None, 0, hip._stream(go.device))
+    assert rc != 0 and "workspace" in hip.last_error()
+    rc = hip.lib.mellin_bias_grad_f32(hip._dp(go), None, 70000, 3, 25, None, hip._dp(gb), None, 0,
+                                      hip._stream(go.device))
+    assert rc != 0 and "65535" in hip.last_error()
+
+
+def test_layer_backward_uses_it():
+    """Through autograd: bias and fused-ReLU gradients of a layer against PyTorch's own composition."""
+    torch.manual_seed(5)
+    x = torch.randn(4, 3, 40, 21, device="cuda")
+    w = (torch.randn(16, 3, 4, 4, device="cuda") * 0.2).requires_grad_(True)
+    b = (torch.randn(16, device="cuda") * 0.1).requires_grad_(True)
+    y = mconv.lcorrlcorr(x, w, b, activation="relu")
+    gy = torch.randn_like(y)
+    gw, gb = torch.autograd.grad(y, (w, b), gy)
+    w2, b2 = w.detach().clone().requires_grad_(True), b.detach().clone().requires_grad_(True)
+    y2 = torch.relu(torch.nn.functional.conv2d(x, w2, b2))
+    gw2, gb2 = torch.autograd.grad(y2, (w2, b2), gy)
+    torch.testing.assert_close(y, y2, rtol=1e-5, atol=1e-5 * 48 ** 0.5)
+    torch.testing.assert_close(gb, gb2, rtol=1e-4, atol=1e-4 * (4 * 37 * 18) ** 0.5)
+    torch.testing.assert_close(gw, gw2, rtol=1e-4, atol=1e-4 * (4 * 37 * 18) ** 0.5)
