@@ -51,6 +51,8 @@ SYMBOLS["mellin_corr2d_forward_workspace"] = (_size_t, [_int, _int] + _DIMS)
 SYMBOLS["mellin_corr2d_forward_ws_f32"] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_bias_grad_workspace"] = (_size_t, [_i64, _i64, _i64])
 SYMBOLS["mellin_bias_grad_f32"] = (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
+SYMBOLS["mellin_pool_pairs_forward_f32"] = (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr])
+SYMBOLS["mellin_pool_pairs_backward_f32"] = (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr])
 SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
 SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
@@ -249,6 +251,27 @@ def bias_grad(grad_out, out=None):
         _check(lib.mellin_bias_grad_f32(_dp(grad_out), _dp(out), n, c, plane, _dp(g) if out is not None else None,
                                         _dp(grad_bias), _ptr(ws.data_ptr()), need, _stream(dev)))
     return g, grad_bias
+
+
+def pool_pairs_forward(x):
+    """(y, which) for a dense float32 x (..., f): maxima over pairs of neighbours along the last axis."""
+    dev = require_device(x)
+    f = x.shape[-1]
+    rows = x.numel() // f if f else 0
+    y = torch.empty(x.shape[:-1] + (f // 2,), dtype=x.dtype, device=dev)
+    which = torch.empty(y.shape, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.mellin_pool_pairs_forward_f32(_dp(x), rows, f, _dp(y), _dp(which), _stream(dev)))
+    return y, which
+
+
+def pool_pairs_backward(grad_y, which, f):
+    dev = require_device(grad_y, which)
+    grad_x = torch.empty(grad_y.shape[:-1] + (f,), dtype=grad_y.dtype, device=dev)
+    rows = grad_x.numel() // f if f else 0
+    with torch.cuda.device(dev):
+        _check(lib.mellin_pool_pairs_backward_f32(_dp(grad_y), _dp(which), rows, f, _dp(grad_x), _stream(dev)))
+    return grad_x
 
 
 def _dims(batch, c_in, c_out, nf, ng, nh, s, d, p, u):

@@ -18,8 +18,33 @@ from typing import Callable, List, Optional, Sequence, Tuple
 import torch
 
 import mconv
+import _mellin_hip as _hip
 
 __all__ = ["ConvStackParams", "ConvStack", "FrameClassifier", "layer_plan", "pack_windows"]
+
+
+class _FreqMaxPool(torch.autograd.Function):
+    """max_pool2d(x, (1, 2)) for dense float32 GPU tensors through the library's pair kernels:
+    one byte per output is kept for the backward pass instead of PyTorch's 8-byte indices."""
+
+    @staticmethod
+    def forward(ctx, x):
+        y, which = _hip.pool_pairs_forward(x.contiguous())
+        ctx.save_for_backward(which)
+        ctx.f = x.shape[-1]
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        (which,) = ctx.saved_tensors
+        return _hip.pool_pairs_backward(grad_y.contiguous(), which, ctx.f)
+
+
+def freq_max_pool(x: torch.Tensor) -> torch.Tensor:
+    """Maximum over pairs of neighbouring frequency bins, ``max_pool2d(x, (1, 2))``."""
+    if x.is_cuda and x.dtype == torch.float32:
+        return _FreqMaxPool.apply(x)
+    return torch.nn.functional.max_pool2d(x, (1, 2))
 
 
 class ConvStackParams:
@@ -143,7 +168,7 @@ class ConvStack(torch.nn.Module):
         for lay, conv in zip(self.plan, self.convs):
             x = conv(x, activation="relu") if fused else self.params.nonlinearity(conv(x))
             if lay["pool"]:
-                x = torch.nn.functional.max_pool2d(x, (1, 2))
+                x = freq_max_pool(x)
         return x
 
 

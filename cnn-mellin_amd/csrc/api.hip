@@ -821,6 +821,29 @@ int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch,
   return MELLIN_OK;
 }
 
+int mellin_pool_pairs_forward_f32(const float *x, int64_t rows, int64_t f, float *y, unsigned char *which,
+                                  void *stream) {
+  const char *fn = __func__;
+  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
+  if (rows * (f / 2) == 0) return MELLIN_OK;
+  if (!x || !y || !which) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e = launch_pool_pairs_forward(x, rows, f, y, which, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+int mellin_pool_pairs_backward_f32(const float *grad_y, const unsigned char *which, int64_t rows, int64_t f,
+                                   float *grad_x, void *stream) {
+  const char *fn = __func__;
+  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
+  if (rows * f == 0) return MELLIN_OK;
+  if (!grad_x || (f / 2 && (!grad_y || !which))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e = launch_pool_pairs_backward(grad_y, which, rows, f, grad_x, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
 int mellin_set_math(int mode) {
   if (mode != MELLIN_MATH_FP32 && mode != MELLIN_MATH_BF16X3 && mode != MELLIN_MATH_BF16X3_ALWAYS)
     return fail(MELLIN_ERR_ARGUMENT, "mellin_set_math: unknown mode %d", mode);

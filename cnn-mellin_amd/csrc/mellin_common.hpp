@@ -153,6 +153,12 @@ size_t bias_grad_workspace_bytes(i64 batch, i64 channels, i64 plane);
 hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, i64 channels, i64 plane,
                             float *grad_masked, float *grad_bias, float *workspace, hipStream_t stream);
 
+// pointwise.hip: max over pairs of neighbours along the last axis of x (rows, f), and its backward
+hipError_t launch_pool_pairs_forward(const float *x, i64 rows, i64 f, float *y, unsigned char *which,
+                                     hipStream_t stream);
+hipError_t launch_pool_pairs_backward(const float *gy, const unsigned char *which, i64 rows, i64 f, float *gx,
+                                      hipStream_t stream);
+
 // half <-> float copies of n elements (16 bytes at a time when both buffers are 16-byte aligned)
 hipError_t launch_half_to_float(const void *src, float *dst, i64 n, hipStream_t stream);
 hipError_t launch_float_to_half(const float *src, void *dst, i64 n, hipStream_t stream);

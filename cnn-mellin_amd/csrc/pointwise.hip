@@ -252,6 +252,60 @@ hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, 
   return hipGetLastError();
 }
 
+// ---- max over pairs of neighbours along the last axis (frequency pooling, window 2) -----
+// y[r, j] = max(x[r, 2 j], x[r, 2 j + 1]) for x (rows, f), j < f / 2 (an odd last column is
+// dropped), as max_pool2d(x, (1, 2)) does; `which` keeps one byte per output: 1 when the
+// second of the pair was taken (strictly greater, or NaN), so that the backward pass
+// needs neither x nor 8-byte indices.
+namespace {
+
+__global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const float *__restrict__ x, i64 rows, i64 f,
+                                                                        i64 fo, float *__restrict__ y,
+                                                                        unsigned char *__restrict__ which) {
+  const i64 total = rows * fo;
+  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (i64)gridDim.x * kPwThreads) {
+    const i64 r = i / fo, j = i - r * fo;
+    const float a = x[r * f + 2 * j], b = x[r * f + 2 * j + 1];
+    const bool second = b > a || b != b;
+    y[i] = second ? b : a;
+    which[i] = second ? 1 : 0;
+  }
+}
+
+__global__ __launch_bounds__(kPwThreads) void pool_pairs_backward_kernel(const float *__restrict__ gy,
+                                                                         const unsigned char *__restrict__ which,
+                                                                         i64 rows, i64 f, i64 fo,
+                                                                         float *__restrict__ gx) {
+  const i64 total = rows * f;
+  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (i64)gridDim.x * kPwThreads) {
+    const i64 r = i / f, c = i - r * f, j = c >> 1;
+    float v = 0.f;
+    if (j < fo && (int)which[r * fo + j] == (int)(c & 1)) v = gy[r * fo + j];
+    gx[i] = v;
+  }
+}
+
+}  // namespace
+
+hipError_t launch_pool_pairs_forward(const float *x, i64 rows, i64 f, float *y, unsigned char *which,
+                                     hipStream_t stream) {
+  const i64 fo = f / 2;
+  if (rows <= 0 || fo <= 0) return hipSuccess;
+  const i64 blocks = std::min<i64>((rows * fo + kPwThreads - 1) / kPwThreads, 1 << 20);
+  hipLaunchKernelGGL(pool_pairs_forward_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x, rows, f, fo,
+                     y, which);
+  return hipGetLastError();
+}
+
+hipError_t launch_pool_pairs_backward(const float *gy, const unsigned char *which, i64 rows, i64 f, float *gx,
+                                      hipStream_t stream) {
+  if (rows <= 0 || f <= 0) return hipSuccess;
+  const i64 blocks = std::min<i64>((rows * f + kPwThreads - 1) / kPwThreads, 1 << 20);
+  hipLaunchKernelGGL(pool_pairs_backward_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy, which,
+                     rows, f, f / 2, gx);
+  return hipGetLastError();
+}
+
 // ---- half <-> float copies (the half-precision entry points compute in fp32) ------
 namespace {
 

@@ -350,6 +350,16 @@ int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch,
                          float *grad_bias, void *workspace, size_t workspace_bytes,
                          void *stream);
 
+/* Frequency pooling of the convolution stack (BASELINE config 5): the maximum over pairs of
+ * neighbours along the last axis, y[r, j] = max(x[r, 2 j], x[r, 2 j + 1]) for x (rows, f) and
+ * j < f / 2 -- what max_pool2d(x, (1, 2)) computes (the first of two equal values wins, NaN
+ * propagates) -- with one byte per output in `which` (1: the second of the pair was taken)
+ * instead of 8-byte indices; backward writes grad_x (rows, f) from grad_y (rows, f / 2). */
+int mellin_pool_pairs_forward_f32(const float *x, int64_t rows, int64_t f, float *y,
+                                  unsigned char *which, void *stream);
+int mellin_pool_pairs_backward_f32(const float *grad_y, const unsigned char *which,
+                                   int64_t rows, int64_t f, float *grad_x, void *stream);
+
 /* Name of the kernel variant the most recent operator-level call of the
  * process (on any thread: PyTorch runs backward passes on a thread of its own)
  * dispatched to (for tests and profiling): "generic", "mfma" (tiled

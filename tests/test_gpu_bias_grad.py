@@ -63,3 +63,26 @@ def test_layer_backward_uses_it():
     torch.testing.assert_close(y, y2, rtol=1e-5, atol=1e-5 * 48 ** 0.5)
     torch.testing.assert_close(gb, gb2, rtol=1e-4, atol=1e-4 * (4 * 37 * 18) ** 0.5)
     torch.testing.assert_close(gw, gw2, rtol=1e-4, atol=1e-4 * (4 * 37 * 18) ** 0.5)
+
+
+@pytest.mark.parametrize("shape", [(4, 8, 50, 38), (2, 3, 7, 41), (3, 2, 5, 2), (2, 2, 3, 1), (1, 64, 777, 38)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_frequency_pool_equals_max_pool2d(shape):
+    """The stack's frequency pooling (pairs of neighbouring bins): values and gradient bit for bit
+    what max_pool2d(x, (1, 2)) gives, ties and an odd last column included."""
+    from conv_stack import freq_max_pool
+    torch.manual_seed(shape[2])
+    x = torch.randn(*shape, device="cuda")
+    x[..., : shape[3] // 2 * 2] = torch.where(torch.rand_like(x[..., : shape[3] // 2 * 2]) < 0.2,
+                                              torch.zeros(()).to(x), x[..., : shape[3] // 2 * 2])   # ties at zero
+    a = x.clone().requires_grad_(True)
+    b = x.clone().requires_grad_(True)
+    if shape[3] < 2:
+        assert freq_max_pool(a).shape == shape[:3] + (0,)
+        return
+    ya, yb = freq_max_pool(a), torch.nn.functional.max_pool2d(b, (1, 2))
+    assert torch.equal(ya, yb)
+    g = torch.randn_like(ya)
+    ya.backward(g)
+    yb.backward(g)
+    assert torch.equal(a.grad, b.grad)
