@@ -259,12 +259,15 @@ hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, 
 // needs neither x nor 8-byte indices.
 namespace {
 
-__global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const float *__restrict__ x, i64 rows, i64 f,
-                                                                        i64 fo, float *__restrict__ y,
+// I: index type (unsigned 32-bit when rows * f fits: a 64-bit division per element costs more
+// than the memory traffic)
+template <typename I>
+__global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const float *__restrict__ x, I rows, I f,
+                                                                        I fo, float *__restrict__ y,
                                                                         unsigned char *__restrict__ which) {
-  const i64 total = rows * fo;
-  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (i64)gridDim.x * kPwThreads) {
-    const i64 r = i / fo, j = i - r * fo;
+  const I total = rows * fo;
+  for (I i = (I)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (I)gridDim.x * kPwThreads) {
+    const I r = i / fo, j = i - r * fo;
     const float a = x[r * f + 2 * j], b = x[r * f + 2 * j + 1];
     const bool second = b > a || b != b;
     y[i] = second ? b : a;
@@ -272,16 +275,25 @@ __global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const fl
   }
 }
 
+__global__ __launch_bounds__(kPwThreads) void zero_words_kernel(float *__restrict__ p, i64 n) {
+  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < n; i += (i64)gridDim.x * kPwThreads) p[i] = 0.f;
+}
+
+// one thread per pair: both words of the pair, and the odd last column with the row's last pair
+template <typename I>
 __global__ __launch_bounds__(kPwThreads) void pool_pairs_backward_kernel(const float *__restrict__ gy,
                                                                          const unsigned char *__restrict__ which,
-                                                                         i64 rows, i64 f, i64 fo,
+                                                                         I rows, I f, I fo,
                                                                          float *__restrict__ gx) {
-  const i64 total = rows * f;
-  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (i64)gridDim.x * kPwThreads) {
-    const i64 r = i / f, c = i - r * f, j = c >> 1;
-    float v = 0.f;
-    if (j < fo && (int)which[r * fo + j] == (int)(c & 1)) v = gy[r * fo + j];
-    gx[i] = v;
+  const I total = rows * fo;
+  for (I i = (I)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (I)gridDim.x * kPwThreads) {
+    const I r = i / fo, j = i - r * fo;
+    const float g = gy[i];
+    const bool second = which[i] != 0;
+    float *o = gx + r * f + 2 * j;
+    o[0] = second ? 0.f : g;
+    o[1] = second ? g : 0.f;
+    if (j == fo - 1 && (f & 1)) o[2] = 0.f;
   }
 }
 
@@ -292,17 +304,32 @@ hipError_t launch_pool_pairs_forward(const float *x, i64 rows, i64 f, float *y, 
   const i64 fo = f / 2;
   if (rows <= 0 || fo <= 0) return hipSuccess;
   const i64 blocks = std::min<i64>((rows * fo + kPwThreads - 1) / kPwThreads, 1 << 20);
-  hipLaunchKernelGGL(pool_pairs_forward_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x, rows, f, fo,
-                     y, which);
+  if (rows * f < ((i64)1 << 31))
+    hipLaunchKernelGGL(pool_pairs_forward_kernel<unsigned>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x,
+                       (unsigned)rows, (unsigned)f, (unsigned)fo, y, which);
+  else
+    hipLaunchKernelGGL(pool_pairs_forward_kernel<i64>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x, rows,
+                       f, fo, y, which);
   return hipGetLastError();
 }
 
 hipError_t launch_pool_pairs_backward(const float *gy, const unsigned char *which, i64 rows, i64 f, float *gx,
                                       hipStream_t stream) {
   if (rows <= 0 || f <= 0) return hipSuccess;
-  const i64 blocks = std::min<i64>((rows * f + kPwThreads - 1) / kPwThreads, 1 << 20);
-  hipLaunchKernelGGL(pool_pairs_backward_kernel, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy, which,
-                     rows, f, f / 2, gx);
+  const i64 fo = f / 2;
+  if (fo == 0) {                                        // one column: nothing was pooled (a kernel, not a memset
+    // node: the call may be recorded into a graph)
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)std::min<i64>((rows + kPwThreads - 1) / kPwThreads, 4096)),
+                       dim3(kPwThreads), 0, stream, gx, rows);
+    return hipGetLastError();
+  }
+  const i64 blocks = std::min<i64>((rows * fo + kPwThreads - 1) / kPwThreads, 1 << 20);
+  if (rows * f < ((i64)1 << 31))
+    hipLaunchKernelGGL(pool_pairs_backward_kernel<unsigned>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
+                       which, (unsigned)rows, (unsigned)f, (unsigned)fo, gx);
+  else
+    hipLaunchKernelGGL(pool_pairs_backward_kernel<i64>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
+                       which, rows, f, fo, gx);
   return hipGetLastError();
 }
 
