@@ -104,6 +104,7 @@ def set_variant(name=None):
 
 
 MATH_FP32, MATH_BF16X3, MATH_BF16X3_ALWAYS = 0, 1, 2
+MATH_F16 = 3          # reported by last_math() only: half-precision operands on the f16 matrix cores
 
 
 def set_math(mode):

@@ -27,6 +27,7 @@ thread_local char g_error[512] = "";
 // Process-wide, not per thread: PyTorch runs the backward pass of device tensors on its
 // autograd thread, and a variant forced from the user's thread must hold there too.
 std::atomic<const char *> g_variant{""};
+std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
 std::atomic<int> g_forced{0};    // 0 automatic, 1 generic, 2 automatic without the newer specialised kernels
@@ -602,13 +603,51 @@ int log_lift_backward(const char *fn, const T *x, const T *gy, double eps, doubl
   batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py,    \
   ux, uy
 
-// ---- half-precision entry points: half tensors, fp32 arithmetic -------------------
-// Each operand is copied to fp32 in the workspace and the fp32 kernels run there.  The
-// matrix-core tile kernel (forward, and the input gradient of layers with many input
-// channels) rounds its results to half precision as it stores them; the other kernels
-// write fp32 into the workspace and the result is copied back to half.  Regions are
-// 256-byte aligned.
+// ---- half-precision entry points: half tensors, fp32 accumulation -----------------
+// Where the tiled matrix-core kernel applies (the forward pass; the input gradient of
+// layers with many input channels) it reads the half-precision tensors as they lie,
+// multiplies on the f16 matrix cores (products of half-precision values are exact in
+// fp32, sums are kept in fp32) and stores half precision: no copies, and the workspace
+// holds at most the filter's fragments.
+// Otherwise each operand is copied to fp32 in the workspace and the fp32 kernels run
+// there; they write fp32 into the workspace and the result is copied back to half.
+// Regions are 256-byte aligned.
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+struct HalfNative {
+  TilePlan pl;
+  size_t lds, frag_bytes;
+  int mt, nt;
+};
+
+// The tiled kernel's plan for `pr` with half-precision operands and results, if it has one
+// and the variant in force allows it.
+bool plan_half_native(SepConv pr, HalfNative &hn) {
+  if (g_forced == 1 || g_widen) return false;
+  pr.in_half = 1;
+  pr.out_half = 1;
+  if (!make_tile_plan(pr, hn.pl, &hn.lds, &hn.mt, &hn.nt)) return false;
+  hn.frag_bytes = tile_fragment_bytes(hn.pl, hn.mt);
+  return true;
+}
+
+int run_half_native(const char *fn, const HalfNative &hn, const void *f, const void *g, const void *bias, void *h,
+                    void *workspace, size_t workspace_bytes, void *stream) {
+  if (hn.frag_bytes && (!workspace || workspace_bytes < hn.frag_bytes))
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, hn.frag_bytes, workspace_bytes);
+  if (hn.frag_bytes && ((uintptr_t)workspace & 15))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: the workspace must be 16-byte aligned", fn);
+  if (!f || !g || !h) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  g_variant = "mfma-f16";
+  g_last_math = MELLIN_MATH_F16;
+  return check_hip(launch_tile_gemm(hn.pl, hn.lds, hn.mt, hn.nt, (const float *)f, (const float *)g,
+                                    (const float *)bias, (float *)h, (hipStream_t)stream,
+                                    hn.frag_bytes ? (float *)workspace : nullptr), fn);
+}
+
+// Input gradients of layers with fewer input channels than this leave most of a 32-row
+// matrix tile empty in the gather form: they keep the fp32 kernels made for them.
+constexpr i64 kHalfGatherMinChannels = 16;
 
 struct HalfLayout {
   size_t in_off, w_off, b_off, out_off, inner_off, total;   // byte offsets of the fp32 copies
@@ -649,6 +688,8 @@ int mellin_corr2d_forward_act_f64(int kind_x, int activation, const double *inpu
 size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;
+  HalfNative hn;
+  if (plan_half_native(forward_problem(kind_x, CORR2D_ARGS), hn)) return hn.frag_bytes;
   return half_layout(n_in, n_w, c_out, n_out, 0).total;
 }
 int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight, const void *bias,
@@ -667,6 +708,13 @@ int mellin_corr2d_forward_act_f16(int kind_x, int activation, const void *input,
                 activation);
   CORR2D_COUNTS;
   if (n_out == 0) return MELLIN_OK;
+  {
+    SepConv pr = forward_problem(kind_x, CORR2D_ARGS);
+    pr.relu = activation == MELLIN_ACT_RELU;
+    HalfNative hn;
+    if (plan_half_native(pr, hn))
+      return run_half_native(__func__, hn, weight, input, bias, out, workspace, workspace_bytes, stream);
+  }
   const HalfLayout l = half_layout(n_in, n_w, c_out, n_out, 0);
   if (!workspace || workspace_bytes < l.total)
     return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, l.total, workspace_bytes);
@@ -690,6 +738,9 @@ int mellin_corr2d_forward_act_f16(int kind_x, int activation, const void *input,
 size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;
+  HalfNative hn;
+  if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
+    return hn.frag_bytes;
   return half_layout(n_w, n_out, 0, n_in, mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS)).total;
 }
 int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void *grad_out, MELLIN_CORR2D_DIMS,
@@ -698,6 +749,11 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
   if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
   CORR2D_COUNTS;
   if (n_in == 0) return MELLIN_OK;
+  {
+    HalfNative hn;
+    if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
+      return run_half_native(__func__, hn, weight, grad_out, nullptr, grad_input, workspace, workspace_bytes, stream);
+  }
   const size_t inner = mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS);
   const HalfLayout l = half_layout(n_w, n_out, 0, n_in, inner);
   if (!workspace || workspace_bytes < l.total)
@@ -854,7 +910,9 @@ int mellin_get_math(void) { return g_math; }
 int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
-  if (!name || !*name) { g_forced = 0; return MELLIN_OK; }
+  const bool widen = name && !strcmp(name, "widen");
+  g_widen = widen;
+  if (!name || !*name || widen) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
   if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }

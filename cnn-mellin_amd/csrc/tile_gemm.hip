@@ -57,6 +57,9 @@ namespace {
 // chunk's filter words are requested into registers before a stage's multiplies and split
 // into the other fragment buffer after them), or, when AF holds the whole filter as
 // fragments already (filter_fragments_kernel), copied from there by direct loads.
+// SPLIT 3 (one chunk) and 4 (several; AF required): F, G and bias are half-precision
+// storage and the products run on the f16 matrix cores (tile_stage.hpp); the signal is
+// staged one value per LDS word like the floats, the filter fragments have one part.
 template <int MT, int NT, bool ACC, int MB, bool HOUT, int SPLIT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
@@ -75,14 +78,18 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   extern __shared__ __align__(16) float lds[];
   constexpr int M_T = MT * 32;
   constexpr int P = kWaves * NT * 32;
+  constexpr bool F16 = SPLIT >= 3;
+  constexpr int EB = F16 ? 2 : 4;                    // bytes per element of F, G and bias
+  constexpr int PARTS = F16 ? 1 : 3;
+  static_assert(!F16 || (HOUT && !ACC), "half-precision operands come with half-precision results");
   const int g_words = pl.CC * pl.R * pl.RS;          // one signal buffer
-  const int w_words = SPLIT ? 12 * (pl.KC16 >> 3) * M_T : M_T * pl.WSS;   // one filter buffer (SPLIT: 3 parts x 16-byte fragments)
+  const int w_words = SPLIT ? 4 * PARTS * (pl.KC16 >> 3) * M_T : M_T * pl.WSS;   // one filter buffer (SPLIT: parts x 16-byte fragments)
   float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
   const int ws_word0 = SPLIT ? (pl.sbuf * g_words + 3) & ~3 : pl.sbuf * g_words;
   float *Ws0 = Gs0 + ws_word0;                       // [1 or 2][M_T][WSS], or the fragments
   // (a constant for the bf16 instances: the code that builds fragments per stage costs the
   // one-chunk kernel 24 registers and 6 % of its time when it is merely compiled in)
-  const bool single_chunk = SPLIT ? SPLIT == 1 : pl.CC >= pl.C;
+  const bool single_chunk = SPLIT ? (SPLIT & 1) : pl.CC >= pl.C;
   // SPLIT keeps four tables of KC16 words: signal offset of tap k of a whole chunk and of
   // the last (shorter) chunk, and the same two for the filter word's byte offset
   const int n_tapoff = SPLIT ? 4 * pl.KC16 : pl.KCp;
@@ -190,10 +197,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     const int sb = (st & 1) * (pl.sbuf - 1) * g_words;    // sbuf == 1: a workgroup has one stage only
     // the sources worked out for a tile's first chunk serve its other chunks; a buffer's
     // zeros (padding, rows without a tap) survive from the tile's chunk two stages back
-    issue_signal<kWaves, kMemo>(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave,
+    issue_signal<kWaves, kMemo, EB>(pl, tg, G, c0, cc, Gs0 + sb, lds_base + 4u * (unsigned)sb, mellin_x, lane, wave,
                                &memo, ch == 0, ch < 2);
     if (!SPLIT && !single_chunk) issue_filter(c0, cc, ws_word0 + (st & 1) * w_words, st < 2);
-    if (SPLIT && !single_chunk && AF) copy_fragments(ch, ws_word0 + (st & 1) * w_words);
+    if (SPLIT && !single_chunk && (AF || SPLIT == 4)) copy_fragments(ch, ws_word0 + (st & 1) * w_words);
   };
 
   // ---- SPLIT: the filter block as fragments ----------------------------------------
@@ -203,14 +210,15 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   // channels past M carry an offset beyond the filter and read as zeros.
   constexpr int kFilterItems = 2;
   constexpr unsigned kDeadOffset = 0x40000000u;
-  struct FilterWords { float x[kFilterItems][8]; };
+  typedef typename std::conditional<F16, unsigned short, float>::type FilterWord;
+  struct FilterWords { FilterWord x[kFilterItems][8]; };
   const int f_groups = SPLIT ? pl.KC16 >> 3 : 1;
   const int cc_last = pl.C - (chunks - 1) * pl.CC;
   __amdgpu_buffer_rsrc_t f_rsrc;
   if (SPLIT) f_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)F, 0, (int)pl.f_bytes, 0x00020000);
   auto load_filter = [&](int ch, int first, FilterWords &fw) {
     const int *ko = tapoff + (ch + 1 == chunks ? 3 : 2) * pl.KC16;
-    const int soff = (int)((unsigned)(ch * pl.CC) * (unsigned)pl.f_c * 4u);
+    const int soff = (int)((unsigned)(ch * pl.CC) * (unsigned)pl.f_c * (unsigned)EB);
     const FastDiv by_groups(f_groups);
 #pragma unroll
     for (int j = 0; j < kFilterItems; ++j) {
@@ -218,12 +226,16 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       if (idx < f_groups * M_T) {
         int m, g;
         by_groups.divmod(idx, m, g);
-        const unsigned row = m0 + m < pl.M ? (unsigned)(m0 + m) * (unsigned)pl.f_m * 4u : kDeadOffset;
+        const unsigned row = m0 + m < pl.M ? (unsigned)(m0 + m) * (unsigned)pl.f_m * (unsigned)EB : kDeadOffset;
         const int4 k0 = *(const int4 *)(ko + 8 * g), k1 = *(const int4 *)(ko + 8 * g + 4);
         const int off[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          fw.x[j][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(f_rsrc, (int)(row + (unsigned)off[i]), soff, 0));
+        for (int i = 0; i < 8; ++i) {
+          if constexpr (F16)
+            fw.x[j][i] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(f_rsrc, (int)(row + (unsigned)off[i]), soff, 0);
+          else
+            fw.x[j][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(f_rsrc, (int)(row + (unsigned)off[i]), soff, 0));
+        }
       }
     }
   };
@@ -235,7 +247,14 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       if (idx < f_groups * M_T) {
         int m, g;
         by_groups.divmod(idx, m, g);
-        store_frag((uintx4 *)buffer, f_groups, M_T, g, m, fw.x[j]);
+        if constexpr (F16) {
+          uintx4 v;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = (unsigned)fw.x[j][2 * i] | ((unsigned)fw.x[j][2 * i + 1] << 16);
+          ((uintx4 *)buffer)[g * M_T + m] = v;
+        } else {
+          store_frag((uintx4 *)buffer, f_groups, M_T, g, m, fw.x[j]);
+        }
       }
     }
   };
@@ -246,13 +265,14 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       int cl, t, fx, fy;
       by_nf.divmod(k, cl, t);
       by_nfy.divmod(t, fx, fy);
-      const int off = cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy;
+      // (the f16 loop adds byte offsets to byte addresses: one vector instruction per word less)
+      const int off = (cl * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy) * (F16 ? 4 : 1);
       if (SPLIT) {
         // (the taps are padded to a multiple of 16, and the last chunk may have fewer
         // channels: such a tap reads the lane's first word, always a staged one, and
         // meets a zero weight)
         const bool whole = k < pl.CC * pl.nf, last = k < cc_last * pl.nf;
-        const int fo = (cl * pl.f_c + t) * 4;
+        const int fo = (cl * pl.f_c + t) * EB;
         tapoff[k] = whole ? off : 0;
         tapoff[pl.KC16 + k] = last ? off : 0;
         tapoff[2 * pl.KC16 + k] = whole ? fo : (int)kDeadOffset;
@@ -262,13 +282,13 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       }
     }
     for (int m = tid; m < M_T; m += kThreads)
-      Bs[m] = (!ACC && bias && m0 + m < pl.M) ? bias[m0 + m] : 0.f;
+      Bs[m] = (!ACC && bias && m0 + m < pl.M) ? (F16 ? (float)((const _Float16 *)bias)[m0 + m] : bias[m0 + m]) : 0.f;
   }
   if (my_stages > 0) {
     if (SPLIT) {
       __syncthreads();                                    // the offset tables
       // (a filter that is one chunk may have more items than one round of the threads)
-      if (!single_chunk && AF) copy_fragments(0, ws_word0);
+      if (!single_chunk && (AF || SPLIT == 4)) copy_fragments(0, ws_word0);
       else for (int first = 0; first < f_groups * M_T; first += kFilterItems * kThreads) {
         FilterWords fw;
         load_filter(0, first, fw);
@@ -308,22 +328,28 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
         live = live && ox < pl.nox_eff && oy < pl.noy_eff;
       }
       if (!live) continue;
-      if (FULL && !ACC && !HOUT && buffer_stores) {
+      if (FULL && !ACC && buffer_stores) {
         // One descriptor for the block's channels of this image; a lane's offset is its
         // position plus whole groups of eight channels, the four channels inside a group
         // are scalar offsets: a store and a quarter of a 32-bit add per word, against a
         // store and a 64-bit add with pointers.
         const __amdgpu_buffer_rsrc_t h_rsrc =
             __builtin_amdgcn_make_buffer_rsrc((void *)Himg, 0, (int)(M_T * hm1), 0x00020000);
-        int voff = (half * 4) * (int)hm1 + lane_q[t] * 4;
+        int voff = (half * 4) * (int)hm1 + lane_q[t] * ES;
+        auto put = [&](float v, int soff) {
+          if constexpr (HOUT)
+            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, (_Float16)v), h_rsrc, voff, soff, 0);
+          else
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), h_rsrc, voff, soff, 0);
+        };
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
           for (int g4 = 0; g4 < 4; ++g4) {
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 0]), h_rsrc, voff, 0, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 1]), h_rsrc, voff, (int)hm1, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 2]), h_rsrc, voff, (int)hm2, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[i][t][4 * g4 + 3]), h_rsrc, voff, (int)hm3, 0);
+            put(acc[i][t][4 * g4 + 0], 0);
+            put(acc[i][t][4 * g4 + 1], (int)hm1);
+            put(acc[i][t][4 * g4 + 2], (int)hm2);
+            put(acc[i][t][4 * g4 + 3], (int)hm3);
             voff += (int)hm8;
           }
         continue;
@@ -394,7 +420,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
       // then between the matrix instructions of its SIMD's other wavefronts)
       __builtin_amdgcn_s_setprio(3);
       issue_stage(st + 1, ch + 1 == chunks ? ti + 1 : ti, ch + 1 == chunks ? 0 : ch + 1);
-      if (SPLIT && !single_chunk && !AF) load_filter(ch + 1 == chunks ? 0 : ch + 1, 0, next_filter);
+      if (SPLIT == 2 && !AF) load_filter(ch + 1 == chunks ? 0 : ch + 1, 0, next_filter);
       __builtin_amdgcn_s_setprio(0);
     }
     if (ch == 0) {
@@ -409,7 +435,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
         int ox, oy;
         by_noy.divmod(q, ox, oy);
         lane_q[t] = q;
-        lane_base[t] = (pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min;
+        lane_base[t] = ((pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min) * (F16 ? 4 : 1);
       }
     }
     if (ch == 0) {
@@ -429,7 +455,12 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     // ---- matrix-core loop over the tap pairs of this chunk
     {
       const int cc = min(pl.CC, pl.C - ch * pl.CC);
-      if (SPLIT)
+      if (F16)
+        multiply_taps_f16<MT, NT>(acc, (const uintx4 *)(Ws0 + (single_chunk ? 0 : (st & 1) * w_words)), M_T,
+                                  tapoff + (ch + 1 == chunks ? pl.KC16 : 0),
+                                  Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base,
+                                  (cc * pl.nf + 15) >> 4, l32, half);
+      else if (SPLIT)
         multiply_taps_split<MT, NT>(acc, (const uintx4 *)(Ws0 + (single_chunk ? 0 : (st & 1) * w_words)), M_T,
                                     tapoff + (ch + 1 == chunks ? pl.KC16 : 0),
                                     Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, pl.KC16,
@@ -439,7 +470,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
                             tapoff + half, Gs0 + (st & 1) * (pl.sbuf - 1) * g_words, lane_base, cc * pl.nf, half);
     }
     // the next stage's fragments: its buffer was last read two stages ago
-    if (SPLIT && !single_chunk && !AF && st + 1 < my_stages) store_filter(next_filter, 0, Ws0 + ((st + 1) & 1) * w_words);
+    if (SPLIT == 2 && !AF && st + 1 < my_stages) store_filter(next_filter, 0, Ws0 + ((st + 1) & 1) * w_words);
   }
   if (my_stages > 0) epilogue();
 #undef pl
@@ -448,8 +479,10 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
 // The whole filter as fragments, once per launch, in the order the stages of the SPLIT
 // kernel copy them: AF[m_tile][chunk][part][group][row] (16-byte words).  One thread per
 // (m_tile, chunk, group, row): eight taps of one output channel, split, three stores.
+// F16: F is half-precision storage and a fragment is the eight values themselves (one part).
+template <bool F16>
 __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int M_T, int chunks,
-                                                               const float *__restrict__ F,
+                                                               const void *__restrict__ Fv,
                                                                uintx4 *__restrict__ AF) {
   const int groups = pl.KC16 >> 3;
   const int per_block = groups * M_T;
@@ -460,13 +493,22 @@ __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int 
   const int m_tile = blk / chunks, ch = blk - m_tile * chunks;
   const int m = within / groups, g = within - m * groups;
   const int cc = min(pl.CC, pl.C - ch * pl.CC), row = m_tile * M_T + m;
-  float x[8];
+  typedef typename std::conditional<F16, unsigned short, float>::type Word;
+  const Word *F = (const Word *)Fv;
+  Word x[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int k = 8 * g + i, cl = k / pl.nf, t = k - cl * pl.nf;
-    x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + t] : 0.f;
+    x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + t] : (Word)0;
   }
-  store_frag(AF + (i64)blk * 3 * per_block, groups, M_T, g, m, x);
+  if constexpr (F16) {
+    uintx4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (unsigned)x[2 * i] | ((unsigned)x[2 * i + 1] << 16);
+    AF[(i64)blk * per_block + g * M_T + m] = v;
+  } else {
+    store_frag(AF + (i64)blk * 3 * per_block, groups, M_T, g, m, x);
+  }
 }
 
 template <int MT, int NT, bool ACC, int MB, bool HOUT = false, int SPLIT = 0>
@@ -520,6 +562,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.accumulate = pr.accumulate;
   pl.relu = pr.relu && !pr.accumulate;
   pl.out_half = pr.out_half && !pr.accumulate;
+  if (pr.in_half && !pl.out_half) return false;          // half-precision operands: half-precision results only
   pl.kind_x = X.kind; pl.sx = (int)X.s; pl.dx = (int)X.d; pl.px = (int)X.p; pl.ux = (int)X.u;
   pl.uy = (int)Y.u;
 
@@ -602,6 +645,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // signal's pitch, and a tile's rows are one contiguous run per channel.
   pl.contig = !mellin_x && !pl.segment && pl.ux == 1 && pl.uy == 1 && pl.cy + pl.by_min == 0 &&
               RSL <= pl.ngy && pl.ngy <= RSL + 8;
+  if (pr.in_half) pl.contig = 0;                          // (16-byte pieces need 4-byte elements)
   if (pl.contig) pl.RS = pl.ngy;
 
 
@@ -633,22 +677,55 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.CC = (int)cc;
   pl.KCp = ((pl.CC * pl.nf + 1) / 2) * 2;
   pl.WSS = pl.KCp + 1;                                             // odd: 32 channels -> 32 banks
-  const bool single = pl.CC >= pl.C;
+  bool single = pl.CC >= pl.C;
   *lds_bytes = 4 * (2 * (size_t)pl.CC * pl.R * pl.RS + (single ? 1 : 2) * (size_t)M_T * pl.WSS +
                     pl.KCp + M_T);
-  if (*lds_bytes > 76 * 1024) return false;
+  if (*lds_bytes > 76 * 1024 && !pr.in_half) return false;
   // the bf16 matrix cores: the filter block as fragments (6 bytes per word, taps padded to
   // a multiple of 16), built by 256 threads of two 8-tap items each
   pl.split = 0;
+  pl.f16 = 0;
   pl.KC16 = 0;
   pl.f_bytes = 0;
-  const i64 f_extent = 4 * ((pr.c_out - 1) * pr.f_m + (pr.c_in - 1) * pr.f_c + nf);
+  const i64 f_extent = (pr.in_half ? 2 : 4) * ((pr.c_out - 1) * pr.f_m + (pr.c_in - 1) * pr.f_c + nf);
+  const size_t frag_word = pr.in_half ? 2 : 6;              // fragment bytes per filter word
   auto split_lds = [&](int sbuf, i64 ccs, bool one_chunk) {
     const size_t kc16 = (size_t)((ccs * pl.nf + 15) / 16) * 16;
-    return 4 * ((((size_t)sbuf * ccs * pl.R * pl.RS) + 3) & ~(size_t)3) + (one_chunk ? 1 : 2) * 6 * kc16 * M_T +
+    return 4 * ((((size_t)sbuf * ccs * pl.R * pl.RS) + 3) & ~(size_t)3) + (one_chunk ? 1 : 2) * frag_word * kc16 * M_T +
            4 * (4 * kc16 + M_T);
   };
-  if (pr.math != MATH_FP32 && f_extent <= ((i64)1 << 30)) {
+  if (pr.in_half) {
+    // the f16 matrix cores: fragments of one part; a filter of several chunks is always
+    // read from ready-made fragments in scratch memory (tile_fragment_bytes)
+    if (f_extent > ((i64)1 << 30)) return false;
+    i64 best = 0;
+    if (split_lds(2, pl.C, true) <= 79 * 1024) {
+      best = pl.C;
+    } else {
+      const size_t budget = *nt == 2 ? 79 * 1024 : 52 * 1024;
+      double best_fill = 0;
+      for (i64 c = std::min<i64>(pl.C, 64); c >= 1; --c) {
+        const i64 kc16 = ((c * pl.nf + 15) / 16) * 16;
+        if (split_lds(2, c, false) > budget) continue;
+        if (best && c < best - 3) break;
+        const i64 n_chunks = (pl.C + c - 1) / c;
+        const i64 last = pl.C - (n_chunks - 1) * c;
+        const double fill = (double)(pl.C * pl.nf) /
+                            (double)((n_chunks - 1) * kc16 + ((last * pl.nf + 15) / 16) * 16);
+        if (!best || fill > best_fill + 1e-9) { best = c; best_fill = fill; }
+      }
+    }
+    if (best < 1 || best * pl.R >= ((i64)1 << 22) || best * ng >= lim) return false;
+    pl.split = 1;
+    pl.f16 = 1;
+    pl.CC = (int)best;
+    single = pl.CC >= pl.C;
+    pl.KC16 = (int)(((best * pl.nf + 15) / 16) * 16);
+    pl.KCp = ((pl.CC * pl.nf + 1) / 2) * 2;
+    pl.WSS = pl.KCp + 1;
+    *lds_bytes = split_lds(2, best, single);
+    pl.f_bytes = (unsigned)f_extent;
+  } else if (pr.math != MATH_FP32 && f_extent <= ((i64)1 << 30)) {
     const i64 item_cap = (2 * kThreads * 8) / M_T;         // taps per chunk the two items per thread cover
     if (single) {
       const i64 kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
@@ -708,7 +785,7 @@ size_t tile_fragment_bytes(const TilePlan &pl, int mt) {
   const int chunks = (pl.C + pl.CC - 1) / pl.CC;
   if (!pl.split || chunks < 2) return 0;
   const size_t m_tiles = (size_t)((pl.M + mt * 32 - 1) / (mt * 32));
-  return m_tiles * chunks * 3 * (size_t)(pl.KC16 >> 3) * (mt * 32) * 16;
+  return m_tiles * chunks * (pl.f16 ? 1 : 3) * (size_t)(pl.KC16 >> 3) * (mt * 32) * 16;
 }
 
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
@@ -716,11 +793,14 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
                             float *h, hipStream_t stream, float *frag_ws) {
   const int M_T = mt * 32;
   const float *af = nullptr;
+  if (pl.f16 && !pl.out_half) return hipErrorInvalidValue;
+  if (pl.f16 && tile_fragment_bytes(pl, mt) && !frag_ws) return hipErrorInvalidValue;   // no per-stage build in that kernel
   if (frag_ws && tile_fragment_bytes(pl, mt)) {
     const int chunks = (pl.C + pl.CC - 1) / pl.CC;
-    const i64 items = (i64)tile_fragment_bytes(pl, mt) / 48;
-    hipLaunchKernelGGL(filter_fragments_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pl, M_T,
-                       chunks, f, (uintx4 *)frag_ws);
+    const i64 items = (i64)tile_fragment_bytes(pl, mt) / (pl.f16 ? 16 : 48);
+    hipLaunchKernelGGL((pl.f16 ? filter_fragments_kernel<true> : filter_fragments_kernel<false>),
+                       dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pl, M_T,
+                       chunks, (const void *)f, (uintx4 *)frag_ws);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     af = frag_ws;
@@ -736,6 +816,10 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
+    if (pl.f16) {                                                                            \
+      if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, true, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      return launch_variant<MT_, NT_, false, 0, true, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+    }                                                                                        \
     if (pl.split && pl.CC >= pl.C) {                                                         \
       if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
       if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \

@@ -35,6 +35,7 @@ struct TilePlan {
   int KCp;                         // CC * nf rounded up to even
   int WSS;                         // stride of the K-major filter block (words)
   int split;                       // products on the bf16 matrix cores, operands as three bf16 parts each
+  int f16;                         // (with split) half-precision operands on the f16 matrix cores instead: one part
   int KC16;                        // split: CC * nf rounded up to a multiple of 16
   unsigned f_bytes;                // split: bytes from the filter's first word to its last one's end
 };
@@ -49,7 +50,9 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
 // scratch every workgroup splits each block again in every tile.
 size_t tile_fragment_bytes(const TilePlan &pl, int mt);
 
-// frag_ws: tile_fragment_bytes() of device memory, 16-byte aligned, or null
+// frag_ws: tile_fragment_bytes() of device memory, 16-byte aligned, or null (required by
+// a half-precision plan whose tile_fragment_bytes() is not zero).  For a plan made from a
+// problem with in_half, f, g and bias point to half-precision storage.
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
                             float *h, hipStream_t stream, float *frag_ws = nullptr);

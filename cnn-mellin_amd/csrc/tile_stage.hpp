@@ -44,14 +44,21 @@ __device__ __forceinline__ void load16_to_lds_at(const float *base, unsigned byt
 // what lets the loads of the next stage stay in flight during the matrix
 // loop; every consumer waits explicitly (wait_all_memory + barrier).  m0
 // carries the LDS base.  Destinations are passed as addresses, not pointers.
-__device__ __forceinline__ void load_to_lds_at(const float *base, unsigned byte_offset, unsigned lds_addr) {
+// EB = 2: the element in memory is 16 bits wide (any 2-byte alignment) and arrives
+// zero-extended, still one element per LDS word.
+template <int EB = 4>
+__device__ __forceinline__ void load_to_lds_at(const void *base, unsigned byte_offset, unsigned lds_addr) {
   const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   const unsigned long long b = (unsigned long long)base;
   const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
   const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
   const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-               :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
+  if (EB == 2)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2"
+                 :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(m0v), "v"(byte_offset), "s"(sbase) : "memory");
 }
 
 __device__ __forceinline__ void wait_all_memory() {
@@ -147,9 +154,24 @@ struct StageMemo {
   int word_src[MB > 0 ? MB : 1];                   // word-wise staging: lane's word of the wave's b-th block
 };
 
-// The same LDS target in every channel of a chunk: channel cl reads cl * g_c floats
-// further on and lands cl planes further on.
-__device__ __forceinline__ void load_channels(const float *base, int g_c, unsigned voff, unsigned lds_addr,
+// The same LDS target in every channel of a chunk: channel cl reads cl * g_c elements
+// (of EB bytes) further on and lands cl planes further on.
+#define MELLIN_CHANNEL_LOADS(INSTR)                                                                         \
+  for (; cl + 4 <= cc; cl += 4) {                    /* four channels per block of straight-line code */   \
+    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\t" INSTR " %0, %3\n\t"                       \
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\t" INSTR " %0, %3\n\t"                   \
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\t" INSTR " %0, %3\n\t"                   \
+                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\t" INSTR " %0, %3"                        \
+                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase), "s"(pb) : "memory", "scc");                  \
+    m0v = __builtin_amdgcn_readfirstlane(m0v + 4u * pb);                                                   \
+  }                                                                                                         \
+  for (; cl < cc; ++cl) {                                                                                   \
+    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\t" INSTR " %0, %3"                            \
+                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase) : "memory");                                   \
+    m0v = __builtin_amdgcn_readfirstlane(m0v + pb);                                                        \
+  }
+template <int EB = 4>
+__device__ __forceinline__ void load_channels(const void *base, int g_c, unsigned voff, unsigned lds_addr,
                                               unsigned plane_bytes, int cc) {
   // One instruction slot is all a staging wavefront gets between the matrix instructions of
   // its SIMD's other wavefront, so the loop is cut to what it needs: the LDS target goes to
@@ -160,26 +182,16 @@ __device__ __forceinline__ void load_channels(const float *base, int g_c, unsign
   const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
   const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
   const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
-  const unsigned step = __builtin_amdgcn_readfirstlane(4u * (unsigned)g_c);
+  const unsigned step = __builtin_amdgcn_readfirstlane((unsigned)EB * (unsigned)g_c);
   const unsigned pb = __builtin_amdgcn_readfirstlane(plane_bytes);
   unsigned v = voff - step;
   unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   cc = __builtin_amdgcn_readfirstlane(cc);           // wave-uniform: say so, or the loop's scalars end up in vector registers
   int cl = 0;
-  for (; cl + 4 <= cc; cl += 4) {                    // four channels per block of straight-line code
-    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
-                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
-                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3\n\t"
-                 "s_add_u32 m0, m0, %4\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3"
-                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase), "s"(pb) : "memory", "scc");
-    m0v = __builtin_amdgcn_readfirstlane(m0v + 4u * pb);
-  }
-  for (; cl < cc; ++cl) {
-    asm volatile("s_mov_b32 m0, %1\n\tv_add_u32 %0, %0, %2\n\tglobal_load_lds_dword %0, %3"
-                 : "+v"(v) : "s"(m0v), "s"(step), "s"(sbase) : "memory");
-    m0v = __builtin_amdgcn_readfirstlane(m0v + pb);
-  }
+  if (EB == 2) { MELLIN_CHANNEL_LOADS("global_load_lds_ushort") }
+  else { MELLIN_CHANNEL_LOADS("global_load_lds_dword") }
 }
+#undef MELLIN_CHANNEL_LOADS
 __device__ __forceinline__ void zero_channels(float *at, int plane, int cc) {
   for (int cl = 0; cl < cc; ++cl) { *at = 0.f; at += plane; }
 }
@@ -192,24 +204,26 @@ __device__ __forceinline__ void zero_channels(float *at, int plane, int cc) {
 // `memo` carries the tile's sources from the call with new_tile set to the calls
 // for the tile's other chunks.  MB < 0: no memo, and everything is written on
 // every call.
-template <int NW = kWaves, int MB = -1, class PL>
+// EB: bytes per element of G (4: float; 2: half precision, staged zero-extended, one
+// element per LDS word like the floats)
+template <int NW = kWaves, int MB = -1, int EB = 4, class PL>
 __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
-                                             const float *__restrict__ G, int c0, int cc,
+                                             const void *__restrict__ G, int c0, int cc,
                                              float *Gs, unsigned gs_addr, bool mellin_x, int lane,
                                              int wave, StageMemo<MB> *memo = nullptr, bool new_tile = true,
                                              bool fresh = true) {
-  const float *Gimg = G + (i64)tg.n * pl.g_n + (i64)c0 * pl.g_c;
+  const char *Gimg = (const char *)G + ((i64)tg.n * pl.g_n + (i64)c0 * pl.g_c) * EB;
   const int g_c = (int)pl.g_c;                         // fits: c_in * ngx * ngy < 2^31
   constexpr bool MEMO = MB > 0;
   if (MB < 0) fresh = true;
   if (!MEMO) new_tile = true;
-  if (pl.contig && tg.vx_min >= 0 && tg.vx_min + tg.R_tile <= pl.ngx) {
+  if (EB == 4 && pl.contig && tg.vx_min >= 0 && tg.vx_min + tg.R_tile <= pl.ngx) {
     // the virtual rows ARE the signal rows vx_min ... of each channel, with the
     // signal's own row pitch: one run of R_tile * ngy words per channel, moved
     // 16 bytes per lane (1 KB per instruction), the pieces dealt out to the waves
     const int count = tg.R_tile * pl.ngy, count4 = count & ~3;
     const int pieces = (count4 + 255) >> 8;
-    const float *src0 = Gimg + tg.vx_min * pl.ngy;
+    const float *src0 = (const float *)Gimg + tg.vx_min * pl.ngy;
     for (int cl = 0, pc = wave; pieces > 0; pc += NW) {    // piece pc of channel cl; pieces go round the waves
       while (pc >= pieces) { pc -= pieces; ++cl; }         // (no pieces at all: a run of under four words)
       if (cl >= cc) break;
@@ -264,7 +278,7 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
       return gx >= 0 ? gx * pl.ngy + gy : -1;
     };
     auto move = [&](int w0, int src) {
-      if (src >= 0) load_channels(Gimg, g_c, (unsigned)src * 4u, gs_addr + 4u * (unsigned)w0, plane_bytes, cc);
+      if (src >= 0) load_channels<EB>(Gimg, g_c, (unsigned)src * EB, gs_addr + 4u * (unsigned)w0, plane_bytes, cc);
       else if (fresh && src == -1) zero_channels(Gs + w0 + lane, plane, cc);
     };
     if (MEMO) {
@@ -330,14 +344,14 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         else { const int qy = vy / pl.uy; if (qy * pl.uy == vy) gy = qy; }
         if (gy >= pl.ngy) gy = -1;
       }
-      const unsigned voff = (unsigned)max(gy, 0) * 4u;
+      const unsigned voff = (unsigned)max(gy, 0) * EB;
       const bool pad_col = gy < 0;
       for (int j = 0; j < mine; ++j) {
         const int s_src = __builtin_amdgcn_readlane(src_off, j);
         const int s_dst = __builtin_amdgcn_readlane(dst_off, j) + cb;
         if (s_src >= 0) {
           // lanes whose column has a source load it; padding columns become zeros
-          if (!pad_col) load_channels(Gimg + s_src, g_c, voff, gs_addr + 4u * (unsigned)s_dst, plane_bytes, cc);
+          if (!pad_col) load_channels<EB>(Gimg + (i64)s_src * EB, g_c, voff, gs_addr + 4u * (unsigned)s_dst, plane_bytes, cc);
           if (fresh && pad_col && in_row) zero_channels(Gs + s_dst + lane, plane, cc);
         } else if (fresh && in_row) {
           zero_channels(Gs + s_dst + lane, plane, cc);         // a row without a source
@@ -493,6 +507,57 @@ __device__ __forceinline__ void multiply_taps_split(floatx16 (&acc)[MT][NT], con
     for (int i = 0; i < MT; ++i)
 #pragma unroll
       for (int t = 0; t < NT; ++t) mfma_split6(acc[i][t], o.ah[i], o.am[i], o.al[i], o.bh[t], o.bm[t], o.bl[t]);
+  };
+  Ops a, b;
+  int s = 0;
+  if (steps > 0) fetch(0, a);
+  for (; s + 1 < steps; s += 2) {
+    fetch(s + 1, b);
+    multiply(a);
+    if (s + 2 < steps) fetch(s + 2, a);
+    multiply(b);
+  }
+  if (s < steps) multiply(a);
+}
+
+// ---- half-precision operands on the f16 matrix cores ----------------------------------
+// The product of two half-precision values is exact in fp32, so v_mfma_f32_32x32x16_f16
+// (fp32 accumulation, subnormal operands kept) needs no splitting: one instruction per
+// sixteen taps.  The staged signal holds one half-precision value per LDS word, in the
+// word's low half, at the same word offsets as the fp32 kernels' (lane_base and tp are
+// BYTE offsets here); the filter block comes as fragments, the eight values
+// k = 8 g .. 8 g + 7 of row r as one 16-byte word at frag[g * rows + r].
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
+
+template <int MT, int NT>
+__device__ __forceinline__ void multiply_taps_f16(floatx16 (&acc)[MT][NT], const uintx4 *frag, int m_rows,
+                                                  const int *tp, const float *Gs, const int (&lane_base)[NT],
+                                                  int steps, int l32, int half) {
+  struct Ops { uintx4 a[MT], b[NT]; };
+  auto fetch = [&](int s, Ops &o) {
+    const int g = 2 * s + half;
+    const int4 o0 = *(const int4 *)(tp + 8 * g), o1 = *(const int4 *)(tp + 8 * g + 4);
+    const int off[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ushortx2 pair;
+        pair.x = *(const unsigned short *)((const char *)Gs + (lane_base[t] + off[2 * i]));
+        pair.y = *(const unsigned short *)((const char *)Gs + (lane_base[t] + off[2 * i + 1]));
+        o.b[t][i] = __builtin_bit_cast(unsigned, pair);
+      }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) o.a[i] = frag[g * m_rows + i * 32 + l32];
+  };
+  auto multiply = [&](const Ops &o) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, o.a[i]),
+                                                           __builtin_bit_cast(halfx8, o.b[t]), acc[i][t], 0, 0, 0);
   };
   Ops a, b;
   int s = 0;

@@ -385,6 +385,7 @@ const char *mellin_last_variant(void);
 #define MELLIN_MATH_FP32 0
 #define MELLIN_MATH_BF16X3 1
 #define MELLIN_MATH_BF16X3_ALWAYS 2
+#define MELLIN_MATH_F16 3            /* reported by mellin_last_math only: half-precision operands on the f16 matrix cores */
 int mellin_set_math(int mode);
 int mellin_get_math(void);
 /* The mode the matrix kernels of the most recent operator-level call actually ran in

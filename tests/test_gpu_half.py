@@ -1,7 +1,9 @@
 """Half precision and autocast (the reference's Autocast registration,
 ext/torch.cpp:405-447, and its tests, tests/test_mconv.py:814-891).
 
-Through the C ABI: half operands, fp32 arithmetic, one rounding of the result.  The
+Through the C ABI: half operands, exact products, fp32 accumulation, one rounding of the
+result -- on the f16 matrix cores straight from the half tensors where the tiled kernel
+applies ("mfma-f16"), else through fp32 copies of the operands and the fp32 kernels.  The
 expected values are the float64 checker on the SAME half-rounded operands, so the only
 error left is the final rounding to half (relative 2^-11) plus the fp32 accumulation
 (rtol 1e-5, atol 1e-5 * sqrt(fan_in)): asserted as rtol 1e-3, atol 1e-3 * sqrt(fan_in) * 1e-2
@@ -35,8 +37,16 @@ def _close(got, exp, fan_in, what):
     assert not bad.any(), "%s: %d of %d off, worst %g" % (what, bad.sum(), bad.size, np.abs(got - exp).max())
 
 
+@pytest.fixture(params=["auto", "widen"])
+def half_path(request):
+    """the kernels that read half tensors themselves where they apply, and the copies to fp32 everywhere"""
+    hip.set_variant(request.param)
+    yield request.param
+    hip.set_variant(None)
+
+
 @pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
-def test_half_passes_match_checker_on_the_same_operands(case):
+def test_half_passes_match_checker_on_the_same_operands(case, half_path):
     kind, n, c_in, c_out, nf, ng, s, d, p, u, r = case
     kind_x = hip.AX_MCORR if kind == "mcorr" else hip.AX_LCORR
     fwd = oracle.mcorrlcorr if kind == "mcorr" else oracle.lcorrlcorr
@@ -53,6 +63,8 @@ def test_half_passes_match_checker_on_the_same_operands(case):
     xg, wg, bg = to_gpu(x), to_gpu(w), to_gpu(b)
     out = torch.full((n, c_out) + nh, float("nan"), dtype=torch.float16, device="cuda")
     hip.corr2d_forward(kind_x, xg, wg, bg, out, dims)
+    assert (hip.last_variant() == "mfma-f16") == (half_path == "auto")
+    assert (hip.last_math() == hip.MATH_F16) == (half_path == "auto")
     _close(out, exp, c_in * nf[0] * nf[1], "forward %s" % (case,))
     go = rng.standard_normal(exp.shape).astype(np.float16)
     egi, egw, _ = bwd(x64, w64, go.astype(np.float64), s, d, p, u)
@@ -69,6 +81,16 @@ def test_workspace_is_required_and_sized():
     x = torch.randn(2, 3, 20, 9, device="cuda").half()
     w = torch.randn(8, 3, 4, 2, device="cuda").half()
     out = torch.empty(2, 8, 4, 8, device="cuda", dtype=torch.float16)
+    # the kernel that reads half tensors needs nothing for a filter this small
+    assert hip.lib.mellin_corr2d_forward_f16_workspace(hip.AX_MCORR, *dims) == 0
+    hip.set_variant("widen")
+    try:
+        _workspace_checks(dims, x, w, out)
+    finally:
+        hip.set_variant(None)
+
+
+def _workspace_checks(dims, x, w, out):
     need = hip.lib.mellin_corr2d_forward_f16_workspace(hip.AX_MCORR, *dims)
     assert need >= 4 * (x.numel() + w.numel() + out.numel())
     small = torch.empty(need - 1, dtype=torch.uint8, device="cuda")
@@ -150,9 +172,13 @@ def test_autocast_column_ops():
     ("lcorr", 3, 3, 40, (8, 4), (70, 41)), ("mcorr", 2, 3, 64, (8, 4), (64, 41)),
     ("lcorr", 2, 48, 70, (3, 3), (30, 21)), ("mcorr", 2, 40, 33, (4, 4), (40, 5)),
 ], ids=["lcorr-few", "mcorr-few", "lcorr-many", "mcorr-many"])
-def test_half_results_are_the_fp32_results_rounded_once(shape):
-    """The half entry points compute in fp32 on the widened operands: whichever kernel
-    stores the result, it must equal the fp32 result rounded to nearest even, bit for bit."""
+def test_half_results_are_the_fp32_results_rounded_once(shape, half_path):
+    """Through the fp32 copies the half entry points compute as the fp32 ones do on the
+    widened operands: whichever kernel stores the result, it must equal the fp32 result
+    rounded to nearest even, bit for bit.  The f16 matrix instructions sum the same exact
+    products in another order: their fp32 sums differ from the fp32 kernels' in the last
+    bits, which moves a result to the neighbouring half value only where the sum lies
+    that close to a rounding boundary -- in under 1 % of the results."""
     kind, n, c_in, c_out, nf, ng = shape
     kind_x = hip.AX_MCORR if kind == "mcorr" else hip.AX_LCORR
     op = mconv.mcorrlcorr if kind == "mcorr" else mconv.lcorrlcorr
@@ -160,9 +186,18 @@ def test_half_results_are_the_fp32_results_rounded_once(shape):
     x = torch.randn((n, c_in) + ng, generator=gen).half().cuda()
     w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_in * nf[0] * nf[1]) ** -0.5).half().cuda()
     b = torch.randn(c_out, generator=gen).half().cuda()
+    def same(got, ref32, fan_in):
+        exp = ref32.half()
+        if half_path == "widen":
+            return torch.equal(got, exp)
+        # half the spacing of half values at the result, plus what fp32 accumulation may differ by
+        half_step = exp.float().abs().clamp_min(2.0 ** -14) * 2.0 ** -11
+        close = (got.float() - ref32).abs() <= 1.001 * half_step + 1e-5 * fan_in ** 0.5
+        return bool(close.all()) and float((got != exp).float().mean()) < 0.01
+
     ref = op(x.float(), w.float(), b.float())
     out = op(x, w, b)
-    assert out.dtype == torch.float16 and torch.equal(out, ref.half())
+    assert out.dtype == torch.float16 and same(out, ref, c_in * nf[0] * nf[1])
     nh = tuple(ref.shape[2:])
     dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), (0, 0), (1, 1))
     go = torch.randn(ref.shape, generator=gen).half().cuda()
@@ -170,7 +205,7 @@ def test_half_results_are_the_fp32_results_rounded_once(shape):
     hip.corr2d_backward_input(kind_x, w.float(), go.float(), gi32, dims)
     gi16 = torch.empty_like(x)
     hip.corr2d_backward_input(kind_x, w, go, gi16, dims)
-    assert torch.equal(gi16, gi32.half())
+    assert same(gi16, gi32, c_out * nf[0] * nf[1])
 
 
 def test_half_views_at_odd_offsets():
@@ -204,7 +239,60 @@ def test_half_views_at_odd_offsets():
         hip.corr2d_backward_weight(hip.AX_LCORR, xg, gog, gw, dims)
         return out.clone(), gi.clone(), gw.clone()
 
-    aligned = run(0)
-    for off in (1, 3):
-        for a, c in zip(aligned, run(off)):
-            assert torch.equal(a, c)
+    for variant in ("auto", "widen"):
+        hip.set_variant(variant)
+        try:
+            aligned = run(0)
+            for off in (1, 3):
+                for a, c in zip(aligned, run(off)):
+                    assert torch.equal(a, c)
+        finally:
+            hip.set_variant(None)
+
+
+def test_wide_layers_read_their_filter_from_fragments_in_the_workspace():
+    """Layers whose channels are staged in several chunks: the filter's fragments are made once
+    per call in the workspace (the only scratch memory the call needs), for the forward pass
+    and, with many input channels, for the input gradient, Mellin and linear."""
+    for kind_x, op in ((hip.AX_LCORR, mconv.lcorrlcorr), (hip.AX_MCORR, mconv.mcorrlcorr)):
+        n, c_in, c_out, nf, ng, s, d, p, u = 3, 150, 130, (3, 3), (40, 23), (1, 1), (2, 1), (2, 1), (1, 1)
+        gen = torch.Generator().manual_seed(5)
+        x = torch.randn((n, c_in) + ng, generator=gen).half().cuda()
+        w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_in * 9) ** -0.5).half().cuda()
+        b = torch.randn(c_out, generator=gen).half().cuda()
+        ref = op(x.float(), w.float(), b.float(), s, d, p, u)
+        nh = tuple(ref.shape[2:])
+        dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, u)
+        need = hip.lib.mellin_corr2d_forward_f16_workspace(kind_x, *dims)
+        assert 0 < need <= 2 * 2 * w.numel() * 2          # the filter once, padded to 16 taps per chunk and whole tiles
+        out = op(x, w, b, s, d, p, u)
+        assert hip.last_variant() == "mfma-f16"
+        tol = 2.0 ** -10 * ref.abs().clamp_min(2.0 ** -14) + 1e-5 * (c_in * 9) ** 0.5
+        assert bool(((out.float() - ref).abs() <= tol).all())
+        go = torch.randn(ref.shape, generator=gen).half().cuda()
+        gi32 = torch.empty_like(x, dtype=torch.float32)
+        hip.corr2d_backward_input(kind_x, w.float(), go.float(), gi32, dims)
+        assert 0 < hip.lib.mellin_corr2d_backward_input_f16_workspace(kind_x, *dims) <= 2 * 2 * w.numel() * 2
+        gi = torch.empty_like(x)
+        hip.corr2d_backward_input(kind_x, w, go, gi, dims)
+        assert hip.last_variant() == "mfma-f16"
+        tol = 2.0 ** -10 * gi32.abs().clamp_min(2.0 ** -14) + 1e-5 * (c_out * 9) ** 0.5
+        assert bool(((gi.float() - gi32).abs() <= tol).all())
+        # too little scratch memory is an error, not a slower path
+        small = torch.empty(need - 16, dtype=torch.uint8, device="cuda")
+        rc = hip.lib.mellin_corr2d_forward_f16(kind_x, x.data_ptr(), w.data_ptr(), b.data_ptr(), *dims,
+                                               out.data_ptr(), small.data_ptr(), need - 16, None)
+        assert rc == 3 and "workspace" in hip.last_error()
+
+
+def test_subnormal_half_operands_are_not_flushed():
+    """Products of subnormal half values with large ones are ordinary numbers; the f16 matrix
+    instructions must take such operands as they are."""
+    n, c_in, c_out, nf, ng = 1, 2, 32, (2, 2), (9, 40)
+    x = torch.full((n, c_in) + ng, 2.0 ** -20, dtype=torch.float16, device="cuda")      # subnormal: below 2^-14
+    x[0, 1] = 3 * 2.0 ** -24
+    w = torch.full((c_out, c_in) + nf, 1024.0, dtype=torch.float16, device="cuda")
+    out = mconv.lcorrlcorr(x, w, None)
+    assert hip.last_variant() == "mfma-f16"
+    exp = 4 * 1024.0 * (2.0 ** -20 + 3 * 2.0 ** -24)
+    assert torch.equal(out, torch.full_like(out, exp))
