@@ -267,7 +267,7 @@ struct TwoPassInput {
 
 bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                          i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px,
-                         i64 py, i64 ux, i64 uy, TwoPassInput &tp) {
+                         i64 py, i64 ux, i64 uy, TwoPassInput &tp, bool half = false) {
   (void)sx;
   const i64 m2 = c_in * nfx;
   // worth it when c_in alone would leave most of a 32-row tile empty and the
@@ -291,6 +291,7 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   pr.h_n = m2 * nhx * ngy; pr.h_m = nhx * ngy;
   pr.accumulate = 0;
   pr.math = g_math;
+  pr.in_half = half;                                   // weight and grad_out as half-precision tensors, Y in fp32
   if (!make_tile_plan(pr, tp.plan, &tp.lds, &tp.mt, &tp.nt)) return false;
   const int conv_x = kind_x == AX_MCORR ? AX_MCONV : AX_LCONV;
   tp.fold = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
@@ -645,6 +646,23 @@ int run_half_native(const char *fn, const HalfNative &hn, const void *f, const v
                                     hn.frag_bytes ? (float *)workspace : nullptr), fn);
 }
 
+// The weight gradient on the f16 matrix cores, if the variant in force allows it and the
+// kernel applies (n_in, n_out: elements of input and grad_out; nothing to sum: no).
+bool plan_half_weight(const SepConv &fwd, i64 n_in, i64 n_out, WgradHalfPlan &hp) {
+  if (g_forced == 1 || g_widen || n_in == 0 || n_out == 0) return false;
+  return make_wgrad_half_plan(fwd, hp) && hp.ws_bytes <= kMaxWorkspaceBytes;
+}
+
+// The two-pass input gradient (layers with few input channels) on half-precision tensors,
+// if the variant in force allows it and the form applies.
+bool plan_half_two_pass(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx,
+                        i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, TwoPassInput &tp) {
+  if (g_forced == 1 || g_widen || c_out * nfx * nfy * nhx * nhy == 0) return false;
+  return plan_two_pass_input(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py, ux, uy,
+                             tp, true) &&
+         tp.ws_bytes + (size_t)(batch * c_in * ngx * ngy) * 4 <= kMaxWorkspaceBytes;
+}
+
 // Input gradients of layers with fewer input channels than this leave most of a 32-row
 // matrix tile empty in the gather form: they keep the fp32 kernels made for them.
 constexpr i64 kHalfGatherMinChannels = 16;
@@ -741,6 +759,8 @@ size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS
   HalfNative hn;
   if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
     return hn.frag_bytes;
+  TwoPassInput tp;
+  if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) return align256(tp.ws_bytes) + (size_t)n_in * 4;
   return half_layout(n_w, n_out, 0, n_in, mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS)).total;
 }
 int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void *grad_out, MELLIN_CORR2D_DIMS,
@@ -753,6 +773,24 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
     HalfNative hn;
     if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
       return run_half_native(__func__, hn, weight, grad_out, nullptr, grad_input, workspace, workspace_bytes, stream);
+    TwoPassInput tp;
+    if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) {
+      // the two-pass form on the half-precision tensors: first-pass rows and the folded
+      // result in fp32 in the workspace, one rounding on the way out
+      const size_t gi_off = align256(tp.ws_bytes), need = gi_off + (size_t)n_in * 4;
+      if (!workspace || workspace_bytes < need)
+        return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, need, workspace_bytes);
+      if (!grad_input || !weight || !grad_out) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+      char *ws = (char *)workspace;
+      hipStream_t st = (hipStream_t)stream;
+      g_variant = "mfma-f16+fold";
+      g_last_math = MELLIN_MATH_F16;
+      hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight, (const float *)grad_out,
+                                      nullptr, (float *)ws, st, tp.frag_bytes ? (float *)(ws + tp.frag_off) : nullptr);
+      if (e == hipSuccess) e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)ws, (float *)(ws + gi_off), st);
+      if (e == hipSuccess) e = launch_float_to_half((const float *)(ws + gi_off), grad_input, n_in, st);
+      return check_hip(e, __func__);
+    }
   }
   const size_t inner = mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS);
   const HalfLayout l = half_layout(n_w, n_out, 0, n_in, inner);
@@ -777,6 +815,8 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
 size_t mellin_corr2d_backward_weight_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS) {
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;
+  WgradHalfPlan hp;
+  if (plan_half_weight(forward_problem(kind_x, CORR2D_ARGS), n_in, n_out, hp)) return hp.ws_bytes;
   return half_layout(n_in, n_out, 0, n_w, mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS)).total;
 }
 int mellin_corr2d_backward_weight_f16(int kind_x, const void *input, const void *grad_out, MELLIN_CORR2D_DIMS,
@@ -785,6 +825,19 @@ int mellin_corr2d_backward_weight_f16(int kind_x, const void *input, const void 
   if ((rc = check_corr2d(__func__, kind_x, CORR2D_ARGS))) return rc;
   CORR2D_COUNTS;
   if (n_w == 0) return MELLIN_OK;
+  {
+    WgradHalfPlan hp;
+    if (plan_half_weight(forward_problem(kind_x, CORR2D_ARGS), n_in, n_out, hp)) {
+      if (!workspace || workspace_bytes < hp.ws_bytes)
+        return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, hp.ws_bytes,
+                    workspace_bytes);
+      if (!grad_weight || !input || !grad_out) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+      g_variant = "mfma-f16";
+      g_last_math = MELLIN_MATH_F16;
+      return check_hip(launch_wgrad_half(hp, grad_out, input, grad_weight, (float *)workspace, (hipStream_t)stream),
+                       __func__);
+    }
+  }
   const size_t inner = mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS);
   const HalfLayout l = half_layout(n_in, n_out, 0, n_w, inner);
   if (!workspace || workspace_bytes < l.total)

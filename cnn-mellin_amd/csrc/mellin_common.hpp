@@ -33,7 +33,7 @@ struct SepConv {
   int accumulate;                // 1: h += result (h pre-initialised); 0: h = bias + result
   int relu = 0;                  // with accumulate == 0: h = max(0, bias + result)
   int out_half = 0;              // with accumulate == 0: h is half-precision storage (matrix-core kernel only)
-  int in_half = 0;               // f, g and bias are half-precision storage (matrix-core kernel only; needs out_half)
+  int in_half = 0;               // f, g and bias are half-precision storage (matrix-core kernel only; accumulate == 0)
   int math = 0;                  // MATH_FP32: fp32 matrix instructions; MATH_BF16X3: bf16 ones on three-part operands
 };
 

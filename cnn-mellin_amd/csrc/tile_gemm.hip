@@ -60,6 +60,7 @@ namespace {
 // SPLIT 3 (one chunk) and 4 (several; AF required): F, G and bias are half-precision
 // storage and the products run on the f16 matrix cores (tile_stage.hpp); the signal is
 // staged one value per LDS word like the floats, the filter fragments have one part.
+// H is half-precision (HOUT) or fp32 storage.
 template <int MT, int NT, bool ACC, int MB, bool HOUT, int SPLIT>
 __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
     TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   constexpr bool F16 = SPLIT >= 3;
   constexpr int EB = F16 ? 2 : 4;                    // bytes per element of F, G and bias
   constexpr int PARTS = F16 ? 1 : 3;
-  static_assert(!F16 || (HOUT && !ACC), "half-precision operands come with half-precision results");
+  static_assert(!F16 || !ACC, "half-precision operands: results are written, not added");
   const int g_words = pl.CC * pl.R * pl.RS;          // one signal buffer
   const int w_words = SPLIT ? 4 * PARTS * (pl.KC16 >> 3) * M_T : M_T * pl.WSS;   // one filter buffer (SPLIT: parts x 16-byte fragments)
   float *Gs0 = lds;                                  // [sbuf][CC][R][RS]
@@ -562,7 +563,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.accumulate = pr.accumulate;
   pl.relu = pr.relu && !pr.accumulate;
   pl.out_half = pr.out_half && !pr.accumulate;
-  if (pr.in_half && !pl.out_half) return false;          // half-precision operands: half-precision results only
+  if (pr.in_half && pr.accumulate) return false;         // half-precision operands: results are written, not added
   pl.kind_x = X.kind; pl.sx = (int)X.s; pl.dx = (int)X.d; pl.px = (int)X.p; pl.ux = (int)X.u;
   pl.uy = (int)Y.u;
 
@@ -793,7 +794,7 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
                             float *h, hipStream_t stream, float *frag_ws) {
   const int M_T = mt * 32;
   const float *af = nullptr;
-  if (pl.f16 && !pl.out_half) return hipErrorInvalidValue;
+  if (pl.f16 && pl.accumulate) return hipErrorInvalidValue;
   if (pl.f16 && tile_fragment_bytes(pl, mt) && !frag_ws) return hipErrorInvalidValue;   // no per-stage build in that kernel
   if (frag_ws && tile_fragment_bytes(pl, mt)) {
     const int chunks = (pl.C + pl.CC - 1) / pl.CC;
@@ -816,9 +817,13 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
-    if (pl.f16) {                                                                            \
+    if (pl.f16 && pl.out_half) {                                                             \
       if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, true, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
       return launch_variant<MT_, NT_, false, 0, true, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+    }                                                                                        \
+    if (pl.f16) {                                                                            \
+      if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, false, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      return launch_variant<MT_, NT_, false, 0, false, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
     }                                                                                        \
     if (pl.split && pl.CC >= pl.C) {                                                         \
       if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \

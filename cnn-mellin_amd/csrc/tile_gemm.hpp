@@ -52,7 +52,8 @@ size_t tile_fragment_bytes(const TilePlan &pl, int mt);
 
 // frag_ws: tile_fragment_bytes() of device memory, 16-byte aligned, or null (required by
 // a half-precision plan whose tile_fragment_bytes() is not zero).  For a plan made from a
-// problem with in_half, f, g and bias point to half-precision storage.
+// problem with in_half, f, g and bias point to half-precision storage; h is half-precision
+// storage when the plan has out_half, else float.
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
                             float *h, hipStream_t stream, float *frag_ws = nullptr);
@@ -83,5 +84,30 @@ bool make_wgrad_plan(const SepConv &fwd, WgradPlan &wp, bool allow_rows = true, 
 
 hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float *input,
                         float *grad_weight, float *workspace, hipStream_t stream);
+
+// wgrad_gemm.hip: W[m, j] = the sum of `partials` blocks of (M_pad x J_pad) floats, in index order;
+// W is float storage, or half-precision storage (rounded once) when half_out
+hipError_t launch_wgrad_reduce(const float *partials_ws, void *W, bool half_out, int partials, int M, int J,
+                               int M_pad, int J_pad, hipStream_t stream);
+
+// Weight gradient of a half-precision layer on the f16 matrix cores (wgrad_f16.hip).
+struct WgradHalfPlan {
+  TilePlan t;                      // staging geometry of the forward problem
+  i64 a_n, a_m;                    // grad_out strides: image, channel (positions are dense)
+  int J, jt;                       // c_in * nfx * nfy; 32-column tiles per wavefront
+  int mbw;                         // wavefronts side by side along the channels (64 each); the rest share a unit's steps
+  int m_groups, j_groups, M_pad, J_pad;
+  int CCj;                         // input channels a column block can touch
+  int RB, UP;                      // output rows per unit; their positions rounded up to 16
+  int S;                           // persistent workgroups per output block
+  size_t lds_bytes, ws_bytes;
+};
+
+// false: the kernel does not apply (outputs wider than 128 columns, sizes beyond its limits)
+bool make_wgrad_half_plan(const SepConv &fwd, WgradHalfPlan &wp);
+
+// grad_out, input and grad_weight are half-precision storage; workspace: wp.ws_bytes
+hipError_t launch_wgrad_half(const WgradHalfPlan &wp, const void *grad_out, const void *input,
+                             void *grad_weight, float *workspace, hipStream_t stream);
 
 }  // namespace mellin

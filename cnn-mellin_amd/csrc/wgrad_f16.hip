@@ -1,0 +1,319 @@
+// Weight gradient of half-precision layers on the f16 matrix cores.
+//
+//   W[m, (c, fx, fy)] = sum_{n, ox, oy} A[n, m, ox, oy] *
+//                       G[n, c, tap_x(ox, fx), tap_y(oy, fy)]
+//
+// A = grad_out and G = the layer's input are half-precision tensors, read as they lie.
+// Products of half values are exact in fp32 and v_mfma_f32_32x32x16_f16 sums them in fp32,
+// so the arithmetic is that of the fp32 kernels on the widened operands, in another order.
+//
+// The product is (M x positions) * (positions x J), J = c_in * nfx * nfy, and the k index of
+// a matrix instruction runs over sixteen CONSECUTIVE output positions of one image (rows
+// flattened), eight per half-wave:
+//   * grad_out: the eight positions of a lane's channel are sixteen consecutive bytes of
+//     global memory (any 2-byte alignment) and are the instruction's operand as they are:
+//     one 16-byte load per lane, a few steps ahead, no LDS;
+//   * input: the rows a unit of work touches are staged as in the forward kernel (direct
+//     global->LDS loads into affine virtual rows, one half value per LDS word), and the
+//     operand of lane (column j) for position q is the 16-bit word at
+//     col_offset[j] + pos_offset[q]; pos_offset is a table in LDS, the same for every unit.
+// A unit is RB output rows of one image.  A workgroup owns 64 * mbw output channels and
+// JT * 32 columns for its whole life and walks a contiguous range of units (image running
+// fastest, so that consecutive units stage the same rows of successive images); its four
+// wavefronts are mbw side by side along the channels times 4 / mbw shares of a unit's
+// steps.  Every wavefront writes its accumulators as one partial block; wgrad_reduce adds
+// the partial blocks in index order (no floating-point atomics: bit-reproducible).
+#include <algorithm>
+
+#include "mellin_common.hpp"
+#include "tile_gemm.hpp"
+#include "tile_stage.hpp"
+
+namespace mellin {
+
+namespace {
+
+constexpr int kF16Memo = 8;                        // 64-word blocks per wave whose staging sources are kept
+constexpr int kAhead = 4;                          // steps whose grad_out operands are in flight
+
+struct __attribute__((packed, aligned(2))) Half8 { uintx4 v; };
+
+template <int JT>
+__global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
+    WgradHalfPlan wp, const _Float16 *__restrict__ A, const _Float16 *__restrict__ G,
+    float *__restrict__ ws) {
+  extern __shared__ __align__(16) float lds[];
+  const TilePlan &pl = wp.t;
+  constexpr int MT = 2;
+  const int x_words = (wp.CCj * pl.R * pl.RS + 3) & ~3;
+  float *Xs0 = lds;                                  // [2][CCj][R][RS], one half value per word
+  int *pos_off = (int *)(Xs0 + 2 * x_words);         // [UP] byte offset of a position's (fx, fy) = (0, 0) word
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, l32 = lane & 31;
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+  const int mb = wave % wp.mbw, ps = wave / wp.mbw, PS = kWaves / wp.mbw;
+
+  const int mg = blockIdx.y / wp.j_groups, jg = blockIdx.y - mg * wp.j_groups;
+  const int M_T = 64 * wp.mbw, J_T = JT * 32;
+  const int m0 = mg * M_T + mb * 64, j0 = jg * J_T;
+  const int c_lo = j0 / pl.nf;
+  const int j_last = min(wp.J, j0 + J_T) - 1;
+  const int ccj = j_last / pl.nf - c_lo + 1;
+
+  int col_off[JT];                                   // bytes
+  {
+    const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
+#pragma unroll
+    for (int t = 0; t < JT; ++t) {
+      const int j = min(j0 + t * 32 + l32, wp.J - 1);   // columns past J are computed but never read back
+      int c, tt, fx, fy;
+      by_nf.divmod(j, c, tt);
+      by_nfy.divmod(tt, fx, fy);
+      col_off[t] = ((c - c_lo) * pl.R * pl.RS + pl.Bx * fx * pl.RS + pl.by * fy) * 4;
+    }
+  }
+  {
+    const FastDiv by_noy(pl.noy);
+    for (int p = tid; p < wp.UP; p += kThreads) {
+      int oxl, oy;
+      by_noy.divmod(p, oxl, oy);
+      pos_off[p] = oxl < wp.RB ? ((pl.Ax * oxl + pl.Cx0) * pl.RS + pl.ay * oy - pl.by_min) * 4 : 0;
+    }
+  }
+
+  // units: image fastest; this workgroup's contiguous range
+  const int units_per_image = (pl.nox_eff + wp.RB - 1) / wp.RB;
+  const int total_units = pl.batch * units_per_image;
+  const int share = total_units / (int)gridDim.x, extra = total_units - share * (int)gridDim.x;
+  const int my_units = share + ((int)blockIdx.x < extra ? 1 : 0);
+  const int first_unit = (int)blockIdx.x * share + min((int)blockIdx.x, extra);
+  const unsigned lds_base = lds_address(lds);
+
+  auto unit_geometry = [&](int unit) {
+    TileGeom g;
+    const int u = unit / pl.batch;
+    g.n = unit - u * pl.batch;
+    g.ox_lo = u * wp.RB;
+    const int rows = min(wp.RB, pl.nox_eff - g.ox_lo);
+    g.oy_lo = 0;
+    g.q0 = g.ox_lo * pl.noy;
+    g.count = rows * pl.noy;
+    g.R_tile = mellin_x ? rows * pl.nfx : pl.ax * (rows - 1) + pl.bx_span + 1;
+    g.vx_min = pl.ax * g.ox_lo + pl.cx + pl.bx_min;
+    g.vy_min = pl.cy + pl.by_min;
+    g.RSL = pl.ay * (pl.noy - 1) + pl.by_span + 1;
+    return g;
+  };
+  StageMemo<kF16Memo> memo = {};
+  auto issue_stage = [&](int ui) {
+    const TileGeom tg = unit_geometry(first_unit + ui);
+    const int b = ui & 1;
+    // units since the rows last changed (or since this workgroup started): the memo is
+    // renewed at 0, and a buffer's zeros are written the first two times it holds these rows
+    const int run = min(tg.n, ui);
+    unsigned zero;                                     // a zero the compiler cannot see through (see tile_gemm.hip)
+    asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
+    issue_signal<kWaves, kF16Memo, 2>(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words),
+                                      mellin_x, lane, wave + (int)zero, &memo, run == 0, run < 2);
+  };
+
+  floatx16 acc[MT][JT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
+
+  // this lane's two channels (one past M reads the last channel's values instead: its rows
+  // of the partial block are never read back)
+  int m_off[MT];                                       // elements: M * Q < 2^30
+#pragma unroll
+  for (int i = 0; i < MT; ++i) m_off[i] = min(m0 + i * 32 + l32, pl.M - 1) * (int)wp.a_m + 8 * half;
+
+  // the operands of one step: words of eight half values
+  auto load_a = [&](const _Float16 *An, int s, uintx4 (&a)[MT]) {      // whole steps only
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a[i] = ((const Half8 *)(An + m_off[i] + 16 * s))->v;
+  };
+  auto fetch_b = [&](const float *Xs, int s, uintx4 (&b)[JT]) {
+    const int4 o0 = *(const int4 *)(pos_off + 16 * s + 8 * half), o1 = *(const int4 *)(pos_off + 16 * s + 8 * half + 4);
+    const int off[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ushortx2 pair;
+        pair.x = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i]));
+        pair.y = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i + 1]));
+        b[t][i] = __builtin_bit_cast(unsigned, pair);
+      }
+  };
+  auto multiply = [&](const uintx4 (&a)[MT], const uintx4 (&b)[JT]) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int t = 0; t < JT; ++t)
+        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a[i]),
+                                                           __builtin_bit_cast(halfx8, b[t]), acc[i][t], 0, 0, 0);
+  };
+
+  __syncthreads();                                     // pos_off
+  if (my_units > 0) issue_stage(0);
+  for (int ui = 0; ui < my_units; ++ui) {
+    const TileGeom tg = unit_geometry(first_unit + ui);
+    const _Float16 *An = A + (i64)tg.n * wp.a_n + tg.q0;
+    const int whole = tg.count >> 4;                   // steps of sixteen positions that exist
+    // this wavefront's steps ps, ps + PS, ...: the first few operands are requested before
+    // the wait for the staged rows
+    uintx4 ring[kAhead][MT];
+#pragma unroll
+    for (int d = 0; d < kAhead; ++d)
+      if (ps + d * PS < whole) load_a(An, ps + d * PS, ring[d]);
+    wait_all_memory();
+    __syncthreads();
+    if (ui + 1 < my_units) {
+      __builtin_amdgcn_s_setprio(3);
+      issue_stage(ui + 1);
+      __builtin_amdgcn_s_setprio(0);
+    }
+    const float *Xs = Xs0 + (ui & 1) * x_words;
+    for (int s0 = ps; s0 < whole; s0 += kAhead * PS) {
+#pragma unroll
+      for (int d = 0; d < kAhead; ++d) {
+        const int s = s0 + d * PS;
+        if (s < whole) {
+          uintx4 b[JT];
+          fetch_b(Xs, s, b);
+          multiply(ring[d], b);
+          if (s + kAhead * PS < whole) load_a(An, s + kAhead * PS, ring[d]);
+        }
+      }
+    }
+    // the last, partial step (by the wavefront whose turn it is): positions past the unit's
+    // end belong to the next unit or to nothing, so both operands are cleared there
+    if ((tg.count & 15) && whole % PS == ps) {
+      const int left = tg.count - 16 * whole - 8 * half;     // of this half-wave's eight positions
+      uintx4 a[MT], b[JT];
+      unsigned keep[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) keep[w] = (2 * w < left ? 0xFFFFu : 0u) | (2 * w + 1 < left ? 0xFFFF0000u : 0u);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const unsigned short *src = (const unsigned short *)(An + m_off[i] + 16 * whole);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const unsigned lo = 2 * w < left ? src[2 * w] : 0u;
+          const unsigned hi = 2 * w + 1 < left ? src[2 * w + 1] : 0u;
+          a[i][w] = lo | (hi << 16);
+        }
+      }
+      fetch_b(Xs, whole, b);
+#pragma unroll
+      for (int t = 0; t < JT; ++t)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) b[t][w] &= keep[w];
+      multiply(a, b);
+    }
+  }
+
+  // ---- every wavefront writes its partial block ------------------------------------
+  float *out = ws + ((i64)((int)blockIdx.x * PS + ps) * wp.M_pad + m0) * wp.J_pad + j0;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < JT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        out[(i64)m * wp.J_pad + t * 32 + l32] = acc[i][t][r];
+      }
+}
+
+template <int JT>
+hipError_t launch_f16(const WgradHalfPlan &wp, dim3 grid, const void *a, const void *g, float *ws,
+                      hipStream_t stream) {
+  auto kern = wgrad_f16_kernel<JT>;
+  if (wp.lds_bytes > 64 * 1024) {
+    static thread_local size_t granted = 0;
+    if (granted < wp.lds_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)wp.lds_bytes);
+      if (e != hipSuccess) return e;
+      granted = wp.lds_bytes;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, (const _Float16 *)a,
+                     (const _Float16 *)g, ws);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool make_wgrad_half_plan(const SepConv &fwd_in, WgradHalfPlan &wp) {
+  // (the forward tiling is only borrowed for its staging geometry: plan it for the fp32 kernel)
+  SepConv fwd = fwd_in;
+  fwd.math = MATH_FP32;
+  fwd.in_half = 0;
+  fwd.out_half = 0;
+  fwd.accumulate = 0;
+  size_t lds_fwd;
+  int mt, nt;
+  if (!make_tile_plan(fwd, wp.t, &lds_fwd, &mt, &nt, 1)) return false;
+  TilePlan &pl = wp.t;
+  if (pl.segment || pl.nox_eff < 1 || pl.noy_eff < 1) return false;
+  if ((i64)pl.M * pl.Q >= ((i64)1 << 30)) return false;          // 32-bit element offsets inside an image
+  const bool mellin_x = pl.kind_x == AX_MCORR || pl.kind_x == AX_MCONV;
+  // whole output rows are staged, element by element
+  pl.contig = 0;
+  pl.RS = (pl.ay * (pl.noy - 1) + pl.by_span + 1) | 1;
+  wp.J = pl.C * pl.nf;
+  wp.jt = wp.J > 96 ? 4 : (wp.J + 31) / 32;
+  wp.mbw = pl.M > 128 ? 4 : (pl.M > 64 ? 2 : 1);
+  const int M_T = 64 * wp.mbw, J_T = wp.jt * 32;
+  wp.m_groups = (pl.M + M_T - 1) / M_T;
+  wp.j_groups = (wp.J + J_T - 1) / J_T;
+  wp.M_pad = wp.m_groups * M_T;
+  wp.J_pad = wp.j_groups * J_T;
+  wp.a_n = (i64)pl.M * pl.Q;
+  wp.a_m = pl.Q;
+  wp.CCj = std::min(pl.C, (J_T - 1 + pl.nf - 1) / pl.nf + 1);
+  if ((i64)wp.CCj * pl.ngx * pl.ngy >= ((i64)1 << 30)) return false;
+  // the largest unit whose rows fit twice in the LDS of a workgroup (two to a CU)
+  wp.RB = 0;
+  for (int rb = std::min(pl.nox_eff, 64); rb >= 1; --rb) {
+    const i64 Rr = mellin_x ? (i64)rb * pl.nfx : (i64)pl.ax * (rb - 1) + pl.bx_span + 1;
+    const i64 up = (((i64)rb * pl.noy + 15) / 16) * 16;
+    const i64 xw = ((i64)wp.CCj * Rr * pl.RS + 3) & ~(i64)3;
+    const i64 bytes = 4 * (2 * xw + up);
+    if (Rr > 8192 || up > 4096 || bytes > 76 * 1024) continue;
+    wp.RB = rb;
+    wp.UP = (int)up;
+    pl.R = (int)Rr;
+    wp.lds_bytes = (size_t)bytes;
+    break;
+  }
+  if (!wp.RB) return false;
+  const i64 units = (i64)pl.batch * ((pl.nox_eff + wp.RB - 1) / wp.RB);
+  const int blocks_y = wp.m_groups * wp.j_groups;
+  wp.S = (int)std::min<i64>(std::max<i64>(1, (256 * 2) / blocks_y), units);
+  wp.ws_bytes = (size_t)wp.S * (kWaves / wp.mbw) * wp.M_pad * wp.J_pad * sizeof(float);
+  return true;
+}
+
+hipError_t launch_wgrad_half(const WgradHalfPlan &wp, const void *grad_out, const void *input,
+                             void *grad_weight, float *workspace, hipStream_t stream) {
+  dim3 grid((unsigned)wp.S, (unsigned)(wp.m_groups * wp.j_groups));
+  hipError_t e = hipErrorInvalidValue;
+  if (wp.jt == 1) e = launch_f16<1>(wp, grid, grad_out, input, workspace, stream);
+  if (wp.jt == 2) e = launch_f16<2>(wp, grid, grad_out, input, workspace, stream);
+  if (wp.jt == 3) e = launch_f16<3>(wp, grid, grad_out, input, workspace, stream);
+  if (wp.jt == 4) e = launch_f16<4>(wp, grid, grad_out, input, workspace, stream);
+  if (e != hipSuccess) return e;
+  return launch_wgrad_reduce(workspace, grad_weight, /*half_out=*/true, wp.S * (kWaves / wp.mbw), wp.t.M, wp.J,
+                             wp.M_pad, wp.J_pad, stream);
+}
+
+}  // namespace mellin

@@ -789,8 +789,9 @@ __global__ __launch_bounds__(kThreads, (MT == 1 ? 3 : 2)) void wgrad_stream_kern
 // W[m, j] = sum over the S partial blocks, in index order.  A block of 256
 // threads handles 16 outputs: 16 threads per output add every 16th partial,
 // then thread 0 of each output adds the 16 sums in order.
+template <typename O>                                  // O: float, or _Float16 (rounded once)
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ ws,
-                                                           float *__restrict__ W, int S, int M,
+                                                           O *__restrict__ W, int S, int M,
                                                            int J, int M_pad, int J_pad) {
   __shared__ float part[16][17];
   const int el = threadIdx.x & 15, ph = threadIdx.x >> 4;
@@ -814,7 +815,7 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restri
     float tot = part[0][el];
 #pragma unroll
     for (int k = 1; k < 16; ++k) tot += part[k][el];
-    W[e] = tot;
+    W[e] = (O)tot;
   }
 }
 
@@ -1071,8 +1072,20 @@ hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float 
   }
   if (e != hipSuccess) return e;
   const int outputs = wp.t.M * wp.J;
-  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)((outputs + 15) / 16)), dim3(256), 0, stream,
+  hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3((unsigned)((outputs + 15) / 16)), dim3(256), 0, stream,
                      (const float *)workspace, grad_weight, wp.S, wp.t.M, wp.J, wp.M_pad, wp.J_pad);
+  return hipGetLastError();
+}
+
+hipError_t launch_wgrad_reduce(const float *partials_ws, void *W, bool half_out, int partials, int M, int J,
+                               int M_pad, int J_pad, hipStream_t stream) {
+  const dim3 grid((unsigned)((M * J + 15) / 16));
+  if (half_out)
+    hipLaunchKernelGGL(wgrad_reduce_kernel<_Float16>, grid, dim3(256), 0, stream, partials_ws, (_Float16 *)W,
+                       partials, M, J, M_pad, J_pad);
+  else
+    hipLaunchKernelGGL(wgrad_reduce_kernel<float>, grid, dim3(256), 0, stream, partials_ws, (float *)W, partials,
+                       M, J, M_pad, J_pad);
   return hipGetLastError();
 }
 

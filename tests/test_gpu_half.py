@@ -27,6 +27,8 @@ CASES = [
     ("mcorr", 2, 3, 64, (8, 4), (96, 41), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),     # tap products underneath
     ("lcorr", 2, 40, 70, (3, 3), (30, 20), (2, 1), (1, 2), (1, 1), (1, 1), (1, 0)),    # many channels
     ("mcorr", 4, 6, 9, (6, 1), (50, 1), (1, 1), (1, 1), (2, 0), (2, 1), (0, 0)),       # 1-D
+    ("lcorr", 1, 5, 200, (2, 3), (23, 19), (1, 2), (2, 1), (1, 2), (1, 1), (0, 1)),    # four channel blocks side by side in the weight gradient
+    ("mcorr", 3, 2, 100, (3, 2), (31, 3), (2, 1), (1, 1), (1, 0), (1, 1), (3, 0)),     # two; rows of two outputs, twelve columns
 ]
 
 
@@ -73,7 +75,72 @@ def test_half_passes_match_checker_on_the_same_operands(case, half_path):
     _close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
     gw = torch.full_like(wg, float("nan"))
     hip.corr2d_backward_weight(kind_x, xg, to_gpu(go), gw, dims)
+    assert (hip.last_variant() == "mfma-f16") == (half_path == "auto")
     _close(gw, egw, n * nh[0] * nh[1], "grad_weight %s" % (case,))
+
+
+def test_random_layers_agree_between_the_two_half_paths():
+    """Random layers (Mellin and linear, 1-D and 2-D, strides, dilations, paddings, extra
+    output rows, one to 260 channels): what the kernels that read half tensors give must be
+    what the fp32 kernels give on fp32 copies, up to the rounding of the result to half and
+    fp32 summation order."""
+    rng = np.random.default_rng(2024)
+    seen = {}
+    done = 0
+    while done < 160:
+        mell = bool(rng.integers(2))
+        kind_x = hip.AX_MCORR if mell else hip.AX_LCORR
+        n = int(rng.integers(1, 6))
+        c_in = int(rng.choice([1, 3, 8, 16, 20, 33, 64, 130, 260]))
+        c_out = int(rng.choice([3, 16, 33, 64, 70, 130, 260]))
+        nf = [(8, 4), (4, 4), (2, 4), (4, 2), (3, 8), (1, 8), (8, 1), (5, 5), (3, 3), (1, 1), (3, 1)][int(rng.integers(11))]
+        ng = (int(rng.integers(nf[0], 60)), int(rng.choice([3, 5, 8, 9, 13, 16, 20, 33, 41, 64, 130])))
+        if rng.integers(6) == 0:
+            nf, ng = (nf[0], 1), (int(rng.integers(nf[0], 300)), 1)
+        if ng[1] < nf[1]:
+            continue
+        s = (int(rng.integers(1, 3)), int(rng.integers(1, 3)) if ng[1] > 1 else 1)
+        d = (int(rng.integers(1, 3)), int(rng.integers(1, 3)) if ng[1] > 1 else 1)
+        p = (int(rng.integers(0, 4)), int(rng.integers(0, 3)) if ng[1] > 1 else 0)
+        r = (int(rng.choice([0, 0, 3, 10])), int(rng.choice([0, 0, 1])) if ng[1] > 1 else 0)
+        size_x = mconv.mcorr_valid_size if mell else mconv.lcorr_valid_size
+        nh = (size_x(nf[0], ng[0], s[0], d[0], p[0], 1) + r[0],
+              mconv.lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], 1) + r[1])
+        if min(nh) <= 0 or n * c_out * nh[0] * nh[1] * c_in * nf[0] * nf[1] > 1e9:
+            continue
+        dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, (1, 1))
+        x = to_gpu(rng.standard_normal((n, c_in) + ng).astype(np.float16))
+        w = to_gpu((rng.standard_normal((c_out, c_in) + nf) * (c_in * nf[0] * nf[1]) ** -0.5).astype(np.float16))
+        b = to_gpu(rng.standard_normal(c_out).astype(np.float16))
+        go = to_gpu((0.1 * rng.standard_normal((n, c_out) + nh)).astype(np.float16))
+        got = {}
+        for variant in ("widen", "auto"):
+            hip.set_variant(variant)
+            try:
+                out = torch.full((n, c_out) + nh, float("nan"), dtype=torch.float16, device="cuda")
+                gi, gw = torch.full_like(x, float("nan")), torch.full_like(w, float("nan"))
+                names = []
+                hip.corr2d_forward(kind_x, x, w, b, out, dims)
+                names.append(hip.last_variant())
+                hip.corr2d_backward_input(kind_x, w, go, gi, dims)
+                names.append(hip.last_variant())
+                hip.corr2d_backward_weight(kind_x, x, go, gw, dims)
+                names.append(hip.last_variant())
+                got[variant] = (out.float(), gi.float(), gw.float())
+            finally:
+                hip.set_variant(None)
+            if variant == "auto":
+                for pass_, name in zip(("forward", "input", "weight"), names):
+                    seen[(pass_, name)] = seen.get((pass_, name), 0) + 1
+        fans = (c_in * nf[0] * nf[1], c_out * nf[0] * nf[1], n * nh[0] * nh[1])
+        for i, what in enumerate(("out", "grad_input", "grad_weight")):
+            ref, res = got["widen"][i], got["auto"][i]
+            tol = 2.0 ** -10 * ref.abs() + 2e-5 * fans[i] ** 0.5 * (0.1 if i else 1.0) + 1e-7
+            assert bool(((ref - res).abs() <= tol).all()), (what, mell, n, c_in, c_out, nf, ng, s, d, p, r)
+        done += 1
+    # the sample exercised every kernel that reads half tensors
+    assert seen.get(("forward", "mfma-f16"), 0) > 100 and seen.get(("weight", "mfma-f16"), 0) > 100
+    assert seen.get(("input", "mfma-f16"), 0) > 30 and seen.get(("input", "mfma-f16+fold"), 0) > 10, seen
 
 
 def test_workspace_is_required_and_sized():
