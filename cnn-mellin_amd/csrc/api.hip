@@ -757,10 +757,12 @@ size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;
   HalfNative hn;
-  if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
-    return hn.frag_bytes;
+  // (the two-pass form where the fp32 path would take it: few input channels, or a Mellin
+  // axis that keeps fewer rows than it is given)
   TwoPassInput tp;
   if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) return align256(tp.ws_bytes) + (size_t)n_in * 4;
+  if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
+    return hn.frag_bytes;
   return half_layout(n_w, n_out, 0, n_in, mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS)).total;
 }
 int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void *grad_out, MELLIN_CORR2D_DIMS,
@@ -771,10 +773,11 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
   if (n_in == 0) return MELLIN_OK;
   {
     HalfNative hn;
-    if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
-      return run_half_native(__func__, hn, weight, grad_out, nullptr, grad_input, workspace, workspace_bytes, stream);
     TwoPassInput tp;
-    if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) {
+    const bool two_pass = plan_half_two_pass(kind_x, CORR2D_ARGS, tp);
+    if (!two_pass && c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
+      return run_half_native(__func__, hn, weight, grad_out, nullptr, grad_input, workspace, workspace_bytes, stream);
+    if (two_pass) {
       // the two-pass form on the half-precision tensors: first-pass rows and the folded
       // result in fp32 in the workspace, one rounding on the way out
       const size_t gi_off = align256(tp.ws_bytes), need = gi_off + (size_t)n_in * 4;

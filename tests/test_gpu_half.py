@@ -339,10 +339,12 @@ def test_wide_layers_read_their_filter_from_fragments_in_the_workspace():
         go = torch.randn(ref.shape, generator=gen).half().cuda()
         gi32 = torch.empty_like(x, dtype=torch.float32)
         hip.corr2d_backward_input(kind_x, w.float(), go.float(), gi32, dims)
-        assert 0 < hip.lib.mellin_corr2d_backward_input_f16_workspace(kind_x, *dims) <= 2 * 2 * w.numel() * 2
         gi = torch.empty_like(x)
         hip.corr2d_backward_input(kind_x, w, go, gi, dims)
-        assert hip.last_variant() == "mfma-f16"
+        # (this Mellin layer keeps fewer rows than it is given: the two-pass form, as in fp32)
+        assert hip.last_variant() == ("mfma-f16" if kind_x == hip.AX_LCORR else "mfma-f16+fold")
+        if kind_x == hip.AX_LCORR:
+            assert 0 < hip.lib.mellin_corr2d_backward_input_f16_workspace(kind_x, *dims) <= 2 * 2 * w.numel() * 2
         tol = 2.0 ** -10 * gi32.abs().clamp_min(2.0 ** -14) + 1e-5 * (c_out * 9) ** 0.5
         assert bool(((gi.float() - gi32).abs() <= tol).all())
         # too little scratch memory is an error, not a slower path

@@ -3,14 +3,16 @@ prints one JSON record per layer (the 1-D grid of config 2: sixteen layers, a se
 import json
 
 import pytest
+import torch
 
 import time_layers
 
 pytestmark = pytest.mark.gpu
 
 
-def test_config2_grid_runs_on_the_matrix_core_kernels(capsys):
-    time_layers.run_cfg2(reps=1)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["float32", "half"])
+def test_config2_grid_runs_on_the_matrix_core_kernels(capsys, dtype):
+    time_layers.run_cfg2(reps=1, dtype=dtype)
     records = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
     assert len(records) == 16
     t_out = {(r["layer"].split()[1], r["layer"].split(" ", 2)[2]): r["out"][1] for r in records}
@@ -19,4 +21,5 @@ def test_config2_grid_runs_on_the_matrix_core_kernels(capsys):
         assert r["in"] == [41, 780, 1] and r["out"][0] == 128
         for name in ("forward", "grad_input", "grad_weight"):
             assert r[name]["variant"].startswith("mfma"), r
+            assert (r[name]["math"] == "f16") == (dtype == torch.float16), r
             assert r[name]["us"] > 0 and r[name]["tflops"] > 0

@@ -4,6 +4,7 @@
     python time_layers.py cfg4            # wide 2-D layer, linear and Mellin x axis
     python time_layers.py cfg2            # 1-D layers over the (s, d, p) grid
     python time_layers.py stack           # the 10-layer 3 -> 256 stacks, layer by layer
+    python time_layers.py cfg4 --dtype half   # the same on half-precision tensors (the stack: under autocast)
 
 Every pass is one call of the C ABI on pre-allocated tensors, timed with HIP events
 on the launch stream.  One JSON object per line: the layer, its output extent, and
@@ -67,32 +68,32 @@ def time_layer(tag, kind_x, x, w, b, s, d, p, r, reps, activation=None):
                      ("grad_weight", lambda: hip.corr2d_backward_weight(kind_x, x, go, gw, dims))):
         us = event_us(fn, reps)
         rec[name] = {"us": round(us, 1), "variant": hip.last_variant(),
-                     "math": "bf16x3" if hip.last_math() == hip.MATH_BF16X3 else "fp32",
+                     "math": {hip.MATH_BF16X3: "bf16x3", hip.MATH_F16: "f16"}.get(hip.last_math(), "fp32"),
                      "tflops": round(2 * macs / us / 1e6, 1)}
     return rec, out
 
 
-def run_cfg4(reps):
+def run_cfg4(reps, dtype):
     import torch
     import _mellin_hip as hip
     gen = torch.Generator(device="cuda").manual_seed(3)
-    x = torch.randn(32, 128, 256, 41, device="cuda", generator=gen)
+    x = torch.randn(32, 128, 256, 41, device="cuda", generator=gen).to(dtype)
     bound = (128 * 9) ** -0.5
-    w = (torch.rand(256, 128, 3, 3, device="cuda", generator=gen) * 2 - 1) * bound
-    b = (torch.rand(256, device="cuda", generator=gen) * 2 - 1) * bound
+    w = ((torch.rand(256, 128, 3, 3, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(256, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
     for kind, name in ((hip.AX_LCORR, "lconv2d"), (hip.AX_MCORR, "mconv2d")):
         rec, _ = time_layer("cfg4 " + name, kind, x, w, b, (1, 1), (2, 1), (2, 1), (2, 1), reps)
         print(json.dumps(rec), flush=True)
 
 
-def run_cfg2(reps):
+def run_cfg2(reps, dtype):
     import torch
     import _mellin_hip as hip
     gen = torch.Generator(device="cuda").manual_seed(1)
-    x = torch.randn(32, 41, 780, 1, device="cuda", generator=gen)
+    x = torch.randn(32, 41, 780, 1, device="cuda", generator=gen).to(dtype)
     bound = (41 * 8) ** -0.5
-    w = (torch.rand(128, 41, 8, 1, device="cuda", generator=gen) * 2 - 1) * bound
-    b = (torch.rand(128, device="cuda", generator=gen) * 2 - 1) * bound
+    w = ((torch.rand(128, 41, 8, 1, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(128, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
     for s in (1, 2):
         for d in (1, 2):
             for p in (0, 3):
@@ -102,7 +103,7 @@ def run_cfg2(reps):
                     print(json.dumps(rec), flush=True)
 
 
-def run_stack(reps):
+def run_stack(reps, dtype):
     import time
     import torch
     import _mellin_hip as hip
@@ -117,7 +118,10 @@ def run_stack(reps):
 
         def step():
             # the conv stack and its Linear -> 62 log-softmax head, summed over frames
-            model(x).square().mean().backward()
+            # (half: fp32 parameters, the layers cast their operands under autocast)
+            with torch.autocast("cuda", enabled=dtype == torch.float16):
+                loss = model(x).float().square().mean()
+            loss.backward()
         for _ in range(3):
             step()
         torch.cuda.synchronize()
@@ -128,11 +132,11 @@ def run_stack(reps):
         name = "mellin" if mellin else "linear"
         print(json.dumps({"stack": name, "forward_backward_ms": round((time.perf_counter() - t0) / reps * 1e3, 2)}),
               flush=True)
-        h = x.detach()
+        h = x.detach().to(dtype)
         for no, (lay, conv) in enumerate(zip(stack.plan, stack.convs), 1):
             kind = hip.AX_MCORR if lay["kind"] == "mcorrlcorr" else hip.AX_LCORR
-            rec, out = time_layer("%s stack layer %d" % (name, no), kind, h, conv.weight.detach(),
-                                  conv.bias.detach() if conv.bias is not None else None,
+            rec, out = time_layer("%s stack layer %d" % (name, no), kind, h, conv.weight.detach().to(dtype),
+                                  conv.bias.detach().to(dtype) if conv.bias is not None else None,
                                   lay["s"], lay["d"], lay["p"], lay["r"], reps)
             print(json.dumps(rec), flush=True)
             h = torch.relu(out)
@@ -146,6 +150,8 @@ def main():
     ap.add_argument("--reps", type=int, default=10, help="timed calls per pass")
     ap.add_argument("--math", choices=["bf16x3", "fp32"], default="bf16x3",
                     help="how the matrix kernels form fp32 products (library default: bf16x3)")
+    ap.add_argument("--dtype", choices=["float32", "half"], default="float32",
+                    help="half: half-precision tensors through the f16 entry points")
     args = ap.parse_args()
     import torch
     if not torch.cuda.is_available():
@@ -153,7 +159,8 @@ def main():
     torch.cuda.set_device(0)
     import _mellin_hip as hip
     hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
-    {"cfg2": run_cfg2, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps)
+    dtype = torch.float16 if args.dtype == "half" else torch.float32
+    {"cfg2": run_cfg2, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps, dtype)
 
 
 if __name__ == "__main__":
