@@ -50,9 +50,10 @@ SYMBOLS = {
 SYMBOLS["mellin_corr2d_forward_workspace"] = (_size_t, [_int, _int] + _DIMS)
 SYMBOLS["mellin_corr2d_forward_ws_f32"] = (_int, [_int, _int, _ptr, _ptr, _ptr] + _DIMS + [_ptr, _ptr, _size_t, _ptr])
 SYMBOLS["mellin_bias_grad_workspace"] = (_size_t, [_i64, _i64, _i64])
-SYMBOLS["mellin_bias_grad_f32"] = (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
-SYMBOLS["mellin_pool_pairs_forward_f32"] = (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr])
-SYMBOLS["mellin_pool_pairs_backward_f32"] = (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr])
+for _t in ("f32", "f16"):
+    SYMBOLS["mellin_bias_grad_" + _t] = (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _size_t, _ptr])
+    SYMBOLS["mellin_pool_pairs_forward_" + _t] = (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr])
+    SYMBOLS["mellin_pool_pairs_backward_" + _t] = (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr])
 SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
 SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
@@ -238,7 +239,7 @@ def log_lift_backward(x, grad_y, eps, tau, flags, outer, t, inner, grad_x, grad_
 
 
 def bias_grad(grad_out, out=None):
-    """(g, grad_bias) for a dense float32 grad_out (N, C, ...): grad_bias = per-channel sums of g, with
+    """(g, grad_bias) for a dense float32 or float16 grad_out (N, C, ...): grad_bias = per-channel sums of g, with
     g = grad_out, or grad_out where `out` > 0 (the backward of a ReLU fused into the forward pass)."""
     dev = require_device(grad_out, out)
     _same_dtype(grad_out, out)
@@ -249,20 +250,28 @@ def bias_grad(grad_out, out=None):
     need = lib.mellin_bias_grad_workspace(n, c, plane)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _check(lib.mellin_bias_grad_f32(_dp(grad_out), _dp(out), n, c, plane, _dp(g) if out is not None else None,
-                                        _dp(grad_bias), _ptr(ws.data_ptr()), need, _stream(dev)))
+        fn = getattr(lib, "mellin_bias_grad_" + _pointwise_suffix(grad_out))
+        _check(fn(_dp(grad_out), _dp(out), n, c, plane, _dp(g) if out is not None else None,
+                  _dp(grad_bias), _ptr(ws.data_ptr()), need, _stream(dev)))
     return g, grad_bias
 
 
+def _pointwise_suffix(t):
+    if t.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("float32 or float16 tensors only, got %s" % t.dtype)
+    return _SUFFIX[t.dtype]
+
+
 def pool_pairs_forward(x):
-    """(y, which) for a dense float32 x (..., f): maxima over pairs of neighbours along the last axis."""
+    """(y, which) for a dense float32 or float16 x (..., f): maxima over pairs of neighbours along the last axis."""
     dev = require_device(x)
     f = x.shape[-1]
     rows = x.numel() // f if f else 0
     y = torch.empty(x.shape[:-1] + (f // 2,), dtype=x.dtype, device=dev)
     which = torch.empty(y.shape, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _check(lib.mellin_pool_pairs_forward_f32(_dp(x), rows, f, _dp(y), _dp(which), _stream(dev)))
+        fn = getattr(lib, "mellin_pool_pairs_forward_" + _pointwise_suffix(x))
+        _check(fn(_dp(x), rows, f, _dp(y), _dp(which), _stream(dev)))
     return y, which
 
 
@@ -271,7 +280,8 @@ def pool_pairs_backward(grad_y, which, f):
     grad_x = torch.empty(grad_y.shape[:-1] + (f,), dtype=grad_y.dtype, device=dev)
     rows = grad_x.numel() // f if f else 0
     with torch.cuda.device(dev):
-        _check(lib.mellin_pool_pairs_backward_f32(_dp(grad_y), _dp(which), rows, f, _dp(grad_x), _stream(dev)))
+        fn = getattr(lib, "mellin_pool_pairs_backward_" + _pointwise_suffix(grad_y))
+        _check(fn(_dp(grad_y), _dp(which), rows, f, _dp(grad_x), _stream(dev)))
     return grad_x
 
 

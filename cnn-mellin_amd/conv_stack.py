@@ -24,7 +24,7 @@ __all__ = ["ConvStackParams", "ConvStack", "FrameClassifier", "layer_plan", "pac
 
 
 class _FreqMaxPool(torch.autograd.Function):
-    """max_pool2d(x, (1, 2)) for dense float32 GPU tensors through the library's pair kernels:
+    """max_pool2d(x, (1, 2)) for dense float32 or float16 GPU tensors through the library's pair kernels:
     one byte per output is kept for the backward pass instead of PyTorch's 8-byte indices."""
 
     @staticmethod
@@ -42,7 +42,7 @@ class _FreqMaxPool(torch.autograd.Function):
 
 def freq_max_pool(x: torch.Tensor) -> torch.Tensor:
     """Maximum over pairs of neighbouring frequency bins, ``max_pool2d(x, (1, 2))``."""
-    if x.is_cuda and x.dtype == torch.float32:
+    if x.is_cuda and x.dtype in (torch.float32, torch.float16):
         return _FreqMaxPool.apply(x)
     return torch.nn.functional.max_pool2d(x, (1, 2))
 

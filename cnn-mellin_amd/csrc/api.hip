@@ -687,6 +687,49 @@ HalfLayout half_layout(i64 a, i64 b, i64 bias, i64 r, size_t inner) {
   const i64 n_in = batch * c_in * ngx * ngy, n_w = c_out * c_in * nfx * nfy,      \
             n_out = batch * c_out * nhx * nhy
 
+template <typename T>
+int bias_grad_entry(const char *fn, const T *grad_out, const T *out, int64_t batch, int64_t channels, int64_t plane,
+                    T *grad_masked, T *grad_bias, void *workspace, size_t workspace_bytes, void *stream) {
+  if (batch < 0 || channels < 0 || plane < 0)
+    return fail(MELLIN_ERR_ARGUMENT, "%s: negative extent", fn);
+  if (batch > 65535 || channels > 65535 || plane > ((int64_t)1 << 40))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: at most 65535 images and channels (got %lld, %lld)", fn, (long long)batch,
+                (long long)channels);
+  if (channels == 0) return MELLIN_OK;
+  if (!grad_bias) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  const size_t need = bias_grad_workspace_bytes(batch, channels, plane);
+  if (need && (!grad_out || (out && !grad_masked))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  if (need && (!workspace || workspace_bytes < need))
+    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, need, workspace_bytes);
+  hipError_t e = launch_bias_grad(grad_out, out, batch, channels, plane, grad_masked, grad_bias, (float *)workspace,
+                                  (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
+template <typename T>
+int pool_pairs_forward_entry(const char *fn, const T *x, int64_t rows, int64_t f, T *y, unsigned char *which,
+                             void *stream) {
+  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
+  if (rows * (f / 2) == 0) return MELLIN_OK;
+  if (!x || !y || !which) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e = launch_pool_pairs_forward(x, rows, f, y, which, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+template <typename T>
+int pool_pairs_backward_entry(const char *fn, const T *grad_y, const unsigned char *which, int64_t rows, int64_t f,
+                              T *grad_x, void *stream) {
+  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
+    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
+  if (rows * f == 0) return MELLIN_OK;
+  if (!grad_x || (f / 2 && (!grad_y || !which))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
+  hipError_t e = launch_pool_pairs_backward(grad_y, which, rows, f, grad_x, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
+  return MELLIN_OK;
+}
+
 extern "C" {
 
 int mellin_version(void) { return 100; }
@@ -915,45 +958,31 @@ size_t mellin_bias_grad_workspace(int64_t batch, int64_t channels, int64_t plane
 int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch, int64_t channels, int64_t plane,
                          float *grad_masked, float *grad_bias, void *workspace, size_t workspace_bytes,
                          void *stream) {
-  const char *fn = __func__;
-  if (batch < 0 || channels < 0 || plane < 0)
-    return fail(MELLIN_ERR_ARGUMENT, "%s: negative extent", fn);
-  if (batch > 65535 || channels > 65535 || plane > ((int64_t)1 << 40))
-    return fail(MELLIN_ERR_ARGUMENT, "%s: at most 65535 images and channels (got %lld, %lld)", fn, (long long)batch,
-                (long long)channels);
-  if (channels == 0) return MELLIN_OK;
-  if (!grad_bias) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  const size_t need = bias_grad_workspace_bytes(batch, channels, plane);
-  if (need && (!grad_out || (out && !grad_masked))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  if (need && (!workspace || workspace_bytes < need))
-    return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", fn, need, workspace_bytes);
-  hipError_t e = launch_bias_grad(grad_out, out, batch, channels, plane, grad_masked, grad_bias, (float *)workspace,
-                                  (hipStream_t)stream);
-  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
-  return MELLIN_OK;
+  return bias_grad_entry<float>(__func__, grad_out, out, batch, channels, plane, grad_masked, grad_bias, workspace,
+                                workspace_bytes, stream);
 }
-
+int mellin_bias_grad_f16(const void *grad_out, const void *out, int64_t batch, int64_t channels, int64_t plane,
+                         void *grad_masked, void *grad_bias, void *workspace, size_t workspace_bytes,
+                         void *stream) {
+  return bias_grad_entry<_Float16>(__func__, (const _Float16 *)grad_out, (const _Float16 *)out, batch, channels, plane,
+                                   (_Float16 *)grad_masked, (_Float16 *)grad_bias, workspace, workspace_bytes, stream);
+}
 int mellin_pool_pairs_forward_f32(const float *x, int64_t rows, int64_t f, float *y, unsigned char *which,
                                   void *stream) {
-  const char *fn = __func__;
-  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
-    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
-  if (rows * (f / 2) == 0) return MELLIN_OK;
-  if (!x || !y || !which) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  hipError_t e = launch_pool_pairs_forward(x, rows, f, y, which, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
-  return MELLIN_OK;
+  return pool_pairs_forward_entry<float>(__func__, x, rows, f, y, which, stream);
+}
+int mellin_pool_pairs_forward_f16(const void *x, int64_t rows, int64_t f, void *y, unsigned char *which,
+                                  void *stream) {
+  return pool_pairs_forward_entry<_Float16>(__func__, (const _Float16 *)x, rows, f, (_Float16 *)y, which, stream);
 }
 int mellin_pool_pairs_backward_f32(const float *grad_y, const unsigned char *which, int64_t rows, int64_t f,
                                    float *grad_x, void *stream) {
-  const char *fn = __func__;
-  if (rows < 0 || f < 0 || rows > ((int64_t)1 << 40) || f > ((int64_t)1 << 30) || rows * f > ((int64_t)1 << 44))
-    return fail(MELLIN_ERR_ARGUMENT, "%s: extents out of range (%lld rows of %lld)", fn, (long long)rows, (long long)f);
-  if (rows * f == 0) return MELLIN_OK;
-  if (!grad_x || (f / 2 && (!grad_y || !which))) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  hipError_t e = launch_pool_pairs_backward(grad_y, which, rows, f, grad_x, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(MELLIN_ERR_RUNTIME, "%s: %s", fn, hipGetErrorString(e));
-  return MELLIN_OK;
+  return pool_pairs_backward_entry<float>(__func__, grad_y, which, rows, f, grad_x, stream);
+}
+int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *which, int64_t rows, int64_t f,
+                                   void *grad_x, void *stream) {
+  return pool_pairs_backward_entry<_Float16>(__func__, (const _Float16 *)grad_y, which, rows, f, (_Float16 *)grad_x,
+                                             stream);
 }
 
 int mellin_set_math(int mode) {

@@ -151,13 +151,17 @@ hipError_t launch_log_lift_backward(const T *x, const T *gy, T eps, T tau, bool 
 // pointwise.hip: per-channel sums of grad_out (N, C, plane), optionally masked by out > 0 (the masked
 // gradient is then written to grad_masked); workspace of bias_grad_workspace_bytes()
 size_t bias_grad_workspace_bytes(i64 batch, i64 channels, i64 plane);
-hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, i64 channels, i64 plane,
-                            float *grad_masked, float *grad_bias, float *workspace, hipStream_t stream);
+// (T: float or _Float16; the sums are fp32 either way)
+template <typename T>
+hipError_t launch_bias_grad(const T *grad_out, const T *out, i64 batch, i64 channels, i64 plane,
+                            T *grad_masked, T *grad_bias, float *workspace, hipStream_t stream);
 
 // pointwise.hip: max over pairs of neighbours along the last axis of x (rows, f), and its backward
-hipError_t launch_pool_pairs_forward(const float *x, i64 rows, i64 f, float *y, unsigned char *which,
+template <typename T>
+hipError_t launch_pool_pairs_forward(const T *x, i64 rows, i64 f, T *y, unsigned char *which,
                                      hipStream_t stream);
-hipError_t launch_pool_pairs_backward(const float *gy, const unsigned char *which, i64 rows, i64 f, float *gx,
+template <typename T>
+hipError_t launch_pool_pairs_backward(const T *gy, const unsigned char *which, i64 rows, i64 f, T *gx,
                                       hipStream_t stream);
 
 // half <-> float copies of n elements (16 bytes at a time when both buffers are 16-byte aligned)

@@ -181,10 +181,11 @@ namespace {
 
 constexpr int kBiasChunk = 4096;
 
-template <bool MASK>
-__global__ __launch_bounds__(kPwThreads) void bias_grad_kernel(const float *__restrict__ go,
-                                                               const float *__restrict__ out,
-                                                               float *__restrict__ gm, float *__restrict__ partial,
+// T: float, or _Float16 (sums in fp32 either way)
+template <bool MASK, typename T>
+__global__ __launch_bounds__(kPwThreads) void bias_grad_kernel(const T *__restrict__ go,
+                                                               const T *__restrict__ out,
+                                                               T *__restrict__ gm, float *__restrict__ partial,
                                                                i64 plane, int chunks) {
   __shared__ float red[kPwThreads / 64];
   const int chunk = blockIdx.x, c = blockIdx.y, n = blockIdx.z, C = gridDim.y, N = gridDim.z;
@@ -193,12 +194,12 @@ __global__ __launch_bounds__(kPwThreads) void bias_grad_kernel(const float *__re
   float s = 0.f;
 #pragma unroll 4
   for (int i = threadIdx.x; i < len; i += kPwThreads) {
-    float v = go[base + i];
+    T v = go[base + i];
     if (MASK) {
-      v = out[base + i] > 0.f ? v : 0.f;
+      v = out[base + i] > (T)0 ? v : (T)0;
       gm[base + i] = v;
     }
-    s += v;
+    s += (float)v;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) s += __shfl_down(s, o);
@@ -211,14 +212,15 @@ __global__ __launch_bounds__(kPwThreads) void bias_grad_kernel(const float *__re
   }
 }
 
+template <typename T>                                  // T: type of the result (rounded once)
 __global__ __launch_bounds__(64) void bias_reduce_kernel(const float *__restrict__ partial, i64 per_channel,
-                                                         float *__restrict__ grad_bias) {
+                                                         T *__restrict__ grad_bias) {
   const float *p = partial + (i64)blockIdx.x * per_channel;
   float a = 0.f;
   for (i64 i = threadIdx.x; i < per_channel; i += 64) a += p[i];
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) a += __shfl_down(a, o);
-  if (threadIdx.x == 0) grad_bias[blockIdx.x] = a;
+  if (threadIdx.x == 0) grad_bias[blockIdx.x] = (T)a;
 }
 
 }  // namespace
@@ -229,28 +231,33 @@ size_t bias_grad_workspace_bytes(i64 batch, i64 channels, i64 plane) {
   return (size_t)(batch * channels * chunks) * sizeof(float);
 }
 
-hipError_t launch_bias_grad(const float *grad_out, const float *out, i64 batch, i64 channels, i64 plane,
-                            float *grad_masked, float *grad_bias, float *workspace, hipStream_t stream) {
+template <typename T>
+hipError_t launch_bias_grad(const T *grad_out, const T *out, i64 batch, i64 channels, i64 plane,
+                            T *grad_masked, T *grad_bias, float *workspace, hipStream_t stream) {
   if (channels <= 0) return hipSuccess;
   if (batch <= 0 || plane <= 0) {                       // empty sums
-    hipLaunchKernelGGL(bias_reduce_kernel, dim3((unsigned)channels), dim3(64), 0, stream, workspace, (i64)0,
+    hipLaunchKernelGGL(bias_reduce_kernel<T>, dim3((unsigned)channels), dim3(64), 0, stream, workspace, (i64)0,
                        grad_bias);
     return hipGetLastError();
   }
   const i64 chunks = (plane + kBiasChunk - 1) / kBiasChunk;
   const dim3 grid((unsigned)chunks, (unsigned)channels, (unsigned)batch);
   if (out)
-    hipLaunchKernelGGL(bias_grad_kernel<true>, grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
+    hipLaunchKernelGGL((bias_grad_kernel<true, T>), grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
                        workspace, plane, (int)chunks);
   else
-    hipLaunchKernelGGL(bias_grad_kernel<false>, grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
+    hipLaunchKernelGGL((bias_grad_kernel<false, T>), grid, dim3(kPwThreads), 0, stream, grad_out, out, grad_masked,
                        workspace, plane, (int)chunks);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(bias_reduce_kernel, dim3((unsigned)channels), dim3(64), 0, stream, workspace, batch * chunks,
+  hipLaunchKernelGGL(bias_reduce_kernel<T>, dim3((unsigned)channels), dim3(64), 0, stream, workspace, batch * chunks,
                      grad_bias);
   return hipGetLastError();
 }
+template hipError_t launch_bias_grad<float>(const float *, const float *, i64, i64, i64, float *, float *, float *,
+                                            hipStream_t);
+template hipError_t launch_bias_grad<_Float16>(const _Float16 *, const _Float16 *, i64, i64, i64, _Float16 *,
+                                               _Float16 *, float *, hipStream_t);
 
 // ---- max over pairs of neighbours along the last axis (frequency pooling, window 2) -----
 // y[r, j] = max(x[r, 2 j], x[r, 2 j + 1]) for x (rows, f), j < f / 2 (an odd last column is
@@ -261,77 +268,88 @@ namespace {
 
 // I: index type (unsigned 32-bit when rows * f fits: a 64-bit division per element costs more
 // than the memory traffic)
-template <typename I>
-__global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const float *__restrict__ x, I rows, I f,
-                                                                        I fo, float *__restrict__ y,
+template <typename I, typename T>
+__global__ __launch_bounds__(kPwThreads) void pool_pairs_forward_kernel(const T *__restrict__ x, I rows, I f,
+                                                                        I fo, T *__restrict__ y,
                                                                         unsigned char *__restrict__ which) {
   const I total = rows * fo;
   for (I i = (I)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (I)gridDim.x * kPwThreads) {
     const I r = i / fo, j = i - r * fo;
-    const float a = x[r * f + 2 * j], b = x[r * f + 2 * j + 1];
+    const T a = x[r * f + 2 * j], b = x[r * f + 2 * j + 1];
     const bool second = b > a || b != b;
     y[i] = second ? b : a;
     which[i] = second ? 1 : 0;
   }
 }
 
-__global__ __launch_bounds__(kPwThreads) void zero_words_kernel(float *__restrict__ p, i64 n) {
-  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < n; i += (i64)gridDim.x * kPwThreads) p[i] = 0.f;
+template <typename T>
+__global__ __launch_bounds__(kPwThreads) void zero_words_kernel(T *__restrict__ p, i64 n) {
+  for (i64 i = (i64)blockIdx.x * kPwThreads + threadIdx.x; i < n; i += (i64)gridDim.x * kPwThreads) p[i] = (T)0;
 }
 
 // one thread per pair: both words of the pair, and the odd last column with the row's last pair
-template <typename I>
-__global__ __launch_bounds__(kPwThreads) void pool_pairs_backward_kernel(const float *__restrict__ gy,
+template <typename I, typename T>
+__global__ __launch_bounds__(kPwThreads) void pool_pairs_backward_kernel(const T *__restrict__ gy,
                                                                          const unsigned char *__restrict__ which,
                                                                          I rows, I f, I fo,
-                                                                         float *__restrict__ gx) {
+                                                                         T *__restrict__ gx) {
   const I total = rows * fo;
   for (I i = (I)blockIdx.x * kPwThreads + threadIdx.x; i < total; i += (I)gridDim.x * kPwThreads) {
     const I r = i / fo, j = i - r * fo;
-    const float g = gy[i];
+    const T g = gy[i];
     const bool second = which[i] != 0;
-    float *o = gx + r * f + 2 * j;
-    o[0] = second ? 0.f : g;
-    o[1] = second ? g : 0.f;
-    if (j == fo - 1 && (f & 1)) o[2] = 0.f;
+    T *o = gx + r * f + 2 * j;
+    o[0] = second ? (T)0 : g;
+    o[1] = second ? g : (T)0;
+    if (j == fo - 1 && (f & 1)) o[2] = (T)0;
   }
 }
 
 }  // namespace
 
-hipError_t launch_pool_pairs_forward(const float *x, i64 rows, i64 f, float *y, unsigned char *which,
+template <typename T>
+hipError_t launch_pool_pairs_forward(const T *x, i64 rows, i64 f, T *y, unsigned char *which,
                                      hipStream_t stream) {
   const i64 fo = f / 2;
   if (rows <= 0 || fo <= 0) return hipSuccess;
   const i64 blocks = std::min<i64>((rows * fo + kPwThreads - 1) / kPwThreads, 1 << 20);
   if (rows * f < ((i64)1 << 31))
-    hipLaunchKernelGGL(pool_pairs_forward_kernel<unsigned>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x,
+    hipLaunchKernelGGL((pool_pairs_forward_kernel<unsigned, T>), dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x,
                        (unsigned)rows, (unsigned)f, (unsigned)fo, y, which);
   else
-    hipLaunchKernelGGL(pool_pairs_forward_kernel<i64>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x, rows,
+    hipLaunchKernelGGL((pool_pairs_forward_kernel<i64, T>), dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, x, rows,
                        f, fo, y, which);
   return hipGetLastError();
 }
 
-hipError_t launch_pool_pairs_backward(const float *gy, const unsigned char *which, i64 rows, i64 f, float *gx,
+template hipError_t launch_pool_pairs_forward<float>(const float *, i64, i64, float *, unsigned char *, hipStream_t);
+template hipError_t launch_pool_pairs_forward<_Float16>(const _Float16 *, i64, i64, _Float16 *, unsigned char *,
+                                                        hipStream_t);
+
+template <typename T>
+hipError_t launch_pool_pairs_backward(const T *gy, const unsigned char *which, i64 rows, i64 f, T *gx,
                                       hipStream_t stream) {
   if (rows <= 0 || f <= 0) return hipSuccess;
   const i64 fo = f / 2;
   if (fo == 0) {                                        // one column: nothing was pooled (a kernel, not a memset
     // node: the call may be recorded into a graph)
-    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)std::min<i64>((rows + kPwThreads - 1) / kPwThreads, 4096)),
+    hipLaunchKernelGGL(zero_words_kernel<T>, dim3((unsigned)std::min<i64>((rows + kPwThreads - 1) / kPwThreads, 4096)),
                        dim3(kPwThreads), 0, stream, gx, rows);
     return hipGetLastError();
   }
   const i64 blocks = std::min<i64>((rows * fo + kPwThreads - 1) / kPwThreads, 1 << 20);
   if (rows * f < ((i64)1 << 31))
-    hipLaunchKernelGGL(pool_pairs_backward_kernel<unsigned>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
+    hipLaunchKernelGGL((pool_pairs_backward_kernel<unsigned, T>), dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
                        which, (unsigned)rows, (unsigned)f, (unsigned)fo, gx);
   else
-    hipLaunchKernelGGL(pool_pairs_backward_kernel<i64>, dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
+    hipLaunchKernelGGL((pool_pairs_backward_kernel<i64, T>), dim3((unsigned)blocks), dim3(kPwThreads), 0, stream, gy,
                        which, rows, f, fo, gx);
   return hipGetLastError();
 }
+template hipError_t launch_pool_pairs_backward<float>(const float *, const unsigned char *, i64, i64, float *,
+                                                      hipStream_t);
+template hipError_t launch_pool_pairs_backward<_Float16>(const _Float16 *, const unsigned char *, i64, i64,
+                                                         _Float16 *, hipStream_t);
 
 // ---- half <-> float copies (the half-precision entry points compute in fp32) ------
 namespace {

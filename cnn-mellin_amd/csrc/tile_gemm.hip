@@ -571,6 +571,10 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // workgroups per CU: 32 channels double the workgroups of a small problem (1-D layers
   // of 780 frames: input gradient 75 -> 61 us, forward up to 25 % faster)
   *mt = (pr.c_out > 32 && pr.batch * ((Q + 127) / 128) * ((pr.c_out + 63) / 64) >= 512) ? 2 : 1;
+  // half-precision operands: 128 channels where the layer has them (the f16 instructions are
+  // through with a staged chunk six times sooner, so what a chunk's staging costs is spread
+  // over twice the products; the accumulators fit because nothing is split in registers)
+  if (pr.in_half && pr.c_out > 64 && pr.batch * ((Q + 255) / 256) * ((pr.c_out + 127) / 128) >= 256) *mt = 4;
   const int M_T = *mt * 32;
   const i64 m_tiles = (pr.c_out + M_T - 1) / M_T;
   // two N tiles per wavefront once that still leaves every CU several tiles (not when
@@ -817,14 +821,7 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   const bool memo = (pl.C + pl.CC - 1) / pl.CC > 2;
 #define MELLIN_TILE_CASE(MT_, NT_)                                                           \
   if (mt == MT_ && nt == NT_) {                                                              \
-    if (pl.f16 && pl.out_half) {                                                             \
-      if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, true, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
-      return launch_variant<MT_, NT_, false, 0, true, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
-    }                                                                                        \
-    if (pl.f16) {                                                                            \
-      if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, false, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
-      return launch_variant<MT_, NT_, false, 0, false, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
-    }                                                                                        \
+    if (pl.f16) return hipErrorInvalidValue;                                                 \
     if (pl.split && pl.CC >= pl.C) {                                                         \
       if (pl.accumulate) return launch_variant<MT_, NT_, true, 0, false, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
       if (pl.out_half) return launch_variant<MT_, NT_, false, 0, true, 1>(pl, lds_bytes, grid, f, g, bias, h, stream, af);   \
@@ -844,6 +841,22 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
     return memo ? launch_variant<MT_, NT_, false, 8>(pl, lds_bytes, grid, f, g, bias, h, stream)   \
                 : launch_variant<MT_, NT_, false, 0>(pl, lds_bytes, grid, f, g, bias, h, stream);  \
   }
+#define MELLIN_F16_CASE(MT_, NT_)                                                            \
+  if (pl.f16 && mt == MT_ && nt == NT_) {                                                    \
+    if (pl.out_half) {                                                                       \
+      if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, true, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+      return launch_variant<MT_, NT_, false, 0, true, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+    }                                                                                        \
+    if (pl.CC >= pl.C) return launch_variant<MT_, NT_, false, 0, false, 3>(pl, lds_bytes, grid, f, g, bias, h, stream, af); \
+    return launch_variant<MT_, NT_, false, 0, false, 4>(pl, lds_bytes, grid, f, g, bias, h, stream, af);                   \
+  }
+  MELLIN_F16_CASE(4, 2)
+  MELLIN_F16_CASE(4, 1)
+  MELLIN_F16_CASE(2, 2)
+  MELLIN_F16_CASE(2, 1)
+  MELLIN_F16_CASE(1, 2)
+  MELLIN_F16_CASE(1, 1)
+#undef MELLIN_F16_CASE
   MELLIN_TILE_CASE(2, 2)
   MELLIN_TILE_CASE(2, 1)
   MELLIN_TILE_CASE(1, 2)

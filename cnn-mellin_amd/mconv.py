@@ -231,7 +231,7 @@ class _Corr2dFunction(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         grad_bias = None
         want_bias = ctx.has_bias and ctx.needs_input_grad[2]
-        if grad_out.dtype == torch.float32 and grad_out.shape[0] <= 65535 and grad_out.shape[1] <= 65535 and \
+        if grad_out.dtype in (torch.float32, torch.float16) and grad_out.shape[0] <= 65535 and grad_out.shape[1] <= 65535 and \
                 (out is not None or want_bias):
             # one pass: the backward of the fused ReLU (pass where out > 0) and the bias gradient
             grad_out, grad_bias = _hip.bias_grad(grad_out, out)

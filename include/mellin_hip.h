@@ -212,10 +212,29 @@ int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input,
 /* Half precision (the data type the reference's Autocast registration casts to,
  * ext/torch.cpp:407-430, before it calls the CUDA kernels instantiated for
  * c10::Half, ext/torch_cuda.cu:45-177): tensors hold IEEE binary16 values in
- * the layouts above; all arithmetic is fp32 (operands are widened, products are
- * accumulated in fp32, the result is rounded to half once).  Every pass needs
- * scratch memory: the byte count comes from the matching *_workspace() call
- * (it includes what the fp32 pass underneath needs; 256-byte aligned buffer). */
+ * the layouts above.  Products of half values are exact in fp32 and are summed in
+ * fp32; the result is rounded to half once (subnormal operands are not flushed).
+ *
+ * The kernels read the half tensors as they lie and multiply on the f16 matrix
+ * cores (v_mfma_f32_32x32x16_f16), one sixth of the matrix work of the fp32 path
+ * on half the bytes: the forward pass and the input gradient through the tiled
+ * kernel (variant "mfma-f16"; the input gradient of layers with few input
+ * channels, or on a Mellin axis that keeps fewer rows than it is given, as two
+ * passes, "mfma-f16+fold", whose intermediate rows and folded result are fp32),
+ * the weight gradient through a kernel of its own whose matrix instructions run
+ * along the output positions ("mfma-f16"; partial sums in fp32, added in a fixed
+ * order).  Scratch memory then holds what those kernels need (the filter cut into
+ * matrix fragments for layers staged in chunks of channels, first-pass rows,
+ * partial sums) -- often nothing for the forward pass.  Where no such kernel
+ * applies (outputs wider than 128 columns in the weight gradient, sizes beyond
+ * the kernels' 32-bit limits, the "generic" and "widen" variants) the operands are
+ * copied to fp32 in the scratch memory, the fp32 kernels run there and the result
+ * is rounded to half: the same arithmetic in another order of summation, so the
+ * two routes agree to the last half bit except where an fp32 sum lies within
+ * its own rounding error of a boundary between two half values.
+ * The byte count of the scratch memory comes from the matching *_workspace() call
+ * (256-byte aligned buffer; query and call under the same variant); too little is
+ * MELLIN_ERR_WORKSPACE. */
 size_t mellin_corr2d_forward_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS);
 int mellin_corr2d_forward_f16(int kind_x, const void *input, const void *weight,
                               const void *bias, MELLIN_CORR2D_DIMS, void *out,
@@ -349,6 +368,12 @@ int mellin_bias_grad_f32(const float *grad_out, const float *out, int64_t batch,
                          int64_t channels, int64_t plane, float *grad_masked,
                          float *grad_bias, void *workspace, size_t workspace_bytes,
                          void *stream);
+/* The same on half-precision tensors (grad_out, out, grad_masked, grad_bias): sums in fp32,
+ * grad_bias rounded to half once; same scratch. */
+int mellin_bias_grad_f16(const void *grad_out, const void *out, int64_t batch,
+                         int64_t channels, int64_t plane, void *grad_masked,
+                         void *grad_bias, void *workspace, size_t workspace_bytes,
+                         void *stream);
 
 /* Frequency pooling of the convolution stack (BASELINE config 5): the maximum over pairs of
  * neighbours along the last axis, y[r, j] = max(x[r, 2 j], x[r, 2 j + 1]) for x (rows, f) and
@@ -359,6 +384,11 @@ int mellin_pool_pairs_forward_f32(const float *x, int64_t rows, int64_t f, float
                                   unsigned char *which, void *stream);
 int mellin_pool_pairs_backward_f32(const float *grad_y, const unsigned char *which,
                                    int64_t rows, int64_t f, float *grad_x, void *stream);
+/* The same on half-precision tensors. */
+int mellin_pool_pairs_forward_f16(const void *x, int64_t rows, int64_t f, void *y,
+                                  unsigned char *which, void *stream);
+int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *which,
+                                   int64_t rows, int64_t f, void *grad_x, void *stream);
 
 /* Name of the kernel variant the most recent operator-level call of the
  * process (on any thread: PyTorch runs backward passes on a thread of its own)
@@ -366,7 +396,8 @@ int mellin_pool_pairs_backward_f32(const float *grad_y, const unsigned char *whi
  * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
- * (two-pass input gradient). */
+ * (two-pass input gradient), "mfma-f16" and "mfma-f16+fold" (half-precision
+ * tensors on the f16 matrix cores). */
 const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).
@@ -395,7 +426,9 @@ int mellin_last_math(void);
 /* Force a variant for subsequent operator-level calls of the process (all threads):
  * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
  * kernels; "two-pass" = automatic choice without the specialised gradient
- * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows"), i.e. the tiled ones.
+ * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows"), i.e. the tiled ones;
+ * "widen" = automatic choice, but the half-precision entry points always go
+ * through fp32 copies of their operands (for comparisons).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);
 
