@@ -90,8 +90,10 @@ hipError_t launch_wgrad(const WgradPlan &wp, const float *grad_out, const float 
 hipError_t launch_wgrad_reduce(const float *partials_ws, void *W, bool half_out, int partials, int M, int J,
                                int M_pad, int J_pad, hipStream_t stream);
 
-// Weight gradient of a half-precision layer on the f16 matrix cores (wgrad_f16.hip).
-struct WgradHalfPlan {
+// Weight gradient with the matrix instructions along the output positions (wgrad_pos.hip):
+// half-precision layers on the f16 matrix cores, fp32 layers on the bf16 ones (three-part operands).
+struct WgradPosPlan {
+  int half;                        // grad_out, input and grad_weight are half-precision storage (else float)
   TilePlan t;                      // staging geometry of the forward problem
   i64 a_n, a_m;                    // grad_out strides: image, channel (positions are dense)
   int J, jt;                       // c_in * nfx * nfy; 32-column tiles per wavefront
@@ -104,10 +106,10 @@ struct WgradHalfPlan {
 };
 
 // false: the kernel does not apply (outputs wider than 128 columns, sizes beyond its limits)
-bool make_wgrad_half_plan(const SepConv &fwd, WgradHalfPlan &wp);
+bool make_wgrad_pos_plan(const SepConv &fwd, WgradPosPlan &wp, bool half);
 
-// grad_out, input and grad_weight are half-precision storage; workspace: wp.ws_bytes
-hipError_t launch_wgrad_half(const WgradHalfPlan &wp, const void *grad_out, const void *input,
-                             void *grad_weight, float *workspace, hipStream_t stream);
+// workspace: wp.ws_bytes
+hipError_t launch_wgrad_pos(const WgradPosPlan &wp, const void *grad_out, const void *input,
+                            void *grad_weight, float *workspace, hipStream_t stream);
 
 }  // namespace mellin

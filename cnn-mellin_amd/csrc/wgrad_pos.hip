@@ -1,22 +1,25 @@
-// Weight gradient of half-precision layers on the f16 matrix cores.
+// Weight gradient with the matrix instructions running along the output positions: for
+// half-precision layers on the f16 matrix cores, for fp32 layers on the bf16 ones.
 //
 //   W[m, (c, fx, fy)] = sum_{n, ox, oy} A[n, m, ox, oy] *
 //                       G[n, c, tap_x(ox, fx), tap_y(oy, fy)]
 //
-// A = grad_out and G = the layer's input are half-precision tensors, read as they lie.
-// Products of half values are exact in fp32 and v_mfma_f32_32x32x16_f16 sums them in fp32,
-// so the arithmetic is that of the fp32 kernels on the widened operands, in another order.
+// A = grad_out and G = the layer's input are read as they lie.  Half precision: products of
+// half values are exact in fp32 and v_mfma_f32_32x32x16_f16 sums them in fp32, so the
+// arithmetic is that of the fp32 kernels on the widened operands, in another order.  fp32:
+// both operands are split into three bf16 parts in registers and a product is six bf16
+// matrix instructions (tile_stage.hpp).
 //
 // The product is (M x positions) * (positions x J), J = c_in * nfx * nfy, and the k index of
 // a matrix instruction runs over sixteen CONSECUTIVE output positions of one image (rows
 // flattened), eight per half-wave:
-//   * grad_out: the eight positions of a lane's channel are sixteen consecutive bytes of
-//     global memory (any 2-byte alignment) and are the instruction's operand as they are:
-//     one 16-byte load per lane, a few steps ahead, no LDS;
+//   * grad_out: the eight positions of a lane's channel are consecutive in global memory
+//     (any element alignment): one or two 16-byte loads per lane straight into registers, a
+//     few steps ahead, no LDS -- for half precision the instruction's operand as it is;
 //   * input: the rows a unit of work touches are staged as in the forward kernel (direct
-//     global->LDS loads into affine virtual rows, one half value per LDS word), and the
-//     operand of lane (column j) for position q is the 16-bit word at
-//     col_offset[j] + pos_offset[q]; pos_offset is a table in LDS, the same for every unit.
+//     global->LDS loads into affine virtual rows, one value per LDS word), and the operand
+//     of lane (column j) for position q is the word at col_offset[j] + pos_offset[q];
+//     pos_offset is a table in LDS, the same for every unit.
 // A unit is RB output rows of one image.  A workgroup owns 64 * mbw output channels and
 // JT * 32 columns for its whole life and walks a contiguous range of units (image running
 // fastest, so that consecutive units stage the same rows of successive images); its four
@@ -24,6 +27,7 @@
 // steps.  Every wavefront writes its accumulators as one partial block; wgrad_reduce adds
 // the partial blocks in index order (no floating-point atomics: bit-reproducible).
 #include <algorithm>
+#include <type_traits>
 
 #include "mellin_common.hpp"
 #include "tile_gemm.hpp"
@@ -34,14 +38,20 @@ namespace mellin {
 namespace {
 
 constexpr int kF16Memo = 8;                        // 64-word blocks per wave whose staging sources are kept
-constexpr int kAhead = 4;                          // steps whose grad_out operands are in flight
 
-struct __attribute__((packed, aligned(2))) Half8 { uintx4 v; };
+struct __attribute__((packed, aligned(2))) Bytes16At2 { uintx4 v; };
+struct __attribute__((packed, aligned(4))) Bytes16At4 { uintx4 v; };
 
-template <int JT>
-__global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
-    WgradHalfPlan wp, const _Float16 *__restrict__ A, const _Float16 *__restrict__ G,
+// F16: A and G are half-precision storage (else float)
+template <int JT, bool F16>
+__global__ __launch_bounds__(kThreads, 2) void wgrad_pos_kernel(
+    WgradPosPlan wp, const void *__restrict__ Av, const void *__restrict__ G,
     float *__restrict__ ws) {
+  typedef typename std::conditional<F16, _Float16, float>::type T;
+  constexpr int EB = sizeof(T);
+  constexpr int kAhead = F16 ? 4 : 2;                // steps whose grad_out operands are in flight
+  constexpr int kRaw = F16 ? 1 : 2;                  // 16-byte words of eight values
+  const T *A = (const T *)Av;
   extern __shared__ __align__(16) float lds[];
   const TilePlan &pl = wp.t;
   constexpr int MT = 2;
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
     const int run = min(tg.n, ui);
     unsigned zero;                                     // a zero the compiler cannot see through (see tile_gemm.hip)
     asm volatile("s_mov_b32 %0, 0" : "=s"(zero));
-    issue_signal<kWaves, kF16Memo, 2>(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words),
+    issue_signal<kWaves, kF16Memo, EB>(pl, tg, G, c_lo, ccj, Xs0 + b * x_words, lds_base + 4u * (unsigned)(b * x_words),
                                       mellin_x, lane, wave + (int)zero, &memo, run == 0, run < 2);
   };
 
@@ -133,42 +143,80 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
 #pragma unroll
   for (int i = 0; i < MT; ++i) m_off[i] = min(m0 + i * 32 + l32, pl.M - 1) * (int)wp.a_m + 8 * half;
 
-  // the operands of one step: words of eight half values
-  auto load_a = [&](const _Float16 *An, int s, uintx4 (&a)[MT]) {      // whole steps only
+  // grad_out of one step as loaded: the lane's eight values per channel tile
+  struct RawA { uintx4 v[MT][kRaw]; };
+  auto load_a = [&](const T *An, int s, RawA &a) {           // whole steps only
 #pragma unroll
-    for (int i = 0; i < MT; ++i) a[i] = ((const Half8 *)(An + m_off[i] + 16 * s))->v;
+    for (int i = 0; i < MT; ++i) {
+      const T *p = An + m_off[i] + 16 * s;
+      if constexpr (F16) {
+        a.v[i][0] = ((const Bytes16At2 *)p)->v;
+      } else {
+        a.v[i][0] = ((const Bytes16At4 *)p)->v;
+        a.v[i][1] = ((const Bytes16At4 *)(p + 4))->v;
+      }
+    }
   };
-  auto fetch_b = [&](const float *Xs, int s, uintx4 (&b)[JT]) {
+  // one step: the input words of the lane's columns at the step's sixteen positions times
+  // grad_out; `left` < 8: only that many of this half-wave's positions exist (both operands
+  // are cleared past them)
+  auto multiply_step = [&](const float *Xs, int s, const RawA &a, int left) {
     const int4 o0 = *(const int4 *)(pos_off + 16 * s + 8 * half), o1 = *(const int4 *)(pos_off + 16 * s + 8 * half + 4);
     const int off[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+    if constexpr (F16) {
+      unsigned keep[4];
 #pragma unroll
-    for (int t = 0; t < JT; ++t)
+      for (int w = 0; w < 4; ++w) keep[w] = (2 * w < left ? 0xFFFFu : 0u) | (2 * w + 1 < left ? 0xFFFF0000u : 0u);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        ushortx2 pair;
-        pair.x = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i]));
-        pair.y = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i + 1]));
-        b[t][i] = __builtin_bit_cast(unsigned, pair);
+      for (int t = 0; t < JT; ++t) {
+        uintx4 b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ushortx2 pair;
+          pair.x = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i]));
+          pair.y = *(const unsigned short *)((const char *)Xs + (col_off[t] + off[2 * i + 1]));
+          b[i] = __builtin_bit_cast(unsigned, pair);
+          if (left < 8) b[i] &= keep[i];
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+          acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a.v[i][0]),
+                                                             __builtin_bit_cast(halfx8, b), acc[i][t], 0, 0, 0);
       }
-  };
-  auto multiply = [&](const uintx4 (&a)[MT], const uintx4 (&b)[JT]) {
+    } else {
+      uintx4 ah[MT], am[MT], al[MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+      for (int i = 0; i < MT; ++i) {
+        float x[8];
 #pragma unroll
-      for (int t = 0; t < JT; ++t)
-        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a[i]),
-                                                           __builtin_bit_cast(halfx8, b[t]), acc[i][t], 0, 0, 0);
+        for (int k = 0; k < 8; ++k) x[k] = __uint_as_float(a.v[i][k >> 2][k & 3]);
+        split8(x, ah[i], am[i], al[i]);
+      }
+#pragma unroll
+      for (int t = 0; t < JT; ++t) {
+        float x[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          x[k] = *(const float *)((const char *)Xs + (col_off[t] + off[k]));
+          if (left < 8 && k >= left) x[k] = 0.f;
+        }
+        uintx4 bh, bm, bl;
+        split8(x, bh, bm, bl);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) mfma_split6(acc[i][t], ah[i], am[i], al[i], bh, bm, bl);
+      }
+    }
   };
 
   __syncthreads();                                     // pos_off
   if (my_units > 0) issue_stage(0);
   for (int ui = 0; ui < my_units; ++ui) {
     const TileGeom tg = unit_geometry(first_unit + ui);
-    const _Float16 *An = A + (i64)tg.n * wp.a_n + tg.q0;
+    const T *An = A + (i64)tg.n * wp.a_n + tg.q0;
     const int whole = tg.count >> 4;                   // steps of sixteen positions that exist
     // this wavefront's steps ps, ps + PS, ...: the first few operands are requested before
     // the wait for the staged rows
-    uintx4 ring[kAhead][MT];
+    RawA ring[kAhead];
 #pragma unroll
     for (int d = 0; d < kAhead; ++d)
       if (ps + d * PS < whole) load_a(An, ps + d * PS, ring[d]);
@@ -185,9 +233,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
       for (int d = 0; d < kAhead; ++d) {
         const int s = s0 + d * PS;
         if (s < whole) {
-          uintx4 b[JT];
-          fetch_b(Xs, s, b);
-          multiply(ring[d], b);
+          multiply_step(Xs, s, ring[d], 8);
           if (s + kAhead * PS < whole) load_a(An, s + kAhead * PS, ring[d]);
         }
       }
@@ -195,27 +241,23 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
     // the last, partial step (by the wavefront whose turn it is): positions past the unit's
     // end belong to the next unit or to nothing, so both operands are cleared there
     if ((tg.count & 15) && whole % PS == ps) {
-      const int left = tg.count - 16 * whole - 8 * half;     // of this half-wave's eight positions
-      uintx4 a[MT], b[JT];
-      unsigned keep[4];
-#pragma unroll
-      for (int w = 0; w < 4; ++w) keep[w] = (2 * w < left ? 0xFFFFu : 0u) | (2 * w + 1 < left ? 0xFFFF0000u : 0u);
+      const int left = min(8, max(0, tg.count - 16 * whole - 8 * half));     // of this half-wave's eight positions
+      RawA a;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        const unsigned short *src = (const unsigned short *)(An + m_off[i] + 16 * whole);
+        const T *src = An + m_off[i] + 16 * whole;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const unsigned lo = 2 * w < left ? src[2 * w] : 0u;
-          const unsigned hi = 2 * w + 1 < left ? src[2 * w + 1] : 0u;
-          a[i][w] = lo | (hi << 16);
+        for (int k = 0; k < 8; ++k) {
+          if constexpr (F16) {
+            const unsigned v = k < left ? (unsigned)((const unsigned short *)src)[k] : 0u;
+            if (k & 1) a.v[i][0][k >> 1] |= v << 16;
+            else a.v[i][0][k >> 1] = v;
+          } else {
+            a.v[i][k >> 2][k & 3] = k < left ? __float_as_uint(src[k]) : 0u;
+          }
         }
       }
-      fetch_b(Xs, whole, b);
-#pragma unroll
-      for (int t = 0; t < JT; ++t)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) b[t][w] &= keep[w];
-      multiply(a, b);
+      multiply_step(Xs, whole, a, left);
     }
   }
 
@@ -232,10 +274,10 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f16_kernel(
       }
 }
 
-template <int JT>
-hipError_t launch_f16(const WgradHalfPlan &wp, dim3 grid, const void *a, const void *g, float *ws,
+template <int JT, bool F16>
+hipError_t launch_pos(const WgradPosPlan &wp, dim3 grid, const void *a, const void *g, float *ws,
                       hipStream_t stream) {
-  auto kern = wgrad_f16_kernel<JT>;
+  auto kern = wgrad_pos_kernel<JT, F16>;
   if (wp.lds_bytes > 64 * 1024) {
     static thread_local size_t granted = 0;
     if (granted < wp.lds_bytes) {
@@ -245,14 +287,14 @@ hipError_t launch_f16(const WgradHalfPlan &wp, dim3 grid, const void *a, const v
       granted = wp.lds_bytes;
     }
   }
-  hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, (const _Float16 *)a,
-                     (const _Float16 *)g, ws);
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
   return hipGetLastError();
 }
 
 }  // namespace
 
-bool make_wgrad_half_plan(const SepConv &fwd_in, WgradHalfPlan &wp) {
+bool make_wgrad_pos_plan(const SepConv &fwd_in, WgradPosPlan &wp, bool half) {
+  wp.half = half;
   // (the forward tiling is only borrowed for its staging geometry: plan it for the fp32 kernel)
   SepConv fwd = fwd_in;
   fwd.math = MATH_FP32;
@@ -270,7 +312,8 @@ bool make_wgrad_half_plan(const SepConv &fwd_in, WgradHalfPlan &wp) {
   pl.contig = 0;
   pl.RS = (pl.ay * (pl.noy - 1) + pl.by_span + 1) | 1;
   wp.J = pl.C * pl.nf;
-  wp.jt = wp.J > 96 ? 4 : (wp.J + 31) / 32;
+  // (fp32: three-part operands take the registers of a fourth column tile)
+  wp.jt = std::min(half ? 4 : 3, (wp.J + 31) / 32);
   wp.mbw = pl.M > 128 ? 4 : (pl.M > 64 ? 2 : 1);
   const int M_T = 64 * wp.mbw, J_T = wp.jt * 32;
   wp.m_groups = (pl.M + M_T - 1) / M_T;
@@ -303,16 +346,22 @@ bool make_wgrad_half_plan(const SepConv &fwd_in, WgradHalfPlan &wp) {
   return true;
 }
 
-hipError_t launch_wgrad_half(const WgradHalfPlan &wp, const void *grad_out, const void *input,
-                             void *grad_weight, float *workspace, hipStream_t stream) {
+hipError_t launch_wgrad_pos(const WgradPosPlan &wp, const void *grad_out, const void *input,
+                            void *grad_weight, float *workspace, hipStream_t stream) {
   dim3 grid((unsigned)wp.S, (unsigned)(wp.m_groups * wp.j_groups));
   hipError_t e = hipErrorInvalidValue;
-  if (wp.jt == 1) e = launch_f16<1>(wp, grid, grad_out, input, workspace, stream);
-  if (wp.jt == 2) e = launch_f16<2>(wp, grid, grad_out, input, workspace, stream);
-  if (wp.jt == 3) e = launch_f16<3>(wp, grid, grad_out, input, workspace, stream);
-  if (wp.jt == 4) e = launch_f16<4>(wp, grid, grad_out, input, workspace, stream);
+  if (wp.half) {
+    if (wp.jt == 1) e = launch_pos<1, true>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 2) e = launch_pos<2, true>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 3) e = launch_pos<3, true>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 4) e = launch_pos<4, true>(wp, grid, grad_out, input, workspace, stream);
+  } else {
+    if (wp.jt == 1) e = launch_pos<1, false>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 2) e = launch_pos<2, false>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 3) e = launch_pos<3, false>(wp, grid, grad_out, input, workspace, stream);
+  }
   if (e != hipSuccess) return e;
-  return launch_wgrad_reduce(workspace, grad_weight, /*half_out=*/true, wp.S * (kWaves / wp.mbw), wp.t.M, wp.J,
+  return launch_wgrad_reduce(workspace, grad_weight, wp.half, wp.S * (kWaves / wp.mbw), wp.t.M, wp.J,
                              wp.M_pad, wp.J_pad, stream);
 }
 

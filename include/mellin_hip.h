@@ -393,7 +393,9 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
 /* Name of the kernel variant the most recent operator-level call of the
  * process (on any thread: PyTorch runs backward passes on a thread of its own)
  * dispatched to (for tests and profiling): "generic", "mfma" (tiled
- * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-fused"
+ * matrix-core kernels), "mfma-rows" (row-wise weight gradient), "mfma-positions"
+ * (weight gradient of layers with many channels: matrix instructions along the
+ * output positions, bf16 matrix cores), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
  * (two-pass input gradient), "mfma-f16" and "mfma-f16+fold" (half-precision
@@ -426,7 +428,8 @@ int mellin_last_math(void);
 /* Force a variant for subsequent operator-level calls of the process (all threads):
  * NULL, "" or "auto" = automatic choice; "generic" = the one-thread-per-output
  * kernels; "two-pass" = automatic choice without the specialised gradient
- * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows"), i.e. the tiled ones;
+ * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows", "mfma-positions"), i.e. the
+ * tiled ones;
  * "widen" = automatic choice, but the half-precision entry points always go
  * through fp32 copies of their operands (for comparisons).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */

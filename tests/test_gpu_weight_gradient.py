@@ -1,5 +1,6 @@
-"""Weight gradient: the row-wise matrix-core kernel and the tiled one must both
-agree with the CPU checker through the C ABI.
+"""Weight gradient: the row-wise matrix-core kernel, the tiled one and the one whose matrix
+instructions run along the output positions (wide layers) must all agree with the CPU
+checker through the C ABI.
 
 Tolerance: rtol 1e-5 / atol 1e-5 * sqrt(fan_in) against the float64 checker
 (fan_in = terms per output = batch * output positions).
@@ -73,3 +74,52 @@ def test_rows_is_run_to_run_deterministic():
     for _ in range(3):
         again, _ = _grad_weight(hip.AX_LCORR, x, go, (64, 3, 8, 4), (1, 1), (1, 1), (0, 0), (1, 1), None)
         assert torch.equal(first, again)
+
+
+WIDE_CASES = [
+    # (op, n, c_in, c_out, nf, ng, s, d, p, u, r): at least 16 input and more than 32 output channels
+    ("lcorrlcorr", 2, 16, 64, (3, 3), (20, 19), (1, 1), (2, 1), (2, 1), (1, 1), (0, 0)),   # dilation and padding
+    ("mcorrlcorr", 3, 20, 40, (4, 2), (30, 9), (2, 1), (1, 1), (1, 0), (2, 1), (0, 0)),    # Mellin with s, p, u; 40 of 64 channel rows used
+    ("lcorrlcorr", 5, 16, 200, (2, 2), (9, 5), (1, 1), (1, 1), (0, 0), (1, 1), (0, 0)),    # four channel blocks side by side; rows of four outputs
+    ("mcorrlcorr", 2, 41, 128, (8, 1), (100, 1), (1, 1), (1, 1), (3, 0), (1, 1), (0, 0)),  # 1-D
+    ("lcorrlcorr", 2, 16, 33, (2, 3), (11, 16), (1, 2), (1, 1), (0, 2), (1, 2), (1, 0)),   # y stride and up-sampling, an extra output row
+    ("lcorrlcorr", 1, 17, 70, (3, 3), (7, 6), (1, 1), (1, 1), (1, 1), (1, 1), (0, 0)),     # one image, 42 positions: a partial step only per unit
+]
+
+
+@pytest.mark.parametrize("case", WIDE_CASES, ids=[str(i) for i in range(len(WIDE_CASES))])
+def test_positions_kernel_matches_checker(case):
+    op, n, c_in, c_out, nf, ng, s, d, p, u, r = case
+    kind_x, fwd, bwd = OPS[op]
+    rng = np.random.default_rng(2000 + WIDE_CASES.index(case))
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float32)
+    w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+    nh = fwd(x, w, None, s, d, p, u, r).shape[2:]
+    assert min(nh) > 0
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    _, exp, _ = bwd(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64), s, d, p, u)
+    fan_in = n * nh[0] * nh[1]
+    got, v1 = _grad_weight(kind_x, x, go, w.shape, s, d, p, u, None)
+    assert v1 == "mfma-positions" and hip.last_math() == hip.MATH_BF16X3, v1
+    assert_close(got, exp, fan_in, "positions %s" % (case,))
+    again, _ = _grad_weight(kind_x, x, go, w.shape, s, d, p, u, None)
+    assert torch.equal(got, again)                        # fixed order of summation
+    other, v2 = _grad_weight(kind_x, x, go, w.shape, s, d, p, u, "two-pass")
+    assert v2 == "mfma", v2
+    assert_close(other, exp, fan_in, "tiles %s" % (case,))
+    # no less accurate than the fp32 instructions beyond the order of summation
+    err = lambda t: float(np.sqrt(np.mean((t.cpu().numpy().astype(np.float64) - exp) ** 2)))
+    assert err(got) <= 3.0 * err(other) + 1e-12, (err(got), err(other))
+
+
+def test_positions_kernel_needs_the_bf16_math_mode():
+    """Under MELLIN_MATH_FP32 wide layers keep the fp32 kernels."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 16, 20, 19)).astype(np.float32)
+    go = rng.standard_normal((2, 64, 18, 17)).astype(np.float32)
+    hip.set_math(hip.MATH_FP32)
+    try:
+        _, v = _grad_weight(hip.AX_LCORR, x, go, (64, 16, 3, 3), (1, 1), (1, 1), (0, 0), (1, 1), None)
+        assert v != "mfma-positions" and hip.last_math() == hip.MATH_FP32
+    finally:
+        hip.set_math(hip.MATH_BF16X3)
