@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
 """Per-pass timings on one MI355X of the layer shapes beside the benchmark's own.
 
+    python time_layers.py cfg3            # the benchmark's own layer, linear and Mellin x axis
     python time_layers.py cfg4            # wide 2-D layer, linear and Mellin x axis
     python time_layers.py cfg2            # 1-D layers over the (s, d, p) grid
     python time_layers.py stack           # the 10-layer 3 -> 256 stacks, layer by layer
@@ -71,6 +72,19 @@ def time_layer(tag, kind_x, x, w, b, s, d, p, r, reps, activation=None):
                      "math": {hip.MATH_BF16X3: "bf16x3", hip.MATH_F16: "f16"}.get(hip.last_math(), "fp32"),
                      "tflops": round(2 * macs / us / 1e6, 1)}
     return rec, out
+
+
+def run_cfg3(reps, dtype):
+    import torch
+    import _mellin_hip as hip
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(32, 3, 512, 41, device="cuda", generator=gen).to(dtype)
+    bound = (3 * 32) ** -0.5
+    w = ((torch.rand(64, 3, 8, 4, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
+    b = ((torch.rand(64, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
+    for kind, name in ((hip.AX_LCORR, "lconv2d"), (hip.AX_MCORR, "mconv2d")):
+        rec, _ = time_layer("cfg3 " + name, kind, x, w, b, (1, 1), (1, 1), (0, 0), (0, 0), reps)
+        print(json.dumps(rec), flush=True)
 
 
 def run_cfg4(reps, dtype):
@@ -146,7 +160,7 @@ def run_stack(reps, dtype):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("config", choices=["cfg2", "cfg4", "stack"])
+    ap.add_argument("config", choices=["cfg2", "cfg3", "cfg4", "stack"])
     ap.add_argument("--reps", type=int, default=10, help="timed calls per pass")
     ap.add_argument("--math", choices=["bf16x3", "fp32"], default="bf16x3",
                     help="how the matrix kernels form fp32 products (library default: bf16x3)")
@@ -160,7 +174,7 @@ def main():
     import _mellin_hip as hip
     hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
     dtype = torch.float16 if args.dtype == "half" else torch.float32
-    {"cfg2": run_cfg2, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps, dtype)
+    {"cfg2": run_cfg2, "cfg3": run_cfg3, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps, dtype)
 
 
 if __name__ == "__main__":
