@@ -685,6 +685,16 @@ bool plan_half_two_pass(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64
          tp.ws_bytes + (size_t)(batch * c_in * ngx * ngy) * 4 <= kMaxWorkspaceBytes;
 }
 
+// The one-kernel input gradient of layers with at most three input channels and a linear x
+// axis on half-precision tensors, if the variant in force allows it and the form applies.
+bool plan_half_fused(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx, i64 ngy, i64 nhx,
+                     i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px, i64 py, i64 ux, i64 uy, IgradPlan &ip) {
+  if (g_forced != 0 || g_widen || c_out * nfx * nfy * nhx * nhy == 0) return false;
+  return make_igrad_plan(kind_x, batch, c_in, c_out, nfx, nfy, ngx, ngy, nhx, nhy, sx, sy, dx, dy, px, py, ux, uy,
+                         ip, 0, 0, -1, MATH_BF16X3) &&
+         ip.stream && ip.ws_bytes <= kMaxWorkspaceBytes;
+}
+
 // Input gradients of layers with fewer input channels than this leave most of a 32-row
 // matrix tile empty in the gather form: they keep the fp32 kernels made for them.
 constexpr i64 kHalfGatherMinChannels = 16;
@@ -822,6 +832,8 @@ size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS
   if (check_corr2d(__func__, kind_x, CORR2D_ARGS)) return 0;
   CORR2D_COUNTS;
   HalfNative hn;
+  IgradPlan ip;
+  if (plan_half_fused(kind_x, CORR2D_ARGS, ip)) return ip.ws_bytes;
   // (the two-pass form where the fp32 path would take it: few input channels, or a Mellin
   // axis that keeps fewer rows than it is given)
   TwoPassInput tp;
@@ -837,6 +849,17 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
   CORR2D_COUNTS;
   if (n_in == 0) return MELLIN_OK;
   {
+    IgradPlan ip;
+    if (plan_half_fused(kind_x, CORR2D_ARGS, ip)) {
+      if (ip.ws_bytes && (!workspace || workspace_bytes < ip.ws_bytes))
+        return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, ip.ws_bytes,
+                    workspace_bytes);
+      if (!grad_input || !weight || !grad_out) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
+      g_variant = "mfma-f16-fused";
+      g_last_math = MELLIN_MATH_F16;
+      return check_hip(launch_igrad_half(ip, weight, grad_out, grad_input, (float *)workspace, (hipStream_t)stream),
+                       __func__);
+    }
     HalfNative hn;
     TwoPassInput tp;
     const bool two_pass = plan_half_two_pass(kind_x, CORR2D_ARGS, tp);

@@ -403,14 +403,15 @@ __global__ __launch_bounds__((KSTEPS * NT <= 128 ? 768 : 512)) void igrad_kernel
 
 // grad_input rows next to a strip boundary: upper strip's partial + lower strip's.
 // One workgroup per (boundary, image * c_in + channel) sums that boundary's rows.
+template <typename O>                                  // O: float, or _Float16 (the sum rounded once)
 __global__ __launch_bounds__(256) void igrad_combine_kernel(const IgradPlan pl,
                                                             const float *__restrict__ WS,
-                                                            float *__restrict__ GI) {
+                                                            O *__restrict__ GI) {
   const int b = blockIdx.x + 1;                        // boundary between strips b - 1 and b
   const i64 nc = blockIdx.y;
   const int g_b = pl.sx * b * pl.Th - pl.px;           // first row the boundary can share
   const float *src = WS + ((nc * (pl.strips - 1) + (b - 1)) * pl.nshared * 2) * pl.ngy;
-  float *out = GI + nc * pl.ngx * pl.ngy;
+  O *out = GI + nc * pl.ngx * pl.ngy;
   const StripMap map(pl);
   const FastDiv by_ngy(pl.ngy);
   for (int i = threadIdx.x; i < pl.nshared * pl.ngy; i += blockDim.x) {
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(256) void igrad_combine_kernel(const IgradPlan pl,
     map.feeding(gx, s_lo, s_hi);
     if (s_lo == s_hi) continue;                        // not shared after clamping: written directly
     const float *p = src + (i64)r * 2 * pl.ngy + gy;
-    out[(i64)gx * pl.ngy + gy] = p[0] + p[pl.ngy];
+    out[(i64)gx * pl.ngy + gy] = (O)(p[0] + p[pl.ngy]);
   }
 }
 
@@ -440,7 +441,7 @@ hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go,
                      pl.lds_bytes, stream, pl, w, go, gi, ws);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || pl.ws_bytes == 0) return e;
-  hipLaunchKernelGGL(igrad_combine_kernel,
+  hipLaunchKernelGGL(igrad_combine_kernel<float>,
                      dim3((unsigned)(pl.strips - 1), (unsigned)(pl.batch * pl.c_in)), dim3(256), 0,
                      stream, pl, ws, gi);
   return hipGetLastError();
@@ -460,10 +461,17 @@ hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go,
 //   * a wavefront folds its products into a private LDS image of the grad_input rows its
 //     positions reach (no other wavefront touches it); at the end the four images are added
 //     up in wave order into the strip's image, which is written out exactly as above.
-template <int MTT, int NT>
-__global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl, const float *__restrict__ W,
-                                                              const float *__restrict__ GO,
-                                                              float *__restrict__ GI, float *__restrict__ WS) {
+// F16: weight, grad_out and grad_input are half-precision storage and the products run on
+// the f16 matrix cores (exact products, fp32 sums: one instruction where the bf16 form
+// needs six, nothing to split); the images, and the partial rows in the workspace, stay
+// fp32, and a result is rounded to half once.
+template <int MTT, int NT, bool F16 = false>
+__global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl, const void *__restrict__ Wv,
+                                                              const void *__restrict__ GOv,
+                                                              void *__restrict__ GIv, float *__restrict__ WS) {
+  typedef typename std::conditional<F16, _Float16, float>::type T;
+  const T *W = (const T *)Wv, *GO = (const T *)GOv;
+  T *GI = (T *)GIv;
   extern __shared__ __align__(16) float lds[];
   constexpr int P = NT * 32, ROWS = MTT * 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -495,7 +503,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     const FastDiv by_rows(ROWS);
     for (int idx0 = tid; idx0 < kgroups * ROWS; idx0 += 4 * 256) {
       // four tasks at a time: all their loads are requested before the first is split
-      float x[4][8];
+      T x[4][8];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int idx = idx0 + u * 256;
@@ -506,7 +514,7 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
         for (int i = 0; i < 8; ++i) {
           const int k = 8 * g + i;
           x[u][i] = (idx < kgroups * ROWS && k < pl.c_out && ci < pl.c_in && m < pl.nf)
-                        ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : 0.f;
+                        ? W[((i64)k * pl.c_in + ci) * pl.nf + m] : (T)0;
         }
       }
 #pragma unroll
@@ -514,7 +522,18 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
         const int idx = idx0 + u * 256;
         int g, row;
         by_rows.divmod(idx, g, row);
-        if (idx < kgroups * ROWS) store_frag(Af, kgroups, ROWS, g, row, x[u]);
+        if (idx < kgroups * ROWS) {
+          if constexpr (F16) {
+            uintx4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              v[i] = (unsigned)__builtin_bit_cast(unsigned short, x[u][2 * i]) |
+                     ((unsigned)__builtin_bit_cast(unsigned short, x[u][2 * i + 1]) << 16);
+            Af[g * ROWS + row] = v;                        // one part: the eight values themselves
+          } else {
+            store_frag(Af, kgroups, ROWS, g, row, x[u]);
+          }
+        }
       }
     }
   }
@@ -535,28 +554,33 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   const int q0 = r0 * pl.nhy, q1 = r1 * pl.nhy;
   const int n_it = (q1 - q0 + P - 1) / P;
   const int total = n_it * ksteps;
-  const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
+  const T *GOn = GO + (i64)n * pl.c_out * pl.nh;
   const FastDiv by_nhy(pl.nhy);
 
   // step st = (iteration, 16 output channels): this lane's eight channels of NT positions.
   // Addresses are 32-bit byte offsets from the image's grad_out (the plan keeps c_out * nh
   // * 4 below 2^31): one add per load, no 64-bit arithmetic in the loop.
-  struct BOp { float v[NT][8]; };
+  typedef typename std::conditional<F16, unsigned short, float>::type BWord;
+  struct BOp { BWord v[NT][8]; };
   // Buffer loads: a lane's byte offset within the image's grad_out is fixed for a tile
   // (position, and which eight of a step's channels), the channel's offset is wave-uniform
   // and travels in a scalar register, so a load costs no vector arithmetic; offsets past
   // the image's c_out * nh words (a last step reaching past c_out) read zeros.
   const __amdgpu_buffer_rsrc_t go_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void *)GOn, 0, pl.c_out * pl.nh * 4, 0x00020000);
-  const int nh4 = pl.nh * 4;
+      __builtin_amdgcn_make_buffer_rsrc((void *)GOn, 0, pl.c_out * pl.nh * (int)sizeof(T), 0x00020000);
+  const int nh4 = pl.nh * (int)sizeof(T);                  // bytes from a channel to the next
   auto load_b = [&](int it, int ks, BOp &o) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int q = min(q0 + it * P + t * 32 + l32, q1 - 1);   // past the range: any valid position, never folded
-      const int voff = q * 4 + 8 * half * nh4;
+      const int voff = q * (int)sizeof(T) + 8 * half * nh4;
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        o.v[t][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(go_rsrc, voff, (16 * ks + i) * nh4, 0));
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (F16)
+          o.v[t][i] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(go_rsrc, voff, (16 * ks + i) * nh4, 0);
+        else
+          o.v[t][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(go_rsrc, voff, (16 * ks + i) * nh4, 0));
+      }
     }
   };
   floatx16 acc[MTT][NT];
@@ -566,20 +590,36 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   const bool quad = (pl.nfy & 3) == 0 && pl.dy == 1;
   auto multiply = [&](auto first_tag, int ks, const BOp &o) {
     constexpr bool kFirst = decltype(first_tag)::value;      // an iteration's first step starts the sums from zero
-    uintx4 bh[NT], bm[NT], bl[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const uintx4 *af = Af + (2 * ks + half) * ROWS + l32;
+    if constexpr (F16) {
+      uintx4 b[NT];
 #pragma unroll
-    for (int a = 0; a < MTT; ++a) {
-      const uintx4 ah = af[a * 32], am = af[af_part + a * 32], al = af[2 * af_part + a * 32];
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        if (kFirst) {
-          const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          acc[a][t] = zero16;
+        for (int i = 0; i < 4; ++i) b[t][i] = (unsigned)o.v[t][2 * i] | ((unsigned)o.v[t][2 * i + 1] << 16);
+#pragma unroll
+      for (int a = 0; a < MTT; ++a) {
+        const uintx4 av = af[a * 32];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          if (kFirst) acc[a][t] = zero16;
+          acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, av),
+                                                             __builtin_bit_cast(halfx8, b[t]), acc[a][t], 0, 0, 0);
         }
-        mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
+      }
+    } else {
+      uintx4 bh[NT], bm[NT], bl[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
+#pragma unroll
+      for (int a = 0; a < MTT; ++a) {
+        const uintx4 ah = af[a * 32], am = af[af_part + a * 32], al = af[2 * af_part + a * 32];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          if (kFirst) acc[a][t] = zero16;
+          mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
+        }
       }
     }
   };
@@ -689,7 +729,8 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   __syncthreads();
   {
     const int gi_c = pl.ngx * pl.ngy, ws_c = (pl.strips - 1) * pl.nshared * 2 * pl.ngy;   // words per input channel
-    float *GIn = GI + (i64)n * pl.c_in * gi_c, *WSn = WS + (i64)n * pl.c_in * ws_c;
+    T *GIn = GI + (i64)n * pl.c_in * gi_c;
+    float *WSn = WS + (i64)n * pl.c_in * ws_c;
     // four rows per trip: their table entries first, then all their reads, then the stores,
     // so that the LDS round trips of the four overlap
     for (int cc = 0; cc < pl.c_in; ++cc)
@@ -720,8 +761,8 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
             float v = 0.f;
 #pragma unroll
             for (int k = 0; k < kWaves; ++k) v += (inside && k < nw[u]) ? x[u][k] : 0.f;
-            float *out = (kind[u] > 0 ? WSn + cc * ws_c : GIn + cc * gi_c) + dst[u];
-            if (kind[u] >= 0) out[gy] = v;
+            if (kind[u] > 0) (WSn + cc * ws_c + dst[u])[gy] = v;
+            else if (kind[u] == 0) (GIn + cc * gi_c + dst[u])[gy] = (T)v;
           }
         }
       }
@@ -734,16 +775,16 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
       const i64 per_c = (i64)zrows * pl.ngy;
       for (i64 i = tid; i < pl.c_in * per_c; i += 256) {
         const i64 cc = i / per_c, w = i - cc * per_c;
-        GI[(((i64)n * pl.c_in + cc) * pl.ngx + z0) * pl.ngy + w] = 0.f;
+        GI[(((i64)n * pl.c_in + cc) * pl.ngx + z0) * pl.ngy + w] = (T)0;
       }
     }
   }
 }
 
-template <int MTT, int NT>
-hipError_t launch_stream_instance(const IgradPlan &pl, const float *w, const float *go, float *gi,
+template <int MTT, int NT, bool F16 = false>
+hipError_t launch_stream_instance(const IgradPlan &pl, const void *w, const void *go, void *gi,
                                   float *ws, hipStream_t stream) {
-  auto kern = igrad_stream_kernel<MTT, NT>;
+  auto kern = igrad_stream_kernel<MTT, NT, F16>;
   if (pl.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)pl.lds_bytes);
@@ -753,9 +794,12 @@ hipError_t launch_stream_instance(const IgradPlan &pl, const float *w, const flo
                      ws);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || pl.ws_bytes == 0) return e;
-  hipLaunchKernelGGL(igrad_combine_kernel,
-                     dim3((unsigned)(pl.strips - 1), (unsigned)(pl.batch * pl.c_in)), dim3(256), 0,
-                     stream, pl, ws, gi);
+  const dim3 cgrid((unsigned)(pl.strips - 1), (unsigned)(pl.batch * pl.c_in));
+  if (F16)
+    hipLaunchKernelGGL(igrad_combine_kernel<_Float16>, cgrid, dim3(256), 0, stream, pl, (const float *)ws,
+                       (_Float16 *)gi);
+  else
+    hipLaunchKernelGGL(igrad_combine_kernel<float>, cgrid, dim3(256), 0, stream, pl, (const float *)ws, (float *)gi);
   return hipGetLastError();
 }
 
@@ -1047,6 +1091,14 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
     return true;
   }
   return false;
+}
+
+hipError_t launch_igrad_half(const IgradPlan &pl, const void *weight, const void *grad_out,
+                             void *grad_input, float *workspace, hipStream_t stream) {
+  if (!pl.stream) return hipErrorInvalidValue;
+  if (pl.c_in == 1) return launch_stream_instance<1, 2, true>(pl, weight, grad_out, grad_input, workspace, stream);
+  if (pl.c_in == 2) return launch_stream_instance<2, 1, true>(pl, weight, grad_out, grad_input, workspace, stream);
+  return launch_stream_instance<3, 1, true>(pl, weight, grad_out, grad_input, workspace, stream);
 }
 
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,

@@ -43,6 +43,11 @@ bool make_igrad_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nf
 hipError_t launch_igrad(const IgradPlan &pl, const float *weight, const float *grad_out,
                         float *grad_input, float *workspace, hipStream_t stream);
 
+// The `stream` form of a plan on half-precision tensors (f16 matrix cores; the workspace
+// keeps fp32 partial rows): weight, grad_out and grad_input are half-precision storage.
+hipError_t launch_igrad_half(const IgradPlan &pl, const void *weight, const void *grad_out,
+                             void *grad_input, float *workspace, hipStream_t stream);
+
 // Tap products of the input gradient for layers with few input channels, any x
 // axis kind: Z[n, ci, m, hx, hy] = sum_co w[co, ci, m] * grad_out[n, co, hx, hy]
 // for every tap m = fx * nfy + fy (rows padded to a multiple of 32 per input

@@ -218,9 +218,11 @@ int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input,
  * The kernels read the half tensors as they lie and multiply on the f16 matrix
  * cores (v_mfma_f32_32x32x16_f16), one sixth of the matrix work of the fp32 path
  * on half the bytes: the forward pass and the input gradient through the tiled
- * kernel (variant "mfma-f16"; the input gradient of layers with few input
- * channels, or on a Mellin axis that keeps fewer rows than it is given, as two
- * passes, "mfma-f16+fold", whose intermediate rows and folded result are fp32),
+ * kernel (variant "mfma-f16"; the input gradient of layers with at most three
+ * input channels and a linear x axis through the one-kernel form,
+ * "mfma-f16-fused"; with few input channels otherwise, or on a Mellin axis that
+ * keeps fewer rows than it is given, as two passes, "mfma-f16+fold", whose
+ * intermediate rows and folded result are fp32),
  * the weight gradient through a kernel of its own whose matrix instructions run
  * along the output positions ("mfma-f16"; partial sums in fp32, added in a fixed
  * order).  Scratch memory then holds what those kernels need (the filter cut into
@@ -398,8 +400,8 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
  * output positions, bf16 matrix cores), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
- * (two-pass input gradient), "mfma-f16" and "mfma-f16+fold" (half-precision
- * tensors on the f16 matrix cores). */
+ * (two-pass input gradient), "mfma-f16", "mfma-f16-fused" and "mfma-f16+fold"
+ * (half-precision tensors on the f16 matrix cores). */
 const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).

@@ -72,6 +72,10 @@ def test_half_passes_match_checker_on_the_same_operands(case, half_path):
     egi, egw, _ = bwd(x64, w64, go.astype(np.float64), s, d, p, u)
     gi = torch.full_like(xg, float("nan"))
     hip.corr2d_backward_input(kind_x, wg, to_gpu(go), gi, dims)
+    if half_path == "auto" and CASES.index(case) in (1, 2, 3):
+        # the three forms that read half tensors: one kernel (at most three input channels, linear x
+        # axis), two passes (few input channels otherwise), the tiled kernel (many)
+        assert hip.last_variant() == {1: "mfma-f16-fused", 2: "mfma-f16+fold", 3: "mfma-f16"}[CASES.index(case)]
     _close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
     gw = torch.full_like(wg, float("nan"))
     hip.corr2d_backward_weight(kind_x, xg, to_gpu(go), gw, dims)
@@ -141,6 +145,7 @@ def test_random_layers_agree_between_the_two_half_paths():
     # the sample exercised every kernel that reads half tensors
     assert seen.get(("forward", "mfma-f16"), 0) > 100 and seen.get(("weight", "mfma-f16"), 0) > 100
     assert seen.get(("input", "mfma-f16"), 0) > 30 and seen.get(("input", "mfma-f16+fold"), 0) > 10, seen
+    assert seen.get(("input", "mfma-f16-fused"), 0) > 3, seen
 
 
 def test_workspace_is_required_and_sized():
