@@ -27,6 +27,8 @@ thread_local char g_error[512] = "";
 // Process-wide, not per thread: PyTorch runs the backward pass of device tensors on its
 // autograd thread, and a variant forced from the user's thread must hold there too.
 std::atomic<const char *> g_variant{""};
+std::atomic<int> g_no_classes{0};       // Mellin layers as one launch, not one per residue class (mellin_set_variant "one-launch")
+std::atomic<int> g_all_classes{0};      // ... one per class whatever the layer's size ("classes": for tests)
 std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
@@ -104,10 +106,73 @@ hipError_t run_sepconv(const SepConv &pr, const T *f, const T *g, const T *bias,
   return launch_sepconv_generic<T>(pr, f, g, bias, h, stream);
 }
 
+// A layer on a Mellin x axis as one launch of the tiled kernel per residue class of the axis
+// (tile_gemm.hip: mellin_classes): no launch meets a (row, filter row) pair without a tap, so
+// none stages or multiplies the zeros that stand for such pairs in the single launch.
+constexpr int kMaxClasses = 8;
+struct ClassPlans {
+  int n = 0;
+  TilePlan pl[kMaxClasses];
+  size_t lds[kMaxClasses], frag_off[kMaxClasses];
+  int mt[kMaxClasses], nt[kMaxClasses];
+  size_t frag_bytes = 0;           // all classes' filter fragments, each region 256-byte aligned
+};
+
+// False: the layer stays with the single launch (one class only or too many, a class with no
+// filter row or no plan on the bf16 / f16 matrix cores, a layer too small to pay for the launches).
+bool plan_mellin_classes(const SepConv &pr, ClassPlans &cp) {
+  if (g_forced != 0 || g_no_classes || pr.accumulate || pr.cls_nfx || (!pr.in_half && pr.math == MATH_FP32)) return false;
+  const double work = (double)pr.batch * pr.x.nh * pr.y.nh * pr.c_out * pr.c_in * pr.x.nf * pr.y.nf;
+  // (correlation axes only, i.e. forward passes: the classes of a convolution axis, six for a
+  // four-row filter with p = 1, are launches too small to win -- measured 10-30 % slower on
+  // most layers of the 10-layer stack, in half precision on all of them)
+  if ((work < 4e9 || pr.x.kind != AX_MCORR) && !g_all_classes) return false;
+  MellinClass mc[kMaxClasses];
+  const int n = mellin_classes(pr.x, mc, kMaxClasses);
+  if (n < 2) return false;
+  cp.n = 0;
+  cp.frag_bytes = 0;
+  for (int r = 0; r < n; ++r) {
+    if (mc[r].first >= pr.x.nh) continue;                   // no output row in this class
+    if (mc[r].nfx == 0) return false;                       // rows that are bias alone: the single launch writes them
+    SepConv c = pr;
+    c.cls_stride = mc[r].stride; c.cls_first = mc[r].first; c.cls_nfx = mc[r].nfx; c.cls_fx = mc[r].fx;
+    if (!c.in_half) c.math = MATH_BF16X3_ALWAYS;
+    const int i = cp.n;
+    if (!make_tile_plan(c, cp.pl[i], &cp.lds[i], &cp.mt[i], &cp.nt[i])) return false;
+    cp.frag_off[i] = cp.frag_bytes;
+    cp.frag_bytes += (tile_fragment_bytes(cp.pl[i], cp.mt[i]) + 255) & ~(size_t)255;
+    ++cp.n;
+  }
+  return cp.n >= 2;
+}
+
+// frag_ws: cp.frag_bytes of scratch memory, or null / too little (fp32 layers then build the
+// fragments per stage; half-precision layers need it when cp.frag_bytes is not zero)
+hipError_t launch_mellin_classes(const ClassPlans &cp, const void *f, const void *g, const void *bias, void *h,
+                                 hipStream_t stream, void *frag_ws, size_t frag_bytes) {
+  const bool use_ws = frag_ws && ((uintptr_t)frag_ws & 15) == 0 && frag_bytes >= cp.frag_bytes;
+  for (int i = 0; i < cp.n; ++i) {
+    float *ws = use_ws && tile_fragment_bytes(cp.pl[i], cp.mt[i]) ? (float *)((char *)frag_ws + cp.frag_off[i]) : nullptr;
+    hipError_t e = launch_tile_gemm(cp.pl[i], cp.lds[i], cp.mt[i], cp.nt[i], (const float *)f, (const float *)g,
+                                    (const float *)bias, (float *)h, stream, ws);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 template <>
 hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
                               const float *bias, float *h, hipStream_t stream, void *frag_ws,
                               size_t frag_bytes) {
+  {
+    ClassPlans cp;
+    if (plan_mellin_classes(pr, cp)) {
+      g_variant = "mfma-classes";
+      g_last_math = MATH_BF16X3;
+      return launch_mellin_classes(cp, f, g, bias, h, stream, frag_ws, frag_bytes);
+    }
+  }
   if (g_forced != 1) {
     TilePlan pl;
     size_t lds = 0;
@@ -189,6 +254,10 @@ SepConv forward_problem(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64
 // fragments (0: it would not use any).
 size_t fragment_bytes(const SepConv &pr) {
   if (g_forced == 1) return 0;
+  {
+    ClassPlans cp;
+    if (plan_mellin_classes(pr, cp)) return cp.frag_bytes;
+  }
   TilePlan pl;
   size_t lds = 0;
   int mt = 0, nt = 0;
@@ -641,6 +710,8 @@ struct HalfNative {
   TilePlan pl;
   size_t lds, frag_bytes;
   int mt, nt;
+  bool classes;                    // one launch per residue class of a Mellin axis instead (cls)
+  ClassPlans cls;
 };
 
 // The tiled kernel's plan for `pr` with half-precision operands and results, if it has one
@@ -649,6 +720,11 @@ bool plan_half_native(SepConv pr, HalfNative &hn) {
   if (g_forced == 1 || g_widen) return false;
   pr.in_half = 1;
   pr.out_half = 1;
+  hn.classes = plan_mellin_classes(pr, hn.cls);
+  if (hn.classes) {
+    hn.frag_bytes = hn.cls.frag_bytes;
+    return true;
+  }
   if (!make_tile_plan(pr, hn.pl, &hn.lds, &hn.mt, &hn.nt)) return false;
   hn.frag_bytes = tile_fragment_bytes(hn.pl, hn.mt);
   return true;
@@ -661,8 +737,12 @@ int run_half_native(const char *fn, const HalfNative &hn, const void *f, const v
   if (hn.frag_bytes && ((uintptr_t)workspace & 15))
     return fail(MELLIN_ERR_ARGUMENT, "%s: the workspace must be 16-byte aligned", fn);
   if (!f || !g || !h) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", fn);
-  g_variant = "mfma-f16";
   g_last_math = MELLIN_MATH_F16;
+  if (hn.classes) {
+    g_variant = "mfma-f16-classes";
+    return check_hip(launch_mellin_classes(hn.cls, f, g, bias, h, (hipStream_t)stream, workspace, workspace_bytes), fn);
+  }
+  g_variant = "mfma-f16";
   return check_hip(launch_tile_gemm(hn.pl, hn.lds, hn.mt, hn.nt, (const float *)f, (const float *)g,
                                     (const float *)bias, (float *)h, (hipStream_t)stream,
                                     hn.frag_bytes ? (float *)workspace : nullptr), fn);
@@ -1040,9 +1120,12 @@ int mellin_get_math(void) { return g_math; }
 int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
-  const bool widen = name && !strcmp(name, "widen");
+  const bool widen = name && !strcmp(name, "widen"), one = name && !strcmp(name, "one-launch");
+  const bool all = name && !strcmp(name, "classes");
   g_widen = widen;
-  if (!name || !*name || widen) { g_forced = 0; return MELLIN_OK; }
+  g_no_classes = one;
+  g_all_classes = all;
+  if (!name || !*name || widen || one || all) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
   if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }

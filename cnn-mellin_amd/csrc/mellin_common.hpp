@@ -34,6 +34,12 @@ struct SepConv {
   int relu = 0;                  // with accumulate == 0: h = max(0, bias + result)
   int out_half = 0;              // with accumulate == 0: h is half-precision storage (matrix-core kernel only)
   int in_half = 0;               // f, g and bias are half-precision storage (matrix-core kernel only; accumulate == 0)
+  // One residue class of a Mellin x axis (matrix-core kernel, bf16 / f16 forms only): the
+  // launch covers the output rows cls_first, cls_first + cls_stride, ... and the cls_nfx
+  // filter rows listed in cls_fx (four bits each, lowest first) -- the rows and filter rows
+  // among which every pair has its tap (tile_gemm.hpp: mellin_classes).  cls_nfx == 0: all.
+  int cls_stride = 1, cls_first = 0, cls_nfx = 0;
+  unsigned long long cls_fx = 0;
   int math = 0;                  // MATH_FP32: fp32 matrix instructions; MATH_BF16X3: bf16 ones on three-part operands
 };
 

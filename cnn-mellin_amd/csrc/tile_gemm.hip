@@ -273,7 +273,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
         // channels: such a tap reads the lane's first word, always a staged one, and
         // meets a zero weight)
         const bool whole = k < pl.CC * pl.nf, last = k < cc_last * pl.nf;
-        const int fo = (cl * pl.f_c + t) * EB;
+        const int fo = (cl * pl.f_c + class_filter_row(pl.cls_fx, fx) * pl.nfy + fy) * EB;   // (the layer's filter row)
         tapoff[k] = whole ? off : 0;
         tapoff[pl.KC16 + k] = last ? off : 0;
         tapoff[2 * pl.KC16 + k] = whole ? fo : (int)kDeadOffset;
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
         const int q = tg.q0 + local;
         int ox, oy;
         by_noy.divmod(q, ox, oy);
-        lane_q[t] = q;
+        lane_q[t] = (pl.cls_first + pl.cls_stride * ox) * pl.noy + oy;     // (== q unless the launch is a residue class)
         lane_base[t] = ((pl.Ax * (ox - tg.ox_lo) + pl.Cx0) * pl.RS + pl.ay * (oy - tg.oy_lo) - pl.by_min) * (F16 ? 4 : 1);
       }
     }
@@ -500,7 +500,8 @@ __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int 
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int k = 8 * g + i, cl = k / pl.nf, t = k - cl * pl.nf;
-    x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + t] : (Word)0;
+    const int fx = t / pl.nfy, ta = class_filter_row(pl.cls_fx, fx) * pl.nfy + (t - fx * pl.nfy);   // the layer's tap
+    x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + ta] : (Word)0;
   }
   if constexpr (F16) {
     uintx4 v;
@@ -546,7 +547,15 @@ static int workgroups_per_cu(size_t lds_bytes, int mt, int nt, bool split) {
 // apply (sizes beyond 32-bit indexing or a single channel not fitting in LDS).
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt, int force_nt) {
   const i64 lim = (i64)1 << 30;
-  const i64 nf = pr.x.nf * pr.y.nf, ng = pr.x.ng * pr.y.ng, Q = pr.x.nh * pr.y.nh;
+  // (a residue class of a Mellin axis: the rows and filter rows of the class)
+  const bool cls = pr.cls_nfx > 0;
+  if (cls && (pr.accumulate || (pr.x.kind != AX_MCORR && pr.x.kind != AX_MCONV) || pr.cls_nfx > 16 || pr.cls_stride < 1 ||
+              pr.cls_first < 0 || pr.x.nf > 16))
+    return false;
+  const i64 nfx_k = cls ? pr.cls_nfx : pr.x.nf;
+  const i64 nox_k = cls ? std::max<i64>(0, (pr.x.nh - pr.cls_first + pr.cls_stride - 1) / pr.cls_stride) : pr.x.nh;
+  const i64 nox_eff_k = cls ? std::max<i64>(0, (pr.x.nh_eff - pr.cls_first + pr.cls_stride - 1) / pr.cls_stride) : pr.x.nh_eff;
+  const i64 nf = nfx_k * pr.y.nf, ng = pr.x.ng * pr.y.ng, Q = nox_k * pr.y.nh;
   if (nf <= 0 || ng <= 0 || Q <= 0 || pr.c_in <= 0 || pr.c_out <= 0 || pr.batch <= 0) return false;
   if (nf > 4096 || ng >= lim || Q >= lim || pr.c_in >= lim || pr.c_out >= lim || pr.batch >= lim) return false;
   if (pr.c_in * ng >= lim * 2 || pr.batch * (Q / 64 + 1) >= lim) return false;
@@ -556,9 +565,12 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   if (Y.p > lim || Y.p < -lim || X.p < -lim) return false;
 
   pl.batch = (int)pr.batch; pl.M = (int)pr.c_out; pl.C = (int)pr.c_in;
-  pl.nfx = (int)X.nf; pl.nfy = (int)Y.nf; pl.nf = (int)nf;
-  pl.ngx = (int)X.ng; pl.ngy = (int)Y.ng; pl.nox = (int)X.nh; pl.noy = (int)Y.nh; pl.Q = (int)Q;
-  pl.nox_eff = (int)X.nh_eff; pl.noy_eff = (int)Y.nh_eff;
+  pl.nfx = (int)nfx_k; pl.nfy = (int)Y.nf; pl.nf = (int)nf;
+  pl.ngx = (int)X.ng; pl.ngy = (int)Y.ng; pl.nox = (int)nox_k; pl.noy = (int)Y.nh; pl.Q = (int)Q;
+  pl.nox_eff = (int)nox_eff_k; pl.noy_eff = (int)Y.nh_eff;
+  pl.cls_stride = cls ? pr.cls_stride : 1;
+  pl.cls_first = cls ? pr.cls_first : 0;
+  pl.cls_fx = cls ? pr.cls_fx : 0xFEDCBA9876543210ull;
   pl.f_m = pr.f_m; pl.f_c = pr.f_c; pl.g_n = pr.g_n; pl.g_c = pr.g_c; pl.h_n = pr.h_n; pl.h_m = pr.h_m;
   pl.accumulate = pr.accumulate;
   pl.relu = pr.relu && !pr.accumulate;
@@ -692,7 +704,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   pl.f16 = 0;
   pl.KC16 = 0;
   pl.f_bytes = 0;
-  const i64 f_extent = (pr.in_half ? 2 : 4) * ((pr.c_out - 1) * pr.f_m + (pr.c_in - 1) * pr.f_c + nf);
+  const i64 f_extent = (pr.in_half ? 2 : 4) * ((pr.c_out - 1) * pr.f_m + (pr.c_in - 1) * pr.f_c + pr.x.nf * pr.y.nf);
   const size_t frag_word = pr.in_half ? 2 : 6;              // fragment bytes per filter word
   auto split_lds = [&](int sbuf, i64 ccs, bool one_chunk) {
     const size_t kc16 = (size_t)((ccs * pl.nf + 15) / 16) * 16;
@@ -783,7 +795,44 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     const i64 wgs = (i64)pl.total_tiles * m_tiles;
     if (wgs > slots2 && wgs <= slots1) { pl.sbuf = 1; *lds_bytes = one; }
   }
+  if (cls && !pl.split) return false;                      // (the filter rows of a class are picked through the fragment tables)
   return true;
+}
+
+// Residue classes of a Mellin x axis.  On a correlation axis the tap of (row h, filter row f)
+// exists iff (h + s)(f + d) is a multiple of p + 1: rows with the same (h + s) mod (p + 1)
+// have taps for the same filter rows.  On a convolution axis it exists iff (p + 1)(h + s) is a
+// multiple of f + d, i.e. iff h + s is a multiple of m_f = (f + d) / gcd(f + d, p + 1): rows
+// with the same (h + s) mod lcm(m_f) do.  A launch over one class meets no pair without a
+// tap (other than taps outside the signal), so nothing is staged or multiplied for them.
+int mellin_classes(const Axis &x, MellinClass *out, int max_classes) {
+  auto gcd = [](i64 a, i64 b) { while (b) { const i64 t = a % b; a = b; b = t; } return a; };
+  if ((x.kind != AX_MCORR && x.kind != AX_MCONV) || x.nf < 1 || x.nf > 16) return 0;
+  i64 L = 1;
+  if (x.kind == AX_MCORR) {
+    L = x.p + 1;
+  } else {
+    for (i64 f = 0; f < x.nf; ++f) {
+      const i64 m = (f + x.d) / gcd(f + x.d, x.p + 1);
+      L = L / gcd(L, m) * m;
+      if (L > max_classes) return 0;
+    }
+  }
+  if (L < 2 || L > max_classes) return 0;
+  const i64 shift = x.s;
+  for (i64 r = 0; r < L; ++r) {
+    MellinClass &c = out[r];
+    c.stride = (int)L;
+    c.first = (int)(((r - shift) % L + L) % L);
+    c.nfx = 0;
+    c.fx = 0;
+    for (i64 f = 0; f < x.nf; ++f) {
+      const bool has = x.kind == AX_MCORR ? (r * (f + x.d)) % (x.p + 1) == 0
+                                          : r % ((f + x.d) / gcd(f + x.d, x.p + 1)) == 0;
+      if (has) c.fx |= (unsigned long long)f << (4 * c.nfx++);
+    }
+  }
+  return (int)L;
 }
 
 size_t tile_fragment_bytes(const TilePlan &pl, int mt) {

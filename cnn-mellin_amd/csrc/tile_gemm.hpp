@@ -38,7 +38,24 @@ struct TilePlan {
   int f16;                         // (with split) half-precision operands on the f16 matrix cores instead: one part
   int KC16;                        // split: CC * nf rounded up to a multiple of 16
   unsigned f_bytes;                // split: bytes from the filter's first word to its last one's end
+  // a residue class of a Mellin x axis (SepConv::cls_*): kernel row i is output row
+  // cls_first + cls_stride * i, kernel filter row j is the layer's filter row (cls_fx >> 4 j) & 15;
+  // nfx / nf / nox / Q above then count the class's rows.  1, 0 and the identity otherwise.
+  int cls_stride, cls_first;
+  unsigned long long cls_fx;
 };
+
+// the layer's filter row behind kernel filter row j
+__host__ __device__ inline int class_filter_row(unsigned long long cls_fx, int j) { return (int)((cls_fx >> (4 * j)) & 15); }
+
+// One residue class of a Mellin axis: output rows first, first + stride, ...; nfx filter rows, listed in fx
+struct MellinClass {
+  int stride, first, nfx;
+  unsigned long long fx;
+};
+// The classes of axis x into out[0 .. n); 0: the axis has one class only, more than
+// max_classes, or is not a Mellin axis (nothing to gain, or too many launches).
+int mellin_classes(const Axis &x, MellinClass *out, int max_classes);
 
 // force_nt: 0 lets the plan pick the number of 32-position tiles per wavefront
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt,

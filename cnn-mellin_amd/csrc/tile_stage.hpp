@@ -267,7 +267,8 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
       if (mellin_x) {
         int oxl, fx;
         by_nfx1.divmod(r, oxl, fx);
-        gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux, pl.mg_p1);
+        gx = mellin_tap32(pl.kind_x, pl.cls_first + pl.cls_stride * (tg.ox_lo + oxl), class_filter_row(pl.cls_fx, fx), pl.ngx, pl.sx, pl.dx,
+                          pl.px + 1, pl.ux, pl.mg_p1);
       } else {
         const int vx = tg.vx_min + r;
         if (vx >= 0) {
@@ -320,7 +321,8 @@ __device__ __forceinline__ void issue_signal(const PL &pl, const TileGeom &tg,
         if (mellin_x) {
           int oxl, fx;
           by_nfx.divmod(r, oxl, fx);
-          gx = mellin_tap32(pl.kind_x, tg.ox_lo + oxl, fx, pl.ngx, pl.sx, pl.dx, pl.px + 1, pl.ux, pl.mg_p1);
+          gx = mellin_tap32(pl.kind_x, pl.cls_first + pl.cls_stride * (tg.ox_lo + oxl), class_filter_row(pl.cls_fx, fx), pl.ngx, pl.sx, pl.dx,
+                          pl.px + 1, pl.ux, pl.mg_p1);
         } else {
           const int vx = tg.vx_min + r;
           if (vx >= 0) {

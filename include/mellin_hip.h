@@ -400,8 +400,12 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
  * output positions, bf16 matrix cores), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
- * (two-pass input gradient), "mfma-f16", "mfma-f16-fused" and "mfma-f16+fold"
- * (half-precision tensors on the f16 matrix cores). */
+ * (two-pass input gradient), "mfma-classes" (a layer on a Mellin axis as one
+ * launch of the tiled kernel per residue class of the axis: rows with the same
+ * (h + s) mod (p + 1) have taps for the same filter rows, so no launch meets a
+ * (row, filter row) pair without a tap), "mfma-f16", "mfma-f16-classes",
+ * "mfma-f16-fused" and "mfma-f16+fold" (half-precision tensors on the f16
+ * matrix cores). */
 const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).
@@ -433,7 +437,9 @@ int mellin_last_math(void);
  * kernels ("mfma-fused", "mfma-taps+fold", "mfma-rows", "mfma-positions"), i.e. the
  * tiled ones;
  * "widen" = automatic choice, but the half-precision entry points always go
- * through fp32 copies of their operands (for comparisons).
+ * through fp32 copies of their operands (for comparisons); "one-launch" /
+ * "classes" = automatic choice, but layers on a Mellin axis never / whatever
+ * their size run as one launch per residue class (for comparisons and tests).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);
 

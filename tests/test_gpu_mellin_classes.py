@@ -1,0 +1,124 @@
+"""A Mellin layer as one launch of the tiled kernel per residue class of its x axis.
+
+On a Mellin correlation axis the tap of (output row h, filter row f) exists iff
+(h + s)(f + d) is a multiple of p + 1, so the rows with the same (h + s) mod (p + 1) have
+taps for the same filter rows; on a convolution axis (the input gradient in gather form)
+rows with the same (h + s) mod lcm_f((f + d) / gcd(f + d, p + 1)) do.  A launch over one
+class walks only the filter rows that class has and writes only its rows: the union of
+the launches must be the layer, to the operator tolerance against the float64 checker
+(rtol 1e-5 / atol 1e-5 * sqrt(fan_in)) in fp32 and to the rounding of a half result
+against the single launch in half precision.  The "classes" variant forces the form on
+layers of any size; by default forward passes of 4 GMAC (taps without a source counted)
+and more take it.
+"""
+import numpy as np
+import pytest
+import torch
+
+import _mellin_hip as hip
+from _gpu import assert_close, to_gpu
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # (n, c_in, c_out, nf, ng, s, d, p, r): two classes, the stack's layer shape, rows past the support
+    (2, 100, 70, (4, 4), (40, 5), (1, 1), (1, 1), (1, 1), (20, 0)),
+    # four classes, two of them with one filter row of four; row-wise staging
+    (2, 40, 33, (4, 3), (60, 24), (1, 1), (1, 1), (3, 2), (7, 0)),
+    # three classes, stride and dilation: class r has the filter rows with r (f + 2) a multiple of 3
+    (3, 20, 64, (6, 2), (50, 9), (2, 1), (2, 1), (2, 0), (0, 1)),
+    # few channels (one chunk), eight filter rows, 1-D
+    (4, 3, 40, (8, 1), (90, 1), (1, 1), (1, 1), (3, 0), (10, 0)),
+    # a class without output rows (one output row, two classes)
+    (2, 16, 16, (2, 2), (2, 8), (1, 1), (1, 1), (1, 0), (0, 0)),
+]
+
+
+seen_gi = []
+
+
+@pytest.fixture
+def classes_forced():
+    hip.set_variant("classes")
+    yield
+    hip.set_variant(None)
+
+
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_classes_match_checker(case, classes_forced):
+    n, c_in, c_out, nf, ng, s, d, p, r = case
+    rng = np.random.default_rng(3000 + CASES.index(case))
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float32)
+    w = (rng.standard_normal((c_out, c_in) + nf) * (c_in * nf[0] * nf[1]) ** -0.5).astype(np.float32)
+    b = rng.standard_normal(c_out).astype(np.float32)
+    exp = oracle.mcorrlcorr(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64), s, d, p, (1, 1), r)
+    nh = exp.shape[2:]
+    assert min(nh) > 0
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    egi, _, _ = oracle.mcorrlcorr_backward(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64),
+                                           s, d, p, (1, 1))
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, (1, 1))
+    out = torch.full(exp.shape, float("nan"), device="cuda")                 # every word must be written
+    hip.corr2d_forward(hip.AX_MCORR, to_gpu(x), to_gpu(w), to_gpu(b), out, dims)
+    single_row = nh[0] == 1
+    assert hip.last_variant() == ("mfma" if single_row else "mfma-classes")  # one class with rows: nothing to split
+    assert_close(out, exp, c_in * nf[0] * nf[1], "forward %s" % (case,))
+    if c_in >= 16 and not single_row:
+        # the gather-form input gradient is a convolution axis
+        gi = torch.full(x.shape, float("nan"), device="cuda")
+        hip.corr2d_backward_input(hip.AX_MCORR, to_gpu(w), to_gpu(go), gi, dims)
+        seen_gi.append(hip.last_variant())                                   # (layers that keep fewer rows than they are given take two passes)
+        assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
+
+
+def test_half_classes_match_the_single_launch(classes_forced):
+    for case in CASES[:3]:
+        n, c_in, c_out, nf, ng, s, d, p, r = case
+        gen = torch.Generator().manual_seed(9)
+        x = torch.randn((n, c_in) + ng, generator=gen).half().cuda()
+        w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_in * nf[0] * nf[1]) ** -0.5).half().cuda()
+        b = torch.randn(c_out, generator=gen).half().cuda()
+        import mconv
+        nh = (mconv.mcorr_valid_size(nf[0], ng[0], s[0], d[0], p[0], 1) + r[0],
+              mconv.lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], 1) + r[1])
+        dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, (1, 1))
+        got = torch.full((n, c_out) + nh, float("nan"), dtype=torch.float16, device="cuda")
+        hip.corr2d_forward(hip.AX_MCORR, x, w, b, got, dims)
+        assert hip.last_variant() == "mfma-f16-classes"
+        hip.set_variant("one-launch")
+        ref = torch.full_like(got, float("nan"))
+        hip.corr2d_forward(hip.AX_MCORR, x, w, b, ref, dims)
+        assert hip.last_variant() == "mfma-f16"
+        hip.set_variant("classes")
+        tol = 2.0 ** -10 * ref.float().abs() + 2e-5 * (c_in * nf[0] * nf[1]) ** 0.5
+        assert bool(((got.float() - ref.float()).abs() <= tol).all()), case
+
+
+def test_large_forward_passes_take_the_classes_by_default():
+    """5 GMAC with the taps without a source counted: one launch per class, and the same
+    values as the single launch up to the order of summation."""
+    n, c_in, c_out, nf, ng, p = 8, 128, 128, (4, 4), (120, 20), (1, 1)
+    gen = torch.Generator().manual_seed(10)
+    x = torch.randn((n, c_in) + ng, generator=gen).cuda()
+    w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_in * 16) ** -0.5).cuda()
+    b = torch.randn(c_out, generator=gen).cuda()
+    import mconv
+    nh = (mconv.mcorr_valid_size(4, 120, 1, 1, 1, 1) + 60, mconv.lcorr_valid_size(4, 20, 1, 1, 1, 1) + 2)
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), p, (1, 1))
+    got = torch.full((n, c_out) + nh, float("nan"), device="cuda")
+    hip.corr2d_forward(hip.AX_MCORR, x, w, b, got, dims)
+    assert hip.last_variant() == "mfma-classes" and hip.last_math() == hip.MATH_BF16X3
+    hip.set_variant("one-launch")
+    try:
+        ref = torch.full_like(got, float("nan"))
+        hip.corr2d_forward(hip.AX_MCORR, x, w, b, ref, dims)
+        assert hip.last_variant() == "mfma"
+    finally:
+        hip.set_variant(None)
+    assert bool(((got - ref).abs() <= 1e-5 * ref.abs() + 1e-5 * (c_in * 16) ** 0.5).all())
+
+
+def test_some_input_gradient_took_the_classes():
+    """(after the parametrized cases of this file: tests run in the order they are written)"""
+    assert "mfma-classes" in seen_gi, seen_gi
