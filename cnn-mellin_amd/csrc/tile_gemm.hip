@@ -35,6 +35,7 @@
 // MT * NT accumulator tiles (16 registers each).  Stores write 128-byte runs
 // of one output row.
 #include <algorithm>
+#include <vector>
 #include <type_traits>
 
 #include "mellin_common.hpp"
@@ -61,19 +62,20 @@ namespace {
 // storage and the products run on the f16 matrix cores (tile_stage.hpp); the signal is
 // staged one value per LDS word like the floats, the filter fragments have one part.
 // H is half-precision (HOUT) or fp32 storage.
+// bx of gx: this workgroup among those that share the plan at plan_base (the whole launch,
+// or one residue class's share of it).
+typedef const __attribute__((address_space(4))) TilePlan ConstPlan;
 template <int MT, int NT, bool ACC, int MB, bool HOUT, int SPLIT>
-__global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
-    TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
+__device__ __forceinline__ void tile_gemm_body(
+    ConstPlan *const plan_base, const int bx, const int gx, const float *__restrict__ F, const float *__restrict__ G,
     const float *__restrict__ bias, float *__restrict__ H, const float *__restrict__ AF) {
-  // The plan is read where it lies, in the kernel-argument segment (it is the
-  // first argument), through a pointer the compiler must treat as new in every
+  // The plan is read where it lies, in the kernel-argument segment, through a pointer the
+  // compiler must treat as new in every
   // iteration of the stage loop: fields are then re-read by scalar loads where
   // they are used instead of all being held in scalar registers for the whole
   // kernel, which had the register allocator spill hundreds of them to vector
   // lanes around the stores and the staging code.
   constexpr int kMemo = MB;
-  typedef const __attribute__((address_space(4))) TilePlan ConstPlan;
-  ConstPlan *const plan_base = (ConstPlan *)__builtin_amdgcn_kernarg_segment_ptr();
   ConstPlan *plp = plan_base;
 #define pl (*plp)
   extern __shared__ __align__(16) float lds[];
@@ -182,9 +184,8 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   };
 
   // ---- stages owned by this workgroup ------------------------------------------
-  // tiles blockIdx.x, blockIdx.x + gridDim.x, ...; each tile has `chunks` stages
-  const int my_tiles = (int)blockIdx.x < pl.total_tiles
-                           ? (pl.total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+  // tiles bx, bx + gx, ...; each tile has `chunks` stages
+  const int my_tiles = bx < pl.total_tiles ? (pl.total_tiles - 1 - bx) / gx + 1 : 0;
   const int my_stages = my_tiles * chunks;
   StageMemo<kMemo> memo = {};
   // (stage_zero: a zero renewed every stage that the compiler cannot see through; adding
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   unsigned stage_zero = 0;
   auto issue_stage = [&](int st, int ti, int ch) {           // st = ti * chunks + ch
     const int wave = wave_id + (int)stage_zero;
-    const TileGeom tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
+    const TileGeom tg = tile_geometry<P>(pl, bx + ti * gx, mellin_x);
     const int c0 = ch * pl.CC, cc = min(pl.CC, pl.C - c0);
     const int sb = (st & 1) * (pl.sbuf - 1) * g_words;    // sbuf == 1: a workgroup has one stage only
     // the sources worked out for a tile's first chunk serve its other chunks; a buffer's
@@ -426,7 +427,7 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
     }
     if (ch == 0) {
       if (st > 0) epilogue();                             // the tile finished one stage ago
-      tg = tile_geometry<P>(pl, blockIdx.x + ti * gridDim.x, mellin_x);
+      tg = tile_geometry<P>(pl, bx + ti * gx, mellin_x);
       // position -> LDS word of its (fx = 0, fy = 0) tap
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -475,6 +476,37 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void til
   }
   if (my_stages > 0) epilogue();
 #undef pl
+}
+
+template <int MT, int NT, bool ACC, int MB, bool HOUT, int SPLIT>
+__global__ __launch_bounds__(kThreads, (NT == 1 ? (SPLIT ? 3 : 4) : 2)) void tile_gemm_kernel(
+    TilePlan plan_arg, const float *__restrict__ F, const float *__restrict__ G,
+    const float *__restrict__ bias, float *__restrict__ H, const float *__restrict__ AF) {
+  // (the plan is the first argument: the kernel-argument segment starts with it)
+  tile_gemm_body<MT, NT, ACC, MB, HOUT, SPLIT>((ConstPlan *)__builtin_amdgcn_kernarg_segment_ptr(), (int)blockIdx.x,
+                                              (int)gridDim.x, F, G, bias, H, AF);
+}
+
+// The residue classes of a Mellin layer in one launch: workgroups wg_end[c - 1] .. wg_end[c] - 1
+// of grid.x are class c's for their whole life, with that class's plan and fragments.
+struct ClassLaunch {
+  TilePlan pl[kMaxTileClasses];
+  int n, wg_end[kMaxTileClasses];
+  long long af_words[kMaxTileClasses];               // where the class's fragments start in AF (floats)
+};
+
+static_assert(sizeof(ClassLaunch) + 5 * sizeof(void *) <= 4096, "kernel arguments are limited to 4 KB");
+
+template <int MT, int NT, bool HOUT, int SPLIT>
+__global__ __launch_bounds__(kThreads, (NT == 1 ? 3 : 2)) void tile_gemm_classes_kernel(
+    ClassLaunch args, const float *__restrict__ F, const float *__restrict__ G,
+    const float *__restrict__ bias, float *__restrict__ H, const float *__restrict__ AF) {
+  typedef const __attribute__((address_space(4))) ClassLaunch ConstArgs;
+  ConstArgs *const a = (ConstArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+  int c = 0, first = 0;
+  for (; c + 1 < a->n && (int)blockIdx.x >= a->wg_end[c]; ++c) first = a->wg_end[c];
+  tile_gemm_body<MT, NT, false, 0, HOUT, SPLIT>((ConstPlan *)&a->pl[c], (int)blockIdx.x - first, a->wg_end[c] - first, F,
+                                               G, bias, H, AF ? AF + a->af_words[c] : AF);
 }
 
 // The whole filter as fragments, once per launch, in the order the stages of the SPLIT
@@ -529,6 +561,23 @@ hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const
     }
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, pl, f, g, bias, h, af);
+  return hipGetLastError();
+}
+
+template <int MT, int NT, bool HOUT, int SPLIT>
+hipError_t launch_classes_variant(const ClassLaunch &args, size_t lds_bytes, dim3 grid, const float *f, const float *g,
+                                  const float *bias, float *h, hipStream_t stream, const float *af) {
+  auto kern = tile_gemm_classes_kernel<MT, NT, HOUT, SPLIT>;
+  if (lds_bytes > 64 * 1024) {
+    static thread_local size_t granted = 0;
+    if (granted < lds_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds_bytes);
+      if (e != hipSuccess) return e;
+      granted = lds_bytes;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, args, f, g, bias, h, af);
   return hipGetLastError();
 }
 
@@ -911,6 +960,91 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
   MELLIN_TILE_CASE(1, 2)
   MELLIN_TILE_CASE(1, 1)
 #undef MELLIN_TILE_CASE
+  return hipErrorInvalidValue;
+}
+
+bool tile_classes_fit_one_launch(const TilePlan *pls, const int *mts, const int *nts, int n) {
+  if (n < 2 || n > kMaxTileClasses) return false;
+  for (int i = 0; i < n; ++i) {
+    const TilePlan &p = pls[i];
+    if (!p.split || p.accumulate || p.sbuf != 2 || p.CC >= p.C) return false;    // bf16 / f16 forms staged in chunks
+    if (mts[i] != mts[0] || nts[i] != nts[0] || p.M != pls[0].M || p.f16 != pls[0].f16 || p.out_half != pls[0].out_half)
+      return false;
+    if (!p.f16 && mts[i] != 2) return false;                                       // (the instances built below)
+  }
+  return true;
+}
+
+hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes, int n, int mt, int nt, const float *f,
+                                    const float *g, const float *bias, float *h, hipStream_t stream, float *frag_ws,
+                                    const size_t *frag_off) {
+  if (!tile_classes_fit_one_launch(pls, std::vector<int>(n, mt).data(), std::vector<int>(n, nt).data(), n))
+    return hipErrorInvalidValue;
+  const int M_T = mt * 32;
+  const bool f16 = pls[0].f16;
+  if (f16 && !frag_ws) return hipErrorInvalidValue;          // no per-stage build in that kernel
+  ClassLaunch args;
+  args.n = n;
+  size_t lds = 0;
+  double work[kMaxTileClasses];                              // per tile
+  for (int i = 0; i < n; ++i) {
+    args.pl[i] = pls[i];
+    lds = std::max(lds, lds_bytes[i]);
+    const int chunks = (pls[i].C + pls[i].CC - 1) / pls[i].CC;
+    work[i] = (double)chunks * pls[i].KC16;
+    args.af_words[i] = 0;
+    if (frag_ws) {
+      const i64 items = (i64)tile_fragment_bytes(pls[i], mt) / (f16 ? 16 : 48);
+      float *ws = (float *)((char *)frag_ws + frag_off[i]);
+      hipLaunchKernelGGL((f16 ? filter_fragments_kernel<true> : filter_fragments_kernel<false>),
+                         dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pls[i], M_T, chunks, (const void *)f,
+                         (uintx4 *)ws);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return e;
+      args.af_words[i] = (long long)(frag_off[i] / 4);
+    }
+  }
+  // persistent workgroups: as many as fit at once, dealt to the classes by their work
+  const int m_tiles = (pls[0].M + M_T - 1) / M_T;
+  const int per_cu = workgroups_per_cu(lds, mt, nt, true);
+  const int slots = std::max(n, (256 * per_cu) / m_tiles);
+  // A class's workgroups take whole tiles in rounds, and the launch lasts as long as the
+  // class that finishes last: one workgroup each, then every further one to the class whose
+  // rounds times work per tile is largest.
+  int gxs[kMaxTileClasses];
+  for (int i = 0; i < n; ++i) gxs[i] = 1;
+  for (int left = slots - n; left > 0; --left) {
+    int worst = -1;
+    double worst_cost = 0;
+    for (int i = 0; i < n; ++i) {
+      if (gxs[i] >= pls[i].total_tiles) continue;
+      const double cost = (double)((pls[i].total_tiles + gxs[i] - 1) / gxs[i]) * work[i];
+      if (worst < 0 || cost > worst_cost) { worst = i; worst_cost = cost; }
+    }
+    if (worst < 0) break;
+    ++gxs[worst];
+  }
+  int end = 0;
+  for (int i = 0; i < n; ++i) {
+    end += gxs[i];
+    args.wg_end[i] = end;
+  }
+  for (int i = n; i < kMaxTileClasses; ++i) args.wg_end[i] = end;
+  dim3 grid((unsigned)end, (unsigned)m_tiles);
+#define MELLIN_CLASSES_CASE(MT_, NT_, SPLIT_)                                                                  \
+  if (mt == MT_ && nt == NT_ && (f16 ? 4 : 2) == SPLIT_) {                                                     \
+    if (pls[0].out_half) return launch_classes_variant<MT_, NT_, true, SPLIT_>(args, lds, grid, f, g, bias, h, stream, frag_ws); \
+    return launch_classes_variant<MT_, NT_, false, SPLIT_>(args, lds, grid, f, g, bias, h, stream, frag_ws);   \
+  }
+  MELLIN_CLASSES_CASE(2, 2, 2)
+  MELLIN_CLASSES_CASE(2, 1, 2)
+  MELLIN_CLASSES_CASE(4, 2, 4)
+  MELLIN_CLASSES_CASE(4, 1, 4)
+  MELLIN_CLASSES_CASE(2, 2, 4)
+  MELLIN_CLASSES_CASE(2, 1, 4)
+  MELLIN_CLASSES_CASE(1, 2, 4)
+  MELLIN_CLASSES_CASE(1, 1, 4)
+#undef MELLIN_CLASSES_CASE
   return hipErrorInvalidValue;
 }
 

@@ -48,6 +48,8 @@ struct TilePlan {
 // the layer's filter row behind kernel filter row j
 __host__ __device__ inline int class_filter_row(unsigned long long cls_fx, int j) { return (int)((cls_fx >> (4 * j)) & 15); }
 
+constexpr int kMaxTileClasses = 8;                  // residue classes one launch can hold
+
 // One residue class of a Mellin axis: output rows first, first + stride, ...; nfx filter rows, listed in fx
 struct MellinClass {
   int stride, first, nfx;
@@ -74,6 +76,16 @@ size_t tile_fragment_bytes(const TilePlan &pl, int mt);
 hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt,
                             const float *f, const float *g, const float *bias,
                             float *h, hipStream_t stream, float *frag_ws = nullptr);
+
+// The plans of a Mellin layer's residue classes in ONE launch: every workgroup belongs to one
+// class for its whole life, the classes share the chip in proportion to their work.
+// tile_classes_fit_one_launch: the plans allow it (same tile shape, all staged in chunks on
+// the bf16 / f16 matrix cores).  frag_ws + frag_off[i]: class i's fragments (required for
+// half precision), or frag_ws null.
+bool tile_classes_fit_one_launch(const TilePlan *pls, const int *mts, const int *nts, int n);
+hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes, int n, int mt, int nt, const float *f,
+                                    const float *g, const float *bias, float *h, hipStream_t stream, float *frag_ws,
+                                    const size_t *frag_off);
 
 // Weight gradient (wgrad_gemm.hip): position tiling and signal staging of the
 // forward problem in `t`, plus the blocking of the (c_out) x (c_in * taps) output.

@@ -403,7 +403,9 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
  * (two-pass input gradient), "mfma-classes" (a layer on a Mellin axis as one
  * launch of the tiled kernel per residue class of the axis: rows with the same
  * (h + s) mod (p + 1) have taps for the same filter rows, so no launch meets a
- * (row, filter row) pair without a tap), "mfma-f16", "mfma-f16-classes",
+ * (row, filter row) pair without a tap), "mfma-f16", "mfma-f16-classes" (the
+ * classes of a half-precision layer sharing one launch) and
+ * "mfma-f16-class-launches" (a launch each),
  * "mfma-f16-fused" and "mfma-f16+fold" (half-precision tensors on the f16
  * matrix cores). */
 const char *mellin_last_variant(void);
@@ -439,7 +441,8 @@ int mellin_last_math(void);
  * "widen" = automatic choice, but the half-precision entry points always go
  * through fp32 copies of their operands (for comparisons); "one-launch" /
  * "classes" = automatic choice, but layers on a Mellin axis never / whatever
- * their size run as one launch per residue class (for comparisons and tests).
+ * their size run per residue class (for comparisons and tests; "class-launches":
+ * like "classes", with a launch per class also where one launch would hold them).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);
 

@@ -85,7 +85,12 @@ def test_half_classes_match_the_single_launch(classes_forced):
         dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, (1, 1))
         got = torch.full((n, c_out) + nh, float("nan"), dtype=torch.float16, device="cuda")
         hip.corr2d_forward(hip.AX_MCORR, x, w, b, got, dims)
-        assert hip.last_variant() == "mfma-f16-classes"
+        # (classes that are all staged in chunks of channels share one launch: the first layer's)
+        assert hip.last_variant() == ("mfma-f16-classes" if case is CASES[0] else "mfma-f16-class-launches"), case
+        hip.set_variant("class-launches")
+        each = torch.full_like(got, float("nan"))
+        hip.corr2d_forward(hip.AX_MCORR, x, w, b, each, dims)
+        assert hip.last_variant() == "mfma-f16-class-launches" and torch.equal(each, got)   # the same plans, the same sums
         hip.set_variant("one-launch")
         ref = torch.full_like(got, float("nan"))
         hip.corr2d_forward(hip.AX_MCORR, x, w, b, ref, dims)

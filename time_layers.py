@@ -166,6 +166,9 @@ def main():
                     help="how the matrix kernels form fp32 products (library default: bf16x3)")
     ap.add_argument("--dtype", choices=["float32", "half"], default="float32",
                     help="half: half-precision tensors through the f16 entry points")
+    ap.add_argument("--variant", default=None,
+                    help="a kernel variant for comparisons (mellin_set_variant: two-pass, one-launch, classes, "
+                         "class-launches, widen, generic)")
     args = ap.parse_args()
     import torch
     if not torch.cuda.is_available():
@@ -173,6 +176,7 @@ def main():
     torch.cuda.set_device(0)
     import _mellin_hip as hip
     hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
+    hip.set_variant(args.variant)
     dtype = torch.float16 if args.dtype == "half" else torch.float32
     {"cfg2": run_cfg2, "cfg3": run_cfg3, "cfg4": run_cfg4, "stack": run_stack}[args.config](args.reps, dtype)
 
