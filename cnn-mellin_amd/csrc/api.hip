@@ -4,8 +4,10 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
+#include <numeric>
 
 #include "../../include/mellin_hip.h"
 #include "mellin_common.hpp"
@@ -344,12 +346,86 @@ struct TwoPassInput {
   size_t frag_off, frag_bytes;     // the first pass's filter fragments, behind Y in the workspace
   int mt, nt;
   Axis fold;
+  // The first pass as a launch per filter row (rows > 0; plan_first_pass_rows): launch i works
+  // out the c_in output channels of filter row fx[i], on the rows of grad_out that have a tap
+  // of that filter row and on no others.
+  int rows = 0;
+  TilePlan row_plan[kMaxClasses];
+  size_t row_lds[kMaxClasses], row_frag_off[kMaxClasses];    // (fragment regions: offsets from frag_off)
+  int row_mt[kMaxClasses], row_nt[kMaxClasses], row_fx[kMaxClasses];
 };
+
+// On a Mellin x axis with p > 0 the fold reads Y[., ci * nfx + fx, hx, .] only where
+// (hx + s)(fx + d) is a multiple of p + 1 and the tap (hx + s)(fx + d)/(p + 1) - u is a row
+// of grad_input: for filter row fx, the rows hx = first, first + q, ... with
+// q = (p + 1) / gcd(fx + d, p + 1), up to the last one whose tap is inside.  A launch per
+// filter row over exactly those rows (a residue class of an identity axis, c_in output
+// channels, the filter and Y addressed with the filter row's offsets and the strides of the
+// (input channel, filter row) layout) multiplies nothing the fold does not read; the single
+// launch works out every (row, filter row) pair.  Taken when that saves a fifth of the
+// 32-channel row blocks or more.  `first` is the single launch's problem.
+bool plan_first_pass_rows(const SepConv &first, i64 c_in, i64 nfx, i64 nfy, i64 nhx, i64 ngx, i64 ngy, i64 sx, i64 dx,
+                          i64 px, i64 ux, TwoPassInput &tp) {
+  tp.rows = 0;
+  if (g_forced != 0 || g_no_classes || px < 1 || nfx < 2 || nfx > kMaxClasses) return false;
+  if (!first.in_half && first.math == MATH_FP32) return false;         // (classes run on the bf16 / f16 matrix cores)
+  i64 lo[kMaxClasses], hi[kMaxClasses], q[kMaxClasses];
+  i64 blocks = 0;
+  int n = 0;
+  for (i64 fx = 0; fx < nfx; ++fx) {
+    const i64 k = fx + dx, g = std::gcd(k, px + 1);
+    const i64 step = (px + 1) / g;
+    // t = hx + s: a multiple of step with u (p + 1) <= t k <= (ngx - 1 + u)(p + 1), hx in [0, nhx)
+    const i64 t_lo = std::max<i64>(sx, (ux * (px + 1) + k - 1) / k);
+    const i64 t_hi = std::min<i64>(nhx - 1 + sx, (ngx - 1 + ux) * (px + 1) / k);
+    const i64 t_first = (t_lo + step - 1) / step * step, t_last = t_hi / step * step;
+    if (t_first > t_last) continue;                                    // no tap of this filter row at all
+    lo[n] = t_first - sx; hi[n] = t_last - sx; q[n] = step;
+    tp.row_fx[n] = (int)fx;
+    blocks += ((c_in + 31) / 32) * ((hi[n] - lo[n]) / step + 1);
+    ++n;
+  }
+  if (n == 0 || blocks * 5 > ((c_in * nfx + 31) / 32) * nhx * 4) return false;
+  size_t frag = 0;
+  for (int i = 0; i < n; ++i) {
+    SepConv c = first;
+    c.x = make_axis(AX_MCORR, 1, nhx, hi[i] + 1, 1, 1, 0, 1);          // tap (h + 1)(0 + 1)/1 - 1 = h: rows pass through
+    c.c_out = c_in;
+    c.f_m = nfx * nfy;
+    c.h_m = nfx * nhx * ngy;
+    c.cls_stride = (int)q[i]; c.cls_first = (int)lo[i]; c.cls_nfx = 1; c.cls_fx = 0;
+    if (!c.in_half) c.math = MATH_BF16X3_ALWAYS;
+    if (!make_tile_plan(c, tp.row_plan[i], &tp.row_lds[i], &tp.row_mt[i], &tp.row_nt[i])) return false;
+    tp.row_frag_off[i] = frag;
+    frag += (tile_fragment_bytes(tp.row_plan[i], tp.row_mt[i]) + 255) & ~(size_t)255;
+  }
+  tp.rows = n;
+  tp.frag_bytes = frag;
+  return true;
+}
+
+// The first pass of a two-pass plan: Y (fp32) from the weight and grad_out (elem_bytes each).
+hipError_t launch_first_pass(const TwoPassInput &tp, const void *weight, const void *grad_out, void *ws,
+                             int elem_bytes, hipStream_t stream) {
+  float *frag = tp.frag_bytes ? (float *)((char *)ws + tp.frag_off) : nullptr;
+  if (tp.rows == 0)
+    return launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight, (const float *)grad_out, nullptr,
+                            (float *)ws, stream, frag);
+  for (int i = 0; i < tp.rows; ++i) {
+    const TilePlan &pl = tp.row_plan[i];
+    const i64 fx = tp.row_fx[i];
+    float *af = tile_fragment_bytes(pl, tp.row_mt[i]) ? (float *)((char *)frag + tp.row_frag_off[i]) : nullptr;
+    hipError_t e = launch_tile_gemm(pl, tp.row_lds[i], tp.row_mt[i], tp.row_nt[i],
+                                    (const float *)((const char *)weight + fx * pl.nfy * elem_bytes),
+                                    (const float *)grad_out, nullptr, (float *)ws + fx * pl.ngx * pl.noy, stream, af);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
 
 bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 ngx,
                          i64 ngy, i64 nhx, i64 nhy, i64 sx, i64 sy, i64 dx, i64 dy, i64 px,
                          i64 py, i64 ux, i64 uy, TwoPassInput &tp, bool half = false) {
-  (void)sx;
   const i64 m2 = c_in * nfx;
   // worth it when c_in alone would leave most of a 32-row tile empty and the
   // (c_in, filter row) pairs fill tiles reasonably
@@ -358,7 +434,15 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   // works on the nhx rows of grad_out, the gather form on the ngx rows of grad_input,
   // most of whose (position, filter row) pairs have no tap at all
   const bool mellin_wide = kind_x == AX_MCORR && c_in >= 16 && 8 * nhx <= 7 * ngx;
-  if ((c_in >= 16 && !mellin_wide) || nfx < 2) return false;
+  // ... or when p > 0 and the first pass can run as a launch per filter row
+  // (plan_first_pass_rows: no product without a tap, where the gather form multiplies a
+  // virtual row of zeros for each), given enough products per word of Y to pay for writing
+  // and reading it: c_out * nfy from 256 on (measured on the 10-layer stack: 644 -> 594 us at
+  // 256, 1157 -> 795 at 512, 3479 -> 1442 at 1024; 370 -> 451 at 128), in half precision,
+  // where the gather form is three times faster and Y is still fp32, from 1024 on
+  // (900 -> 744 us; 458 -> 570 at 512)
+  const bool mellin_rows = kind_x == AX_MCORR && c_in >= 16 && px >= 1 && c_out * nfy >= (half ? 1024 : 256);
+  if ((c_in >= 16 && !mellin_wide && !mellin_rows) || nfx < 2) return false;
   if ((double)batch * m2 * nhx * ngy * 4.0 > (double)kMaxWorkspaceBytes) return false;
   const i64 pad = ((m2 + 31) / 32) * 32;
   if (pad * 2 > m2 * 3) return false;
@@ -379,6 +463,8 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   tp.ws_bytes = (size_t)(batch * m2 * nhx * ngy) * sizeof(float);
   tp.frag_bytes = tile_fragment_bytes(tp.plan, tp.mt);
   tp.frag_off = (tp.ws_bytes + 255) & ~(size_t)255;
+  if (kind_x == AX_MCORR) plan_first_pass_rows(pr, c_in, nfx, nfy, nhx, ngx, ngy, sx, dx, px, ux, tp);
+  if (c_in >= 16 && !mellin_wide && tp.rows == 0) return false;
   if (tp.frag_bytes) tp.ws_bytes = tp.frag_off + tp.frag_bytes;
   return true;
 }
@@ -487,12 +573,9 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
     }
     if (which == IN_TWO_PASS) {
       const TwoPassInput &tp = ips.two;
-      g_variant = "mfma+fold";
-      g_last_math = tp.plan.split ? MATH_BF16X3 : MATH_FP32;
-      hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight,
-                                      (const float *)grad_out, nullptr, (float *)workspace,
-                                      (hipStream_t)stream,
-                                      tp.frag_bytes ? (float *)((char *)workspace + tp.frag_off) : nullptr);
+      g_variant = tp.rows ? "mfma-filter-rows+fold" : "mfma+fold";
+      g_last_math = tp.rows || tp.plan.split ? MATH_BF16X3 : MATH_FP32;
+      hipError_t e = launch_first_pass(tp, weight, grad_out, workspace, 4, (hipStream_t)stream);
       if (e == hipSuccess)
         e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)workspace,
                           (float *)grad_input, (hipStream_t)stream);
@@ -969,10 +1052,9 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
       if (!grad_input || !weight || !grad_out) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
       char *ws = (char *)workspace;
       hipStream_t st = (hipStream_t)stream;
-      g_variant = "mfma-f16+fold";
+      g_variant = tp.rows ? "mfma-f16-filter-rows+fold" : "mfma-f16+fold";
       g_last_math = MELLIN_MATH_F16;
-      hipError_t e = launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight, (const float *)grad_out,
-                                      nullptr, (float *)ws, st, tp.frag_bytes ? (float *)(ws + tp.frag_off) : nullptr);
+      hipError_t e = launch_first_pass(tp, weight, grad_out, ws, 2, st);
       if (e == hipSuccess) e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)ws, (float *)(ws + gi_off), st);
       if (e == hipSuccess) e = launch_float_to_half((const float *)(ws + gi_off), grad_input, n_in, st);
       return check_hip(e, __func__);

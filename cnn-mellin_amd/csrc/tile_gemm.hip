@@ -793,15 +793,15 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     pl.f_bytes = (unsigned)f_extent;
   } else if (pr.math != MATH_FP32 && f_extent <= ((i64)1 << 30)) {
     const i64 item_cap = (2 * kThreads * 8) / M_T;         // taps per chunk the two items per thread cover
-    if (single) {
-      const i64 kc16 = ((pl.C * pl.nf + 15) / 16) * 16;
-      if (split_lds(2, pl.C, true) <= 79 * 1024) {
-        pl.split = 1;
-        pl.KC16 = (int)kc16;
-        *lds_bytes = split_lds(2, pl.C, true);
-      }
+    // (a layer that fits whole as fp32 words but not with its fragments: in chunks when the
+    // bf16 form is asked for by name, else it stays on the fp32 instructions)
+    const bool whole_split = single && split_lds(2, pl.C, true) <= 79 * 1024;
+    if (whole_split) {
+      pl.split = 1;
+      pl.KC16 = (int)(((pl.C * pl.nf + 15) / 16) * 16);
+      *lds_bytes = split_lds(2, pl.C, true);
     } else if (pr.math == MATH_BF16X3_ALWAYS ||
-               (double)pr.batch * (double)Q * (double)pr.c_out * (double)pr.c_in * (double)nf >= 8e8) {
+               (!single && (double)pr.batch * (double)Q * (double)pr.c_out * (double)pr.c_in * (double)nf >= 8e8)) {
       // (layers under 0.8 GMAC (virtual rows counted) stay on the fp32 instructions: config 2's 1-D Mellin layers,
       // 0.12-0.52 GMAC, measured 25-60 % slower with fragments staged per chunk)
       // chunks: the largest that fits the LDS of a workgroup (two to a CU with two position
@@ -827,7 +827,8 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
         pl.KC16 = (int)(((best * pl.nf + 15) / 16) * 16);
         pl.KCp = ((pl.CC * pl.nf + 1) / 2) * 2;
         pl.WSS = pl.KCp + 1;
-        *lds_bytes = split_lds(2, best, pl.CC >= pl.C);
+        single = pl.CC >= pl.C;
+        *lds_bytes = split_lds(2, best, single);
       }
     }
     if (pl.split) pl.f_bytes = (unsigned)f_extent;

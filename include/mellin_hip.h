@@ -221,8 +221,9 @@ int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input,
  * kernel (variant "mfma-f16"; the input gradient of layers with at most three
  * input channels and a linear x axis through the one-kernel form,
  * "mfma-f16-fused"; with few input channels otherwise, or on a Mellin axis that
- * keeps fewer rows than it is given, as two passes, "mfma-f16+fold", whose
- * intermediate rows and folded result are fp32),
+ * keeps fewer rows than it is given, as two passes, "mfma-f16+fold" or
+ * "mfma-f16-filter-rows+fold", whose intermediate rows and folded result are
+ * fp32),
  * the weight gradient through a kernel of its own whose matrix instructions run
  * along the output positions ("mfma-f16"; partial sums in fp32, added in a fixed
  * order).  Scratch memory then holds what those kernels need (the filter cut into
@@ -400,14 +401,16 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
  * output positions, bf16 matrix cores), "mfma-fused"
  * (one-kernel input gradient, linear x axis, few input channels),
  * "mfma-taps+fold" (tap products + gather, few input channels), "mfma+fold"
- * (two-pass input gradient), "mfma-classes" (a layer on a Mellin axis as one
+ * (two-pass input gradient), "mfma-filter-rows+fold" (the same on a Mellin axis
+ * with p > 0, the first pass as a launch per filter row over the rows of
+ * grad_out that have a tap of that filter row), "mfma-classes" (a layer on a Mellin axis as one
  * launch of the tiled kernel per residue class of the axis: rows with the same
  * (h + s) mod (p + 1) have taps for the same filter rows, so no launch meets a
  * (row, filter row) pair without a tap), "mfma-f16", "mfma-f16-classes" (the
  * classes of a half-precision layer sharing one launch) and
  * "mfma-f16-class-launches" (a launch each),
- * "mfma-f16-fused" and "mfma-f16+fold" (half-precision tensors on the f16
- * matrix cores). */
+ * "mfma-f16-fused", "mfma-f16+fold" and "mfma-f16-filter-rows+fold"
+ * (half-precision tensors on the f16 matrix cores). */
 const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).
@@ -441,7 +444,10 @@ int mellin_last_math(void);
  * "widen" = automatic choice, but the half-precision entry points always go
  * through fp32 copies of their operands (for comparisons); "one-launch" /
  * "classes" = automatic choice, but layers on a Mellin axis never / whatever
- * their size run per residue class (for comparisons and tests; "class-launches":
+ * their size run per residue class ("one-launch" also keeps the first pass of a
+ * two-pass input gradient in one launch, and input gradients that would take two
+ * passes only for the launches per filter row in the gather form; for comparisons
+ * and tests; "class-launches":
  * like "classes", with a launch per class also where one launch would hold them).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);

@@ -65,7 +65,7 @@ def test_with_and_without_scratch_memory(case):
     gi_ws = torch.full(x.shape, float("nan"), device="cuda")
     hip.corr2d_backward_input(kind, wg, gog, gi_ws, dims)
     variant = hip.last_variant()
-    assert variant in ("mfma", "mfma+fold") and hip.last_math() == hip.MATH_BF16X3
+    assert variant in ("mfma", "mfma+fold", "mfma-filter-rows+fold") and hip.last_math() == hip.MATH_BF16X3
     if variant == "mfma":
         gi_plain = torch.full(x.shape, float("nan"), device="cuda")
         rc = hip.lib.mellin_corr2d_backward_input_f32(kind, hip._dp(wg), hip._dp(gog), *dims, hip._dp(gi_plain),

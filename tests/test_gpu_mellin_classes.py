@@ -124,6 +124,86 @@ def test_large_forward_passes_take_the_classes_by_default():
     assert bool(((got - ref).abs() <= 1e-5 * ref.abs() + 1e-5 * (c_in * 16) ** 0.5).all())
 
 
+# Input gradients in two passes (layers that keep fewer rows than they are given): the first
+# pass as a launch per filter row, each over the rows of grad_out that have a tap of it.
+ROW_CASES = [
+    # (n, c_in, c_out, nf, ng, s, d, p, r): steps 3, 1, 3 (the wide benchmark layer in small)
+    (2, 64, 40, (3, 3), (60, 9), (1, 1), (2, 1), (2, 1), (0, 0)),
+    # steps 2, 1, 2, 1 and rows past the support (taps beyond grad_input)
+    (2, 128, 32, (4, 4), (80, 5), (1, 1), (1, 1), (1, 1), (5, 0)),
+    # p + 1 = 4: steps 4, 2, 4, 1, 4, 2; stride 2
+    (1, 96, 33, (6, 2), (90, 7), (2, 1), (1, 1), (3, 0), (0, 0)),
+    # p + 1 = 6: steps 6, 3, 2, 3, 6, 1, 6, 3
+    (2, 64, 16, (8, 1), (120, 6), (1, 1), (1, 1), (5, 0), (0, 0)),
+    # 1-D, dilation 3 with p + 1 = 3: steps 1, 3, 3, 1
+    (3, 64, 20, (4, 1), (100, 1), (1, 1), (3, 1), (2, 0), (0, 0)),
+    # layers that keep their rows, as in the 10-layer stack: the form from 256 products per
+    # first-pass word on (c_out * nfy), in half precision from 1024 on
+    (2, 64, 64, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
+    (1, 32, 256, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
+]
+
+
+def _row_case(case, seed):
+    import mconv
+    n, c_in, c_out, nf, ng, s, d, p, r = case
+    nh = (mconv.mcorr_valid_size(nf[0], ng[0], s[0], d[0], p[0], 1) + r[0],
+          mconv.lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], 1) + r[1])
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((c_out, c_in) + nf) * (c_out * nf[0] * nf[1]) ** -0.5).astype(np.float32)
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    return nh, w, go, hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, (1, 1))
+
+
+@pytest.mark.parametrize("case", ROW_CASES, ids=[str(i) for i in range(len(ROW_CASES))])
+def test_first_pass_per_filter_row_matches_checker(case):
+    n, c_in, c_out, nf, ng, s, d, p, r = case
+    nh, w, go, dims = _row_case(case, 3100 + ROW_CASES.index(case))
+    x0 = np.zeros((n, c_in) + ng)
+    egi, _, _ = oracle.mcorrlcorr_backward(x0, w.astype(np.float64), go.astype(np.float64), s, d, p, (1, 1))
+    gi = torch.full((n, c_in) + ng, float("nan"), device="cuda")
+    hip.corr2d_backward_input(hip.AX_MCORR, to_gpu(w), to_gpu(go), gi, dims)
+    assert hip.last_variant() == "mfma-filter-rows+fold" and hip.last_math() == hip.MATH_BF16X3
+    assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input %s" % (case,))
+    # the single launch sums the same products in the same order
+    hip.set_variant("one-launch")
+    try:
+        ref = torch.full_like(gi, float("nan"))
+        hip.corr2d_backward_input(hip.AX_MCORR, to_gpu(w), to_gpu(go), ref, dims)
+        assert hip.last_variant() == ("mfma+fold" if 8 * nh[0] <= 7 * ng[0] else "mfma")
+    finally:
+        hip.set_variant(None)
+    if hip.last_math() == hip.MATH_BF16X3 and hip.last_variant() == "mfma+fold":
+        assert torch.equal(gi, ref)
+
+
+@pytest.mark.parametrize("case", ROW_CASES, ids=[str(i) for i in range(len(ROW_CASES))])
+def test_half_first_pass_per_filter_row(case):
+    n, c_in, c_out, nf, ng, s, d, p, r = case
+    nh, w, go, dims = _row_case(case, 3200 + ROW_CASES.index(case))
+    wh, goh = torch.from_numpy(w).half().cuda(), torch.from_numpy(go).half().cuda()
+    gi = torch.full((n, c_in) + ng, float("nan"), dtype=torch.float16, device="cuda")
+    hip.corr2d_backward_input(hip.AX_MCORR, wh, goh, gi, dims)
+    if 8 * nh[0] > 7 * ng[0] and c_out * nf[1] < 1024:
+        assert hip.last_variant() == "mfma-f16"                               # the gather form
+        return
+    assert hip.last_variant() == "mfma-f16-filter-rows+fold"
+    hip.set_variant("one-launch")
+    try:
+        ref = torch.full_like(gi, float("nan"))
+        hip.corr2d_backward_input(hip.AX_MCORR, wh, goh, ref, dims)
+        single = hip.last_variant()
+        assert single == ("mfma-f16+fold" if 8 * nh[0] <= 7 * ng[0] else "mfma-f16")
+    finally:
+        hip.set_variant(None)
+    if single == "mfma-f16+fold":
+        assert torch.equal(gi, ref)                                           # the same sums, rounded once
+    egi, _, _ = oracle.mcorrlcorr_backward(np.zeros((n, c_in) + ng), wh.cpu().double().numpy(),
+                                           goh.cpu().double().numpy(), s, d, p, (1, 1))
+    err = (gi.double().cpu().numpy() - egi)
+    assert np.all(np.abs(err) <= 2.0 ** -10 * np.abs(egi) + 2e-5 * (c_out * nf[0] * nf[1]) ** 0.5)
+
+
 def test_some_input_gradient_took_the_classes():
     """(after the parametrized cases of this file: tests run in the order they are written)"""
     assert "mfma-classes" in seen_gi, seen_gi
