@@ -363,12 +363,18 @@ struct TwoPassInput {
 // channels, the filter and Y addressed with the filter row's offsets and the strides of the
 // (input channel, filter row) layout) multiplies nothing the fold does not read; the single
 // launch works out every (row, filter row) pair.  Taken when that saves a fifth of the
-// 32-channel row blocks or more.  `first` is the single launch's problem.
+// 32-channel row blocks or more and the layer is large enough to pay for the launches.
+// `first` is the single launch's problem.
 bool plan_first_pass_rows(const SepConv &first, i64 c_in, i64 nfx, i64 nfy, i64 nhx, i64 ngx, i64 ngy, i64 sx, i64 dx,
                           i64 px, i64 ux, TwoPassInput &tp) {
   tp.rows = 0;
   if (g_forced != 0 || g_no_classes || px < 1 || nfx < 2 || nfx > kMaxClasses) return false;
   if (!first.in_half && first.math == MATH_FP32) return false;         // (classes run on the bf16 / f16 matrix cores)
+  // (a launch and a fragment launch per filter row: layers whose whole first pass is 16 GMAC
+  // or more, unless the form is asked for by name -- a 1-D layer of 0.5 GMAC with eight filter
+  // rows measured 56 -> 159 us)
+  const double work = (double)first.batch * (double)(c_in * nfx) * (double)(nhx * ngy) * (double)first.c_in * (double)nfy;
+  if (work < 1.6e10 && !g_all_classes) return false;
   i64 lo[kMaxClasses], hi[kMaxClasses], q[kMaxClasses];
   i64 blocks = 0;
   int n = 0;

@@ -158,8 +158,7 @@ def test_wide_mellin_layers_take_the_dense_two_pass_path(case):
     exp, _, _ = oracle.mcorrlcorr_backward(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64),
                                            s, d, p, u)
     got, v = _grad_input(hip.AX_MCORR, w, go, (n, c_in) + ng, s, d, p, u, None)
-    # (with p = 3 the first pass runs as a launch per filter row, over the rows that have a tap of it)
-    assert v == ("mfma-filter-rows+fold" if WIDE_MELLIN_CASES.index(case) == 1 else "mfma+fold"), v
+    assert v == "mfma+fold", v
     assert_close(got, exp, c_out * nf[0] * nf[1], "two-pass %s" % (case,))
     other, v2 = _grad_input(hip.AX_MCORR, w, go, (n, c_in) + ng, s, d, p, u, "generic")
     assert v2 == "generic", v2

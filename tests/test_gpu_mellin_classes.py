@@ -156,7 +156,7 @@ def _row_case(case, seed):
 
 
 @pytest.mark.parametrize("case", ROW_CASES, ids=[str(i) for i in range(len(ROW_CASES))])
-def test_first_pass_per_filter_row_matches_checker(case):
+def test_first_pass_per_filter_row_matches_checker(case, classes_forced):
     n, c_in, c_out, nf, ng, s, d, p, r = case
     nh, w, go, dims = _row_case(case, 3100 + ROW_CASES.index(case))
     x0 = np.zeros((n, c_in) + ng)
@@ -172,20 +172,20 @@ def test_first_pass_per_filter_row_matches_checker(case):
         hip.corr2d_backward_input(hip.AX_MCORR, to_gpu(w), to_gpu(go), ref, dims)
         assert hip.last_variant() == ("mfma+fold" if 8 * nh[0] <= 7 * ng[0] else "mfma")
     finally:
-        hip.set_variant(None)
+        hip.set_variant("classes")
     if hip.last_math() == hip.MATH_BF16X3 and hip.last_variant() == "mfma+fold":
         assert torch.equal(gi, ref)
 
 
 @pytest.mark.parametrize("case", ROW_CASES, ids=[str(i) for i in range(len(ROW_CASES))])
-def test_half_first_pass_per_filter_row(case):
+def test_half_first_pass_per_filter_row(case, classes_forced):
     n, c_in, c_out, nf, ng, s, d, p, r = case
     nh, w, go, dims = _row_case(case, 3200 + ROW_CASES.index(case))
     wh, goh = torch.from_numpy(w).half().cuda(), torch.from_numpy(go).half().cuda()
     gi = torch.full((n, c_in) + ng, float("nan"), dtype=torch.float16, device="cuda")
     hip.corr2d_backward_input(hip.AX_MCORR, wh, goh, gi, dims)
     if 8 * nh[0] > 7 * ng[0] and c_out * nf[1] < 1024:
-        assert hip.last_variant() == "mfma-f16"                               # the gather form
+        assert hip.last_variant() in ("mfma-f16-classes", "mfma-f16-class-launches")   # the gather form
         return
     assert hip.last_variant() == "mfma-f16-filter-rows+fold"
     hip.set_variant("one-launch")
@@ -195,13 +195,50 @@ def test_half_first_pass_per_filter_row(case):
         single = hip.last_variant()
         assert single == ("mfma-f16+fold" if 8 * nh[0] <= 7 * ng[0] else "mfma-f16")
     finally:
-        hip.set_variant(None)
+        hip.set_variant("classes")
     if single == "mfma-f16+fold":
         assert torch.equal(gi, ref)                                           # the same sums, rounded once
     egi, _, _ = oracle.mcorrlcorr_backward(np.zeros((n, c_in) + ng), wh.cpu().double().numpy(),
                                            goh.cpu().double().numpy(), s, d, p, (1, 1))
     err = (gi.double().cpu().numpy() - egi)
     assert np.all(np.abs(err) <= 2.0 ** -10 * np.abs(egi) + 2e-5 * (c_out * nf[0] * nf[1]) ** 0.5)
+
+
+def test_large_input_gradients_take_the_filter_rows_by_default():
+    """A first pass of 20 GMAC on a layer that keeps its rows: a launch per filter row, and the
+    same values as the gather form up to the order of summation."""
+    n, c_in, c_out, nf, ng, p = 16, 128, 256, (4, 4), (120, 20), (1, 1)
+    import mconv
+    nh = (mconv.mcorr_valid_size(4, 120, 1, 1, 1, 1) + 60, mconv.lcorr_valid_size(4, 20, 1, 1, 1, 1) + 2)
+    assert nh[0] == ng[0]
+    gen = torch.Generator().manual_seed(11)
+    w = (torch.randn((c_out, c_in) + nf, generator=gen) * (c_out * 16) ** -0.5).cuda()
+    go = torch.randn((n, c_out) + nh, generator=gen).cuda()
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), p, (1, 1))
+    got = torch.full((n, c_in) + ng, float("nan"), device="cuda")
+    hip.corr2d_backward_input(hip.AX_MCORR, w, go, got, dims)
+    assert hip.last_variant() == "mfma-filter-rows+fold" and hip.last_math() == hip.MATH_BF16X3
+    hip.set_variant("one-launch")
+    try:
+        ref = torch.full_like(got, float("nan"))
+        hip.corr2d_backward_input(hip.AX_MCORR, w, go, ref, dims)
+        assert hip.last_variant() == "mfma"
+    finally:
+        hip.set_variant(None)
+    assert bool(((got - ref).abs() <= 1e-5 * ref.abs() + 1e-5 * (c_out * 16) ** 0.5).all())
+    # half precision: 1024 products per first-pass word
+    gh = torch.full((n, c_in) + ng, float("nan"), dtype=torch.float16, device="cuda")
+    hip.corr2d_backward_input(hip.AX_MCORR, w.half(), go.half(), gh, dims)
+    assert hip.last_variant() == "mfma-f16-filter-rows+fold"
+    ref16 = torch.full_like(gh, float("nan"))
+    hip.set_variant("one-launch")
+    try:
+        hip.corr2d_backward_input(hip.AX_MCORR, w.half(), go.half(), ref16, dims)
+        assert hip.last_variant() == "mfma-f16"
+    finally:
+        hip.set_variant(None)
+    tol = 2.0 ** -10 * ref16.float().abs() + 2e-5 * (c_out * 16) ** 0.5
+    assert bool(((gh.float() - ref16.float()).abs() <= tol).all())
 
 
 def test_some_input_gradient_took_the_classes():
