@@ -1021,7 +1021,7 @@ size_t mellin_corr2d_backward_input_f16_workspace(int kind_x, MELLIN_CORR2D_DIMS
   // (the two-pass form where the fp32 path would take it: few input channels, or a Mellin
   // axis that keeps fewer rows than it is given)
   TwoPassInput tp;
-  if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) return align256(tp.ws_bytes) + (size_t)n_in * 4;
+  if (plan_half_two_pass(kind_x, CORR2D_ARGS, tp)) return tp.ws_bytes;
   if (c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
     return hn.frag_bytes;
   return half_layout(n_w, n_out, 0, n_in, mellin_corr2d_backward_input_workspace(kind_x, 4, CORR2D_ARGS)).total;
@@ -1050,9 +1050,9 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
     if (!two_pass && c_in >= kHalfGatherMinChannels && plan_half_native(input_gather_problem(kind_x, CORR2D_ARGS), hn))
       return run_half_native(__func__, hn, weight, grad_out, nullptr, grad_input, workspace, workspace_bytes, stream);
     if (two_pass) {
-      // the two-pass form on the half-precision tensors: first-pass rows and the folded
-      // result in fp32 in the workspace, one rounding on the way out
-      const size_t gi_off = align256(tp.ws_bytes), need = gi_off + (size_t)n_in * 4;
+      // the two-pass form on the half-precision tensors: first-pass rows in fp32 in the
+      // workspace, the fold sums them in fp32 and rounds once on the way out
+      const size_t need = tp.ws_bytes;
       if (!workspace || workspace_bytes < need)
         return fail(MELLIN_ERR_WORKSPACE, "%s: needs %zu bytes of workspace, got %zu", __func__, need, workspace_bytes);
       if (!grad_input || !weight || !grad_out) return fail(MELLIN_ERR_ARGUMENT, "%s: null pointer", __func__);
@@ -1061,8 +1061,7 @@ int mellin_corr2d_backward_input_f16(int kind_x, const void *weight, const void 
       g_variant = tp.rows ? "mfma-f16-filter-rows+fold" : "mfma-f16+fold";
       g_last_math = MELLIN_MATH_F16;
       hipError_t e = launch_first_pass(tp, weight, grad_out, ws, 2, st);
-      if (e == hipSuccess) e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)ws, (float *)(ws + gi_off), st);
-      if (e == hipSuccess) e = launch_float_to_half((const float *)(ws + gi_off), grad_input, n_in, st);
+      if (e == hipSuccess) e = launch_fold_x(tp.fold, batch * c_in, ngx, ngy, (const float *)ws, grad_input, st, true);
       return check_hip(e, __func__);
     }
   }

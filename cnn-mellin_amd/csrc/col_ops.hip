@@ -48,8 +48,9 @@ __global__ __launch_bounds__(256) void spec2col_kernel(const T *__restrict__ g, 
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void col2spec_kernel(const T *__restrict__ gg, T *__restrict__ g,
+// O: the type g is stored in (sums are formed in T)
+template <typename T, typename O = T>
+__global__ __launch_bounds__(256) void col2spec_kernel(const T *__restrict__ gg, O *__restrict__ g,
                                                        Axis x, Axis y, i64 c_in, i64 batch,
                                                        int transposed_g, int transposed_gg) {
   // x, y: convolution-kind axes with nf = taps, ng = column extent, nh = signal extent
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(256) void col2spec_kernel(const T *__restrict__ gg,
         if (oy >= 0) acc += src[((fx * y.nf + fy) * x.ng + ox) * y.ng + oy];
       }
     }
-    g[i] = acc;
+    g[i] = (O)acc;
   }
 }
 
@@ -117,8 +118,8 @@ __global__ __launch_bounds__(256) void spec2col_plane_kernel(const T *__restrict
 // once per thread; for a filter row with a tap, the loads of four filter columns of all eight
 // pairs are requested before the first is summed (positions without a tap read a word that is
 // there and add zero), so a thread waits for memory once per filter row, not once per tap.
-template <typename T>
-__global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict__ gg, T *__restrict__ g,
+template <typename T, typename O = T>
+__global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict__ gg, O *__restrict__ g,
                                                              Axis x, Axis y, int c_in, int batch,
                                                              int transposed_g, int transposed_gg,
                                                              i64 per_pair) {   // words from one pair's columns to the next
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
-      if (nc0 + b < pairs) g[(i64)(nc0 + b) * plane + q] = acc[b];
+      if (nc0 + b < pairs) g[(i64)(nc0 + b) * plane + q] = (O)acc[b];
   }
 }
 
@@ -224,20 +225,20 @@ hipError_t launch_spec2col(const Axis &x, const Axis &y, i64 c_in, i64 batch, in
   return hipGetLastError();
 }
 
-template <typename T>
+template <typename T, typename O>
 hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
-                           int transposed_gg, const T *gg, T *g, hipStream_t stream) {
+                           int transposed_gg, const T *gg, O *g, hipStream_t stream) {
   const i64 total = batch * c_in * x.nh * y.nh;
   if (total == 0) return hipSuccess;
   const i64 plane = x.nh * y.nh;
   if (fits_plane_kernels(x, y, c_in, batch, plane, x.nf * y.nf * x.ng * y.ng)) {
     const i64 gx = (plane + 255) / 256, groups = (batch * c_in + 7) / 8;
     const i64 gz = std::max<i64>(1, std::min<i64>(groups, std::min<i64>(65535, (8192 + gx - 1) / gx)));
-    hipLaunchKernelGGL(col2spec_plane_kernel<T>, dim3((unsigned)gx, 1, (unsigned)gz), dim3(256), 0, stream, gg,
+    hipLaunchKernelGGL((col2spec_plane_kernel<T, O>), dim3((unsigned)gx, 1, (unsigned)gz), dim3(256), 0, stream, gg,
                        g, x, y, (int)c_in, (int)batch, transposed_g, transposed_gg, x.nf * y.nf * x.ng * y.ng);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(col2spec_kernel<T>, dim3(blocks_for(total)), dim3(256), 0, stream, gg, g, x, y, c_in,
+  hipLaunchKernelGGL((col2spec_kernel<T, O>), dim3(blocks_for(total)), dim3(256), 0, stream, gg, g, x, y, c_in,
                      batch, transposed_g, transposed_gg);
   return hipGetLastError();
 }
@@ -260,9 +261,11 @@ template hipError_t launch_spec2col<float>(const Axis &, const Axis &, i64, i64,
                                            float *, hipStream_t);
 template hipError_t launch_spec2col<double>(const Axis &, const Axis &, i64, i64, int, int, const double *,
                                             double *, hipStream_t);
-template hipError_t launch_col2spec<float>(const Axis &, const Axis &, i64, i64, int, int, const float *,
-                                           float *, hipStream_t);
-template hipError_t launch_col2spec<double>(const Axis &, const Axis &, i64, i64, int, int, const double *,
-                                            double *, hipStream_t);
+template hipError_t launch_col2spec<float, float>(const Axis &, const Axis &, i64, i64, int, int, const float *,
+                                                  float *, hipStream_t);
+template hipError_t launch_col2spec<float, _Float16>(const Axis &, const Axis &, i64, i64, int, int, const float *,
+                                                     _Float16 *, hipStream_t);
+template hipError_t launch_col2spec<double, double>(const Axis &, const Axis &, i64, i64, int, int, const double *,
+                                                    double *, hipStream_t);
 
 }  // namespace mellin

@@ -115,12 +115,13 @@ hipError_t launch_fold_xy(const Axis &x, const Axis &y, i64 batch_cin, int nf_pa
 }
 
 hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
-                         float *grad_input, hipStream_t stream) {
+                         void *grad_input, hipStream_t stream, bool half_out) {
   // x: convolution-kind axis with nf = nfx, ng = nhx (rows of Y), nh = ngx (rows of grad_input);
   // Y is (batch_cin, nfx, 1, nhx, ngy): columns with an identity y axis
   (void)ngx;
   const Axis y = make_axis(AX_LCONV, 1, ngy, ngy, 1, 1, 0, 1);
-  return launch_col2spec<float>(x, y, batch_cin, 1, 0, 0, Y, grad_input, stream);
+  if (half_out) return launch_col2spec<float, _Float16>(x, y, batch_cin, 1, 0, 0, Y, (_Float16 *)grad_input, stream);
+  return launch_col2spec<float, float>(x, y, batch_cin, 1, 0, 0, Y, (float *)grad_input, stream);
 }
 
 }  // namespace mellin

@@ -127,15 +127,17 @@ template <typename T>
 hipError_t launch_sepreduce_generic(const SepReduce &pr, const T *a, const T *g,
                                     T *w, hipStream_t stream);
 
+// (half_out: grad_input is half-precision storage, each fp32 sum rounded once)
 hipError_t launch_fold_x(const Axis &x, i64 batch_cin, i64 ngx, i64 ngy, const float *Y,
-                         float *grad_input, hipStream_t stream);
+                         void *grad_input, hipStream_t stream, bool half_out = false);
 
 template <typename T>
 hipError_t launch_spec2col(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
                            int transposed_gg, const T *g, T *gg, hipStream_t stream);
-template <typename T>
+// (O: the type g is stored in; sums are formed in T)
+template <typename T, typename O = T>
 hipError_t launch_col2spec(const Axis &x, const Axis &y, i64 c_in, i64 batch, int transposed_g,
-                           int transposed_gg, const T *gg, T *g, hipStream_t stream);
+                           int transposed_gg, const T *gg, O *g, hipStream_t stream);
 
 bool launch_col2spec_padded(const Axis &x, const Axis &y, i64 pairs, i64 taps_padded, const float *gg,
                             float *g, hipStream_t stream, hipError_t *err);

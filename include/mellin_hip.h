@@ -222,8 +222,8 @@ int mellin_corr2d_forward_ws_f32(int kind_x, int activation, const float *input,
  * input channels and a linear x axis through the one-kernel form,
  * "mfma-f16-fused"; with few input channels otherwise, or on a Mellin axis that
  * keeps fewer rows than it is given, as two passes, "mfma-f16+fold" or
- * "mfma-f16-filter-rows+fold", whose intermediate rows and folded result are
- * fp32),
+ * "mfma-f16-filter-rows+fold", whose intermediate rows are fp32 and whose fold
+ * rounds each fp32 sum to half once),
  * the weight gradient through a kernel of its own whose matrix instructions run
  * along the output positions ("mfma-f16"; partial sums in fp32, added in a fixed
  * order).  Scratch memory then holds what those kernels need (the filter cut into
