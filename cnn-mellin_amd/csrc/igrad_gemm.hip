@@ -633,32 +633,41 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
           int hxr, hy;
           by_nhy.divmod(rel, hxr, hy);
           float *dst = myplane + pl.sx * hxr * pl.Wp + pl.sy * hy;
+          // One filter column at a time (neighbouring positions share words across columns; the
+          // four columns of a filter row sit at fixed distances from the first).  The images of
+          // the input channels are different memory: their words of a column are read together,
+          // added and written together, so that a tile's fold waits for LDS once per filter
+          // column and not once per column and channel.
+          if (quad) {
+            float *pj[MTT][4];
+#pragma unroll
+            for (int a = 0; a < MTT; ++a)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) pj[a][j] = dst + a * wplane_words + off[4 * j];
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+              float v[MTT][4];
+#pragma unroll
+              for (int a = 0; a < MTT; ++a)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[a][j] = pj[a][j][c4];
+#pragma unroll
+              for (int a = 0; a < MTT; ++a)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) pj[a][j][c4] = v[a][j] + acc[a][t][4 * j + c4];
+            }
+            continue;
+          }
 #pragma unroll
           for (int a = 0; a < MTT; ++a) {
             float *pa = dst + a * wplane_words;
-            if (quad) {
-              // (one filter column at a time, as below: neighbouring positions share words across
-              // columns; the four columns of a filter row sit at fixed distances from the first)
-              float *pj[4];
 #pragma unroll
-              for (int j = 0; j < 4; ++j) pj[j] = pa + off[4 * j];
+            for (int c4 = 0; c4 < 4; ++c4) {
+              float v[4];
 #pragma unroll
-              for (int c4 = 0; c4 < 4; ++c4) {
-                float v[4];
+              for (int j = 0; j < 4; ++j) v[j] = pa[off[4 * j + c4]];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = pj[j][c4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) pj[j][c4] = v[j] + acc[a][t][4 * j + c4];
-              }
-            } else {
-#pragma unroll
-              for (int c4 = 0; c4 < 4; ++c4) {
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = pa[off[4 * j + c4]];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) pa[off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
-              }
+              for (int j = 0; j < 4; ++j) pa[off[4 * j + c4]] = v[j] + acc[a][t][4 * j + c4];
             }
           }
         }
