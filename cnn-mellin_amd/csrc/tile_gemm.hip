@@ -274,7 +274,7 @@ __device__ __forceinline__ void tile_gemm_body(
         // channels: such a tap reads the lane's first word, always a staged one, and
         // meets a zero weight)
         const bool whole = k < pl.CC * pl.nf, last = k < cc_last * pl.nf;
-        const int fo = (cl * pl.f_c + class_filter_row(pl.cls_fx, fx) * pl.nfy + fy) * EB;   // (the layer's filter row)
+        const int fo = (cl * pl.f_c + class_filter_row(pl.cls_fx, fx) * pl.f_pitch + pl.f_off + fy) * EB;   // (the layer's filter row and column)
         tapoff[k] = whole ? off : 0;
         tapoff[pl.KC16 + k] = last ? off : 0;
         tapoff[2 * pl.KC16 + k] = whole ? fo : (int)kDeadOffset;
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int 
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int k = 8 * g + i, cl = k / pl.nf, t = k - cl * pl.nf;
-    const int fx = t / pl.nfy, ta = class_filter_row(pl.cls_fx, fx) * pl.nfy + (t - fx * pl.nfy);   // the layer's tap
+    const int fx = t / pl.nfy, ta = class_filter_row(pl.cls_fx, fx) * pl.f_pitch + pl.f_off + (t - fx * pl.nfy);   // the layer's tap
     x[i] = (row < pl.M && k < cc * pl.nf) ? F[(i64)row * pl.f_m + (i64)(ch * pl.CC + cl) * pl.f_c + ta] : (Word)0;
   }
   if constexpr (F16) {
@@ -594,7 +594,8 @@ static int workgroups_per_cu(size_t lds_bytes, int mt, int nt, bool split) {
 
 // Fill `pl` for the problem `pr`; returns false when the tiled kernel does not
 // apply (sizes beyond 32-bit indexing or a single channel not fitting in LDS).
-bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt, int force_nt) {
+bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt, int force_nt,
+                    bool trim_columns) {
   const i64 lim = (i64)1 << 30;
   // (a residue class of a Mellin axis: the rows and filter rows of the class)
   const bool cls = pr.cls_nfx > 0;
@@ -604,7 +605,31 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   const i64 nfx_k = cls ? pr.cls_nfx : pr.x.nf;
   const i64 nox_k = cls ? std::max<i64>(0, (pr.x.nh - pr.cls_first + pr.cls_stride - 1) / pr.cls_stride) : pr.x.nh;
   const i64 nox_eff_k = cls ? std::max<i64>(0, (pr.x.nh_eff - pr.cls_first + pr.cls_stride - 1) / pr.cls_stride) : pr.x.nh_eff;
-  const i64 nf = nfx_k * pr.y.nf, ng = pr.x.ng * pr.y.ng, Q = nox_k * pr.y.nh;
+  // Filter columns with a tap inside the signal for some output column (layers on one or two
+  // frequency bins with a padded 4-wide filter: half the columns have none, and a plan that
+  // keeps them stages zeros for them and multiplies them).  Only the two ends are cut:
+  //   correlation  gy = s oy + d fy - p,   convolution  gy = s oy - d fy + p,   0 <= gy < ng
+  // over oy in [0, nh_eff); the kernel then sees columns fy_lo .. fy_hi as a filter of its own
+  // with p - d fy_lo for p.
+  i64 fy_lo = 0, fy_hi = pr.y.nf - 1;
+  if (trim_columns && pr.y.u == 1 && pr.y.nh_eff >= 1 && pr.y.d >= 1 && pr.y.nf >= 1 &&
+      (pr.y.kind == AX_LCORR || pr.y.kind == AX_LCONV)) {
+    const i64 span = pr.y.s * (pr.y.nh_eff - 1);           // s oy runs over [0, span]
+    i64 lo, hi;
+    if (pr.y.kind == AX_LCORR) {
+      lo = -floor_div(-(pr.y.p - span), pr.y.d);           // d fy - p + span >= 0
+      hi = floor_div(pr.y.ng - 1 + pr.y.p, pr.y.d);        // d fy - p <= ng - 1
+    } else {
+      lo = -floor_div(-(pr.y.p - (pr.y.ng - 1)), pr.y.d);  // -d fy + p <= ng - 1
+      hi = floor_div(pr.y.p + span, pr.y.d);               // -d fy + p + span >= 0
+    }
+    lo = std::max<i64>(lo, 0);
+    hi = std::min<i64>(hi, pr.y.nf - 1);
+    if (lo <= hi) { fy_lo = lo; fy_hi = hi; }
+  }
+  const bool trimmed = fy_lo > 0 || fy_hi < pr.y.nf - 1;
+  const i64 nfy_k = fy_hi - fy_lo + 1, py_k = pr.y.p - pr.y.d * fy_lo;
+  const i64 nf = nfx_k * nfy_k, ng = pr.x.ng * pr.y.ng, Q = nox_k * pr.y.nh;
   if (nf <= 0 || ng <= 0 || Q <= 0 || pr.c_in <= 0 || pr.c_out <= 0 || pr.batch <= 0) return false;
   if (nf > 4096 || ng >= lim || Q >= lim || pr.c_in >= lim || pr.c_out >= lim || pr.batch >= lim) return false;
   if (pr.c_in * ng >= lim * 2 || pr.batch * (Q / 64 + 1) >= lim) return false;
@@ -614,7 +639,8 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   if (Y.p > lim || Y.p < -lim || X.p < -lim) return false;
 
   pl.batch = (int)pr.batch; pl.M = (int)pr.c_out; pl.C = (int)pr.c_in;
-  pl.nfx = (int)nfx_k; pl.nfy = (int)Y.nf; pl.nf = (int)nf;
+  pl.nfx = (int)nfx_k; pl.nfy = (int)nfy_k; pl.nf = (int)nf;
+  pl.f_pitch = (int)Y.nf; pl.f_off = (int)fy_lo;
   pl.ngx = (int)X.ng; pl.ngy = (int)Y.ng; pl.nox = (int)nox_k; pl.noy = (int)Y.nh; pl.Q = (int)Q;
   pl.nox_eff = (int)nox_eff_k; pl.noy_eff = (int)Y.nh_eff;
   pl.cls_stride = cls ? pr.cls_stride : 1;
@@ -662,7 +688,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // y axis: column = ay * oy + by * fy + cy - min
   pl.ay = (int)Y.s;
   pl.by = Y.kind == AX_LCORR ? (int)Y.d : -(int)Y.d;
-  pl.cy = Y.kind == AX_LCORR ? -(int)Y.p : (int)Y.p;
+  pl.cy = Y.kind == AX_LCORR ? -(int)py_k : (int)py_k;
   const i64 by_ext = (i64)pl.by * (pl.nfy - 1);
   pl.by_min = (int)(by_ext < 0 ? by_ext : 0);
   pl.by_span = (int)(by_ext < 0 ? -by_ext : by_ext);
@@ -845,7 +871,9 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     const i64 wgs = (i64)pl.total_tiles * m_tiles;
     if (wgs > slots2 && wgs <= slots1) { pl.sbuf = 1; *lds_bytes = one; }
   }
-  if (cls && !pl.split) return false;                      // (the filter rows of a class are picked through the fragment tables)
+  // (columns, like the filter rows of a class, are picked through the fragment tables)
+  if (trimmed && !pl.split) return make_tile_plan(pr, pl, lds_bytes, mt, nt, force_nt, false);
+  if (cls && !pl.split) return false;
   return true;
 }
 

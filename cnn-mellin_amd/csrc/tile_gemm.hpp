@@ -9,6 +9,10 @@ struct TilePlan {
   // problem (all fit 32 bits; checked by make_tile_plan)
   int batch, M, C;                 // images, output channels, contracted channels
   int nfx, nfy, nf;                // filter extent and nfx * nfy
+  // The kernel's filter columns are columns f_off .. f_off + nfy - 1 of a filter whose rows
+  // are f_pitch words apart: columns none of whose taps lies inside the signal for any output
+  // column are left out of the plan (bf16 / f16 plans only; else f_off = 0, f_pitch = nfy).
+  int f_pitch, f_off;
   int ngx, ngy;                    // signal extent
   int nox, noy, Q;                 // allocated output extent and nox * noy
   int nox_eff, noy_eff;            // outputs at or past these have no tap
@@ -61,7 +65,7 @@ int mellin_classes(const Axis &x, MellinClass *out, int max_classes);
 
 // force_nt: 0 lets the plan pick the number of 32-position tiles per wavefront
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt,
-                    int force_nt = 0);
+                    int force_nt = 0, bool trim_columns = true);
 
 // Bytes of scratch memory in which a launch keeps the filter as bf16 fragments, block by
 // block as the stages read them (0: the layer does not run on the bf16 matrix cores, or
