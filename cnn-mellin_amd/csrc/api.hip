@@ -32,6 +32,7 @@ std::atomic<const char *> g_variant{""};
 std::atomic<int> g_no_classes{0};       // Mellin layers as one launch, not one per residue class (mellin_set_variant "one-launch")
 std::atomic<int> g_split_classes{0};    // ... every class a launch of its own ("class-launches": for comparisons)
 std::atomic<int> g_all_classes{0};      // ... one per class whatever the layer's size ("classes": for tests)
+std::atomic<int> g_whole_classes{0};    // ... a class's rows never cut into ranges ("whole-classes": for comparisons)
 std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
@@ -119,11 +120,12 @@ struct ClassPlans {
   size_t lds[kMaxClasses], frag_off[kMaxClasses];
   int mt[kMaxClasses], nt[kMaxClasses];
   size_t frag_bytes = 0;           // all classes' filter fragments, each region 256-byte aligned
+  bool cut = false;                // classes cut into ranges of rows (plan_mellin_classes)
 };
 
 // False: the layer stays with the single launch (one class only or too many, a class with no
 // filter row or no plan on the bf16 / f16 matrix cores, a layer too small to pay for the launches).
-bool plan_mellin_classes(const SepConv &pr, ClassPlans &cp) {
+bool plan_mellin_classes(const SepConv &pr, ClassPlans &cp, bool allow_cut = true) {
   if (g_forced != 0 || g_no_classes || pr.accumulate || pr.cls_nfx || (!pr.in_half && pr.math == MATH_FP32)) return false;
   const double work = (double)pr.batch * pr.x.nh * pr.y.nh * pr.c_out * pr.c_in * pr.x.nf * pr.y.nf;
   // (correlation axes only, i.e. forward passes: the classes of a convolution axis, six for a
@@ -133,20 +135,96 @@ bool plan_mellin_classes(const SepConv &pr, ClassPlans &cp) {
   MellinClass mc[kMaxClasses];
   const int n = mellin_classes(pr.x, mc, kMaxClasses);
   if (n < 2) return false;
-  cp.n = 0;
-  cp.frag_bytes = 0;
+  // the launches: a class, or a range of a class's rows (rows first, first + stride, ... < end)
+  struct Item { int stride, first, end, nfx; unsigned long long fx; };
+  Item items[kMaxClasses];
+  int n_items = 0;
   for (int r = 0; r < n; ++r) {
     if (mc[r].first >= pr.x.nh) continue;                   // no output row in this class
     if (mc[r].nfx == 0) return false;                       // rows that are bias alone: the single launch writes them
+    items[n_items++] = Item{mc[r].stride, mc[r].first, (int)pr.x.nh, mc[r].nfx, mc[r].fx};
+  }
+  cp.cut = false;
+  if (pr.x.kind == AX_MCORR && allow_cut && !pr.in_half && !g_whole_classes && !g_split_classes) {
+    // On a correlation axis the tap of filter row f is inside the signal for the rows up to
+    // h_f = floor((ng - 1 + u)(p + 1) / (f + d)) - s only: a layer whose output reaches past
+    // the support of its later filter rows (a stack that keeps its number of rows) stages
+    // and multiplies rows of zeros for those pairs.  A class's rows are cut at the h_f of its
+    // filter rows, each range a unit of work with the filter rows that still have taps
+    // there, when that leaves out a tenth of the (row, filter row) pairs or more and the
+    // units stay within the limit; ranges of under sixteen rows join the range before them.
+    // The units share one kernel instance and one launch (launch_mellin_classes).  fp32
+    // layers only: over the forward passes of the 10-layer stack 8.35 -> 7.44 ms (eight
+    // layers 12-21 % faster, the two 128 -> 128 layers on 10 bins 8 % slower); in half
+    // precision, where the classes share a launch already, 3.10 -> 3.06 ms with layers
+    // moving either way by up to 20 %, so half-precision classes stay whole.
+    Item cut[kMaxClasses];
+    int n_cut = 0;
+    double pairs_whole = 0, pairs_cut = 0;
+    bool ok = true;
+    for (int i = 0; i < n_items && ok; ++i) {
+      const Item &it = items[i];
+      i64 end_f[16], ends[16];
+      int n_ends = 0;
+      for (int j = 0; j < it.nfx; ++j) {
+        const i64 f = class_filter_row(it.fx, j);
+        const i64 h_f = (pr.x.ng - 1 + pr.x.u) * (pr.x.p + 1) / (f + pr.x.d) - pr.x.s;
+        end_f[j] = std::max<i64>(0, std::min<i64>(it.end, h_f + 1));
+        bool seen = false;
+        for (int e = 0; e < n_ends; ++e) seen = seen || ends[e] == end_f[j];
+        if (!seen) ends[n_ends++] = end_f[j];
+      }
+      std::sort(ends, ends + n_ends);
+      if (ends[n_ends - 1] < it.end) { ok = false; break; }           // rows past every tap: bias alone
+      pairs_whole += (double)((it.end - it.first + it.stride - 1) / it.stride) * it.nfx;
+      i64 lo = 0;
+      const int first_of_class = n_cut;
+      for (int e = 0; e < n_ends; ++e) {
+        const i64 hi = ends[e];
+        // the class's first row at or after lo
+        const i64 first = lo <= it.first ? it.first : it.first + (lo - it.first + it.stride - 1) / it.stride * it.stride;
+        const i64 rows = first < hi ? (hi - first + it.stride - 1) / it.stride : 0;
+        if (rows == 0) continue;
+        if (rows < 16 && n_cut > first_of_class) {                    // joins the range before it (a superset of its filter rows)
+          pairs_cut += (double)rows * cut[n_cut - 1].nfx;
+          cut[n_cut - 1].end = (int)hi;
+          lo = hi;
+          continue;
+        }
+        if (n_cut == kMaxClasses) { ok = false; break; }
+        Item c{it.stride, (int)first, (int)hi, 0, 0};
+        for (int j = 0; j < it.nfx; ++j)
+          if (end_f[j] >= hi) c.fx |= (unsigned long long)class_filter_row(it.fx, j) << (4 * c.nfx++);
+        pairs_cut += (double)rows * c.nfx;
+        cut[n_cut++] = c;
+        lo = hi;
+      }
+    }
+    if (ok && n_cut > n_items && pairs_cut <= 0.9 * pairs_whole) {
+      n_items = n_cut;
+      for (int i = 0; i < n_cut; ++i) items[i] = cut[i];
+      cp.cut = true;
+    }
+  }
+  cp.n = 0;
+  cp.frag_bytes = 0;
+  for (int r = 0; r < n_items; ++r) {
     SepConv c = pr;
-    c.cls_stride = mc[r].stride; c.cls_first = mc[r].first; c.cls_nfx = mc[r].nfx; c.cls_fx = mc[r].fx;
+    c.cls_stride = items[r].stride; c.cls_first = items[r].first; c.cls_nfx = items[r].nfx; c.cls_fx = items[r].fx;
+    c.x.nh = items[r].end;
+    c.x.nh_eff = std::min<i64>(pr.x.nh_eff, items[r].end);
     if (!c.in_half) c.math = MATH_BF16X3_ALWAYS;
     const int i = cp.n;
-    if (!make_tile_plan(c, cp.pl[i], &cp.lds[i], &cp.mt[i], &cp.nt[i])) return false;
+    // (ranges of one layer share the tile shape of the first: one kernel instance for all)
+    if (!make_tile_plan(c, cp.pl[i], &cp.lds[i], &cp.mt[i], &cp.nt[i], cp.cut && i > 0 ? cp.nt[0] : 0, true,
+                        cp.cut && i > 0 ? cp.mt[0] : 0))
+      return cp.cut ? plan_mellin_classes(pr, cp, false) : false;
     cp.frag_off[i] = cp.frag_bytes;
     cp.frag_bytes += (tile_fragment_bytes(cp.pl[i], cp.mt[i]) + 255) & ~(size_t)255;
     ++cp.n;
   }
+  // (ranges are worth their number only as one launch)
+  if (cp.cut && !tile_classes_fit_one_launch(cp.pl, cp.mt, cp.nt, cp.n)) return plan_mellin_classes(pr, cp, false);
   return cp.n >= 2;
 }
 
@@ -160,7 +238,7 @@ hipError_t launch_mellin_classes(const ClassPlans &cp, const void *f, const void
   // of the 10-layer stack than a launch per class: no gaps, the chip shared by the work of the
   // classes); in fp32, where a class's launch is long enough to fill the chip by itself, a
   // launch per class was the faster by 5 %.
-  if (!g_split_classes && cp.pl[0].f16 && use_ws && tile_classes_fit_one_launch(cp.pl, cp.mt, cp.nt, cp.n)) {
+  if (!g_split_classes && (cp.pl[0].f16 || cp.cut) && use_ws && tile_classes_fit_one_launch(cp.pl, cp.mt, cp.nt, cp.n)) {
     if (one_launch) *one_launch = true;
     return launch_tile_gemm_classes(cp.pl, cp.lds, cp.n, cp.mt[0], cp.nt[0], (const float *)f, (const float *)g,
                                     (const float *)bias, (float *)h, stream, use_ws ? (float *)frag_ws : nullptr,
@@ -181,7 +259,11 @@ hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
                               size_t frag_bytes) {
   {
     ClassPlans cp;
-    if (plan_mellin_classes(pr, cp)) {
+    bool classes = plan_mellin_classes(pr, cp);
+    // (ranges need the scratch memory for their fragments: without it, whole classes)
+    if (classes && cp.cut && !(frag_ws && ((uintptr_t)frag_ws & 15) == 0 && frag_bytes >= cp.frag_bytes))
+      classes = plan_mellin_classes(pr, cp, false);
+    if (classes) {
       g_variant = "mfma-classes";
       g_last_math = MATH_BF16X3;
       return launch_mellin_classes(cp, f, g, bias, h, stream, frag_ws, frag_bytes);
@@ -422,7 +504,7 @@ hipError_t launch_first_pass(const TwoPassInput &tp, const void *weight, const v
     const i64 fx = tp.row_fx[i];
     float *af = tile_fragment_bytes(pl, tp.row_mt[i]) ? (float *)((char *)frag + tp.row_frag_off[i]) : nullptr;
     hipError_t e = launch_tile_gemm(pl, tp.row_lds[i], tp.row_mt[i], tp.row_nt[i],
-                                    (const float *)((const char *)weight + fx * pl.nfy * elem_bytes),
+                                    (const float *)((const char *)weight + fx * pl.f_pitch * elem_bytes),
                                     (const float *)grad_out, nullptr, (float *)ws + fx * pl.ngx * pl.noy, stream, af);
     if (e != hipSuccess) return e;
   }
@@ -1224,11 +1306,13 @@ int mellin_last_math(void) { return g_last_math; }
 int mellin_set_variant(const char *name) {
   const bool widen = name && !strcmp(name, "widen"), one = name && !strcmp(name, "one-launch");
   const bool all = name && !strcmp(name, "classes"), each = name && !strcmp(name, "class-launches");
+  const bool whole = name && !strcmp(name, "whole-classes");
   g_widen = widen;
   g_no_classes = one;
   g_all_classes = all || each;
   g_split_classes = each;
-  if (!name || !*name || widen || one || all || each) { g_forced = 0; return MELLIN_OK; }
+  g_whole_classes = whole;
+  if (!name || !*name || widen || one || all || each || whole) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
   if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }

@@ -595,7 +595,7 @@ static int workgroups_per_cu(size_t lds_bytes, int mt, int nt, bool split) {
 // Fill `pl` for the problem `pr`; returns false when the tiled kernel does not
 // apply (sizes beyond 32-bit indexing or a single channel not fitting in LDS).
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt, int force_nt,
-                    bool trim_columns) {
+                    bool trim_columns, int force_mt) {
   const i64 lim = (i64)1 << 30;
   // (a residue class of a Mellin axis: the rows and filter rows of the class)
   const bool cls = pr.cls_nfx > 0;
@@ -662,6 +662,10 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // through with a staged chunk six times sooner, so what a chunk's staging costs is spread
   // over twice the products; the accumulators fit because nothing is split in registers)
   if (pr.in_half && pr.c_out > 64 && pr.batch * ((Q + 255) / 256) * ((pr.c_out + 127) / 128) >= 256) *mt = 4;
+  if (force_mt) {
+    if ((force_mt != 1 && force_mt != 2 && force_mt != 4) || (force_mt == 4 && !pr.in_half)) return false;
+    *mt = force_mt;
+  }
   const int M_T = *mt * 32;
   const i64 m_tiles = (pr.c_out + M_T - 1) / M_T;
   // two N tiles per wavefront once that still leaves every CU several tiles (not when
@@ -872,7 +876,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     if (wgs > slots2 && wgs <= slots1) { pl.sbuf = 1; *lds_bytes = one; }
   }
   // (columns, like the filter rows of a class, are picked through the fragment tables)
-  if (trimmed && !pl.split) return make_tile_plan(pr, pl, lds_bytes, mt, nt, force_nt, false);
+  if (trimmed && !pl.split) return make_tile_plan(pr, pl, lds_bytes, mt, nt, force_nt, false, force_mt);
   if (cls && !pl.split) return false;
   return true;
 }

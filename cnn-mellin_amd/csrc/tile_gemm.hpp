@@ -64,8 +64,9 @@ struct MellinClass {
 int mellin_classes(const Axis &x, MellinClass *out, int max_classes);
 
 // force_nt: 0 lets the plan pick the number of 32-position tiles per wavefront
+// force_mt: likewise for the 32-channel tiles per workgroup (launches that share a kernel instance)
 bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt, int *nt,
-                    int force_nt = 0, bool trim_columns = true);
+                    int force_nt = 0, bool trim_columns = true, int force_mt = 0);
 
 // Bytes of scratch memory in which a launch keeps the filter as bf16 fragments, block by
 // block as the stages read them (0: the layer does not run on the bf16 matrix cores, or

@@ -447,7 +447,8 @@ int mellin_last_math(void);
  * their size run per residue class ("one-launch" also keeps the first pass of a
  * two-pass input gradient in one launch, and input gradients that would take two
  * passes only for the launches per filter row in the gather form; for comparisons
- * and tests; "class-launches":
+ * and tests; "whole-classes": automatic choice, but a class's rows are never cut
+ * into ranges by where the filter rows' taps leave the signal; "class-launches":
  * like "classes", with a launch per class also where one launch would hold them).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
 int mellin_set_variant(const char *name);

@@ -141,6 +141,9 @@ ROW_CASES = [
     # first-pass word on (c_out * nfy), in half precision from 1024 on
     (2, 64, 64, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
     (1, 32, 256, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
+    # one output column under a dilated 8-wide filter: the first pass keeps filter columns 1-4
+    # only, and the filter row's offset into the weight is still counted in whole filter rows
+    (2, 64, 130, (4, 8), (35, 8), (1, 1), (1, 2), (1, 2), (3, 1)),
 ]
 
 
