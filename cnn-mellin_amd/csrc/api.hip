@@ -32,6 +32,7 @@ std::atomic<const char *> g_variant{""};
 std::atomic<int> g_no_classes{0};       // Mellin layers as one launch, not one per residue class (mellin_set_variant "one-launch")
 std::atomic<int> g_split_classes{0};    // ... every class a launch of its own ("class-launches": for comparisons)
 std::atomic<int> g_all_classes{0};      // ... one per class whatever the layer's size ("classes": for tests)
+std::atomic<int> g_no_yfold{0};         // tap products stored per filter column, not summed over them ("tap-columns": for comparisons)
 std::atomic<int> g_whole_classes{0};    // ... a class's rows never cut into ranges ("whole-classes": for comparisons)
 std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
@@ -602,6 +603,7 @@ int choose_input_plan(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 n
   }
   if (forced == 0 && make_tap_product_plan(batch, c_in, c_out, nfx, nfy, nhx, nhy, ips.taps) &&
       ips.taps.ws_bytes <= kMaxWorkspaceBytes) {
+    if (!g_no_yfold) enable_tap_yfold(ips.taps, nfx, nfy, nhx, nhy, ngy, sy, dy, py, uy);
     ips.ws_bytes = ips.taps.ws_bytes;
     return IN_TAPS;
   }
@@ -654,8 +656,11 @@ int corr2d_backward_input(const char *fn, int kind_x, const T *weight,
       if (e == hipSuccess) {
         const Axis fx = make_axis(conv_x, nfx, nhx, ngx, ux, dx, px, sx);
         const Axis fy = make_axis(AX_LCONV, nfy, nhy, ngy, uy, dy, py, sy);
-        e = launch_fold_xy(fx, fy, batch * c_in, ips.taps.nf_pad, (const float *)workspace,
-                           (float *)grad_input, (hipStream_t)stream);
+        if (ips.taps.yfold)                                  // (the kernel has summed the filter columns)
+          e = launch_fold_x(fx, batch * c_in, ngx, ngy, (const float *)workspace, grad_input, (hipStream_t)stream);
+        else
+          e = launch_fold_xy(fx, fy, batch * c_in, ips.taps.nf_pad, (const float *)workspace,
+                             (float *)grad_input, (hipStream_t)stream);
       }
       return check_hip(e, fn);
     }
@@ -1306,13 +1311,14 @@ int mellin_last_math(void) { return g_last_math; }
 int mellin_set_variant(const char *name) {
   const bool widen = name && !strcmp(name, "widen"), one = name && !strcmp(name, "one-launch");
   const bool all = name && !strcmp(name, "classes"), each = name && !strcmp(name, "class-launches");
-  const bool whole = name && !strcmp(name, "whole-classes");
+  const bool whole = name && !strcmp(name, "whole-classes"), columns = name && !strcmp(name, "tap-columns");
   g_widen = widen;
   g_no_classes = one;
   g_all_classes = all || each;
   g_split_classes = each;
   g_whole_classes = whole;
-  if (!name || !*name || widen || one || all || each || whole) { g_forced = 0; return MELLIN_OK; }
+  g_no_yfold = columns;
+  if (!name || !*name || widen || one || all || each || whole || columns) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
   if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
   if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }

@@ -160,6 +160,27 @@ __global__ __launch_bounds__(256) void col2spec_plane_kernel(const T *__restrict
     T acc[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc[b] = T(0);
+    if (nfy == 1 && nfx <= 8) {
+      // one column per filter row (the fold over x alone): the taps of all filter rows are
+      // worked out first, then every load is requested (a row without a tap re-reads the
+      // pair's first word and adds a zero), then the sums are formed in filter-row order --
+      // one wait for memory instead of one per filter row
+      int off[8];
+#pragma unroll
+      for (int fx = 0; fx < 8; ++fx) {
+        const int ox = fx < nfx ? tap32(x.kind, gx, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u) : -1;
+        off[fx] = (ox >= 0 && oy_first[0] >= 0) ? (fx * (int)x.ng + ox) * (int)y.ng + oy_first[0] : -1;
+      }
+      T v[8][NB];
+#pragma unroll
+      for (int fx = 0; fx < 8; ++fx)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) v[fx][b] = src[b][max(off[fx], 0)];
+#pragma unroll
+      for (int fx = 0; fx < 8; ++fx)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] += off[fx] >= 0 ? v[fx][b] : T(0);
+    } else
     for (int fx = 0; fx < nfx; ++fx) {
       const int ox = tap32(x.kind, gx, fx, (int)x.ng, (int)x.s, (int)x.d, (int)x.p, (int)x.u);
       if (ox < 0) continue;

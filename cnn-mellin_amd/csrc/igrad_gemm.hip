@@ -817,7 +817,16 @@ hipError_t launch_stream_instance(const IgradPlan &pl, const void *w, const void
 // Same operands, staging and work split over wavefronts as above; the
 // accumulators are stored instead of folded.  A workgroup takes pl.cpw chunks
 // of 64 positions of pl.jobs consecutive images.
-template <int KSTEPS>
+//
+// YF (plan.yfold): a lane's registers 4 g .. 4 g + 3 are the four filter columns fy of filter
+// row fx = 2 g + (lane / 32) at the lane's position, and column fy of position q belongs to
+// grad_input column hy(q) + fy - py: the sum over fy of a grad_input column takes the value of
+// fy = k from the lane k positions back.  Positions are the flattened (hx, hy), so for the first
+// three positions of a row "k positions back" reaches into the row before: those terms are
+// that row's last three columns (nhy .. nhy + 2), and the lane stores them there.  A workgroup
+// takes whole rows and three more positions, which produce the last row's tail; the values of
+// the tile before (the three lanes a tile's first lanes reach back to) stay in registers.
+template <int KSTEPS, bool YF>
 __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan pl,
                                                           const float *__restrict__ W,
                                                           const float *__restrict__ GO,
@@ -830,18 +839,21 @@ __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan p
   const int lane = threadIdx.x & 63;
   const int tid = wave * 64 + lane, nthreads = pl.units * 64;
   const int half = lane >> 5, l32 = lane & 31;
-  const int groups_x = (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
+  const int groups_x = YF ? (pl.nhx + pl.rows_wg - 1) / pl.rows_wg : (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
   const int image_group = blockIdx.x / groups_x, chunk_group = blockIdx.x - image_group * groups_x;
   const int n_want = image_group * pl.jobs + job;
   const bool active = n_want < pl.batch;
   const int n = active ? n_want : pl.batch - 1;
-  const int c_first = chunk_group * pl.cpw;
-  const int nchunks = min(pl.cpw, pl.chunks_per_image - c_first);
+  // positions [q_lo, q_hi) in chunks of 64 from q_lo (YF: whole rows, and three positions more)
+  const int row_a = chunk_group * pl.rows_wg;
+  const int q_lo = YF ? row_a * pl.nhy : chunk_group * pl.cpw * P;
+  const int q_hi = YF ? min(pl.nhx, row_a + pl.rows_wg) * pl.nhy : pl.nh;
+  const int nchunks = YF ? (q_hi - q_lo + 3 + P - 1) / P : min(pl.cpw, pl.chunks_per_image - chunk_group * pl.cpw);
   float *Bs = lds + job * K * P;
   const unsigned bs_addr = lds_address(lds) + 4u * (unsigned)(job * K * P);
 
   // channels past c_out and positions past the image are never loaded: keep them finite
-  if ((c_first + nchunks) * P > pl.nh) {
+  if (q_lo + nchunks * P > pl.nh) {
     for (int i = tid; i < K * P; i += nthreads) Bs[i] = 0.f;
   } else {
     for (int i = pl.c_out * P + tid; i < K * P; i += nthreads) Bs[i] = 0.f;
@@ -859,9 +871,9 @@ __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan p
   const float *GOn = GO + (i64)n * pl.c_out * pl.nh;
   const int row_in = lane >> 4, seg = lane & 15;          // 16 lanes x 16 bytes per channel row
   auto issue = [&](int c, int k_lo) {                     // channels [k_lo, k_lo + KH) of chunk c
-    const int q0 = c * P;
+    const int q0 = q_lo + c * P;
     const int k_hi = min(k_lo + KH, pl.c_out);
-    if (q0 + P <= pl.nh) {
+    if (q0 + P <= pl.nh && (q0 & 3) == 0) {                // (16-byte pieces)
       for (int k0 = k_lo + wave * 4; k0 < k_hi; k0 += pl.units * 4) {
         const int k = k0 + row_in;
         const unsigned voff = (unsigned)(row_in * pl.nh + q0 + 4 * (seg ^ ((k & 1) << 3))) * 4u;
@@ -881,9 +893,17 @@ __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan p
   float *Zrow = Z + ((i64)(n * pl.c_in + ci) * pl.nf_pad + mt * 32 + half * 4) * pl.nh;
   const int m_base = mt * 32 + half * 4;
 
+  // YF: columns fy = 1, 2, 3 of the tile before (zeros at the start of the rows)
+  float prev[4][3];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int k = 0; k < 3; ++k) prev[g][k] = 0.f;
+  const FastDiv by_nhy(YF ? pl.nhy : 1);
+
   __syncthreads();
-  issue(c_first, 0);
-  issue(c_first, KH);
+  issue(0, 0);
+  issue(0, KH);
   for (int c = 0; c < nchunks; ++c) {
     wait_all_memory();
     __syncthreads();
@@ -898,18 +918,52 @@ __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan p
       for (int t = 0; t < NT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
     __syncthreads();                                   // the first half is free
-    if (c + 1 < nchunks) issue(c_first + c + 1, 0);
+    if (c + 1 < nchunks) issue(c + 1, 0);
 #pragma unroll
     for (int s = KSTEPS / 2; s < KSTEPS; ++s)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], Bs[bo[t] + 2 * s * P], acc[t], 0, 0, 0);
     __syncthreads();                                   // the second half is free
-    if (c + 1 < nchunks) issue(c_first + c + 1, KH);
-    if (active) {
+    if (c + 1 < nchunks) issue(c + 1, KH);
+    if constexpr (YF) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        const int q = (c_first + c) * P + t * 32 + l32;
+        const int q = q_lo + c * P + t * 32 + l32;
+        const bool real = q < q_hi;
+        int hx, hy;
+        by_nhy.divmod(q, hx, hy);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float z[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) z[j] = real ? acc[t][4 * g + j] : 0.f;
+          float same = z[0], tail = 0.f;
+#pragma unroll
+          for (int k = 1; k < 4; ++k) {
+            const int from = ((half << 5) | ((l32 - k) & 31)) << 2;       // the lane k positions back, in this tile or the one before
+            const float cur = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(z[k])));
+            const float old = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(prev[g][k - 1])));
+            const float v = l32 >= k ? cur : old;
+            if (hy >= k) same += v;
+            else tail += v;
+          }
+#pragma unroll
+          for (int k = 1; k < 4; ++k) prev[g][k - 1] = z[k];
+          const int fx = mt * 8 + 2 * g + half;
+          if (active && fx < pl.nfx) {
+            float *Yc = Z + ((i64)(n * pl.c_in + ci) * pl.nfx + fx) * pl.nhx * pl.ngy;
+            const int gy = hy - pl.py;
+            if (real && gy >= 0 && gy < pl.ngy) Yc[(i64)hx * pl.ngy + gy] = same;
+            const int gt = pl.nhy + hy - pl.py;                            // the row before: its columns past nhy - 1
+            if (hy < 3 && hx > row_a && q < q_hi + 3 && gt >= 0 && gt < pl.ngy) Yc[(i64)(hx - 1) * pl.ngy + gt] = tail;
+          }
+        }
+      }
+    } else if (active) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int q = q_lo + c * P + t * 32 + l32;
         if (q < pl.nh) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -925,13 +979,13 @@ __global__ __launch_bounds__(768) void tap_product_kernel(const TapProductPlan p
 template <int KSTEPS>
 hipError_t launch_tap_product_instance(const TapProductPlan &pl, const float *w, const float *go,
                                        float *z, hipStream_t stream) {
-  auto kern = tap_product_kernel<KSTEPS>;
+  auto kern = pl.yfold ? tap_product_kernel<KSTEPS, true> : tap_product_kernel<KSTEPS, false>;
   if (pl.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)pl.lds_bytes);
     if (e != hipSuccess) return e;
   }
-  const int groups_x = (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
+  const int groups_x = pl.yfold ? (pl.nhx + pl.rows_wg - 1) / pl.rows_wg : (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;
   const int image_groups = (pl.batch + pl.jobs - 1) / pl.jobs;
   hipLaunchKernelGGL(kern, dim3((unsigned)(image_groups * groups_x)), dim3(64 * pl.units * pl.jobs),
                      pl.lds_bytes, stream, pl, w, go, z);
@@ -967,7 +1021,32 @@ bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64
   pl.lds_bytes = 4 * (size_t)(2 * pl.ksteps * 64) * pl.jobs;
   pl.ws_bytes = 4 * (size_t)batch * c_in * pl.nf_pad * nh;
   if (image_groups * ((pl.chunks_per_image + pl.cpw - 1) / pl.cpw) >= ((i64)1 << 31)) return false;
+  pl.yfold = 0;
+  pl.nfx = (int)nfx; pl.nhx = (int)nhx; pl.nhy = (int)nhy; pl.ngy = 0; pl.py = 0; pl.rows_wg = 1;
   return true;
+}
+
+void enable_tap_yfold(TapProductPlan &pl, i64 nfx, i64 nfy, i64 nhx, i64 nhy, i64 ngy, i64 sy, i64 dy, i64 py,
+                      i64 uy) {
+  // (rows of at least three positions: "k positions back" then reaches the row before at most)
+  if (nfy != 4 || sy != 1 || dy != 1 || uy != 1 || py < 0 || ngy > nhy + 3 - py || ngy < 1 || nhy < 3) return;
+  if (nhx * nhy + 64 >= ((i64)1 << 22) || pl.jobs != 1) return;          // (float-reciprocal index split)
+  // rows per workgroup: a multiple of what keeps a workgroup's first position a multiple of
+  // four (16-byte loads); among those that leave the chip two workgroups per CU, the one
+  // whose rows (and three positions more) fill their 64-position chunks best
+  const i64 step = nhy % 4 == 0 ? 1 : (nhy % 2 == 0 ? 2 : 4);
+  i64 best = step;
+  double best_fill = 0;
+  for (i64 r = step; r <= 16 * step && r <= std::max<i64>(nhx, step); r += step) {
+    const i64 wgs = pl.batch * ((nhx + r - 1) / r);
+    const double fill = (double)(r * nhy) / (double)(64 * ((r * nhy + 3 + 63) / 64));
+    if (r > step && wgs < 512) break;
+    if (fill > best_fill + 1e-9) { best = r; best_fill = fill; }
+  }
+  if ((double)pl.batch * ((nhx + best - 1) / best) >= (double)((i64)1 << 31)) return;
+  pl.yfold = 1;
+  pl.ngy = (int)ngy; pl.py = (int)py; pl.rows_wg = (int)best;
+  pl.ws_bytes = 4 * (size_t)pl.batch * pl.c_in * nfx * nhx * ngy;
 }
 
 hipError_t launch_tap_product(const TapProductPlan &pl, const float *weight, const float *grad_out,

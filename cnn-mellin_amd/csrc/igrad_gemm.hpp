@@ -58,7 +58,19 @@ struct TapProductPlan {
   int chunks_per_image, cpw;         // 64-position chunks; chunks per workgroup
   int nf_pad;                        // mtn * 32
   size_t lds_bytes, ws_bytes;        // ws: Z
+  // yfold: the kernel sums the four filter columns of a filter row itself and stores
+  //   Y[n, ci, fx, hx, gy] = sum_fy Z[n, ci, fx * 4 + fy, hx, gy + py - fy]
+  // (a quarter of Z; ws then holds Y, (batch, c_in, nfx, nhx, ngy)); a fold over x finishes.
+  // A workgroup then takes rows_wg whole rows of grad_out.
+  int yfold, nfx, nhx, nhy, ngy, py, rows_wg;
 };
+
+// Switches the plan to the y-folding form where it applies: four filter columns, unit
+// stride, dilation and up-sampling along y, left padding only, grad_out rows of three
+// positions or more, and a grad_input row that the taps of a grad_out row cover
+// (ngy <= nhy + 3 - py).
+void enable_tap_yfold(TapProductPlan &pl, i64 nfx, i64 nfy, i64 nhx, i64 nhy, i64 ngy, i64 sy, i64 dy, i64 py,
+                      i64 uy);
 
 bool make_tap_product_plan(i64 batch, i64 c_in, i64 c_out, i64 nfx, i64 nfy, i64 nhx, i64 nhy,
                            TapProductPlan &pl);

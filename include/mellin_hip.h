@@ -447,7 +447,9 @@ int mellin_last_math(void);
  * their size run per residue class ("one-launch" also keeps the first pass of a
  * two-pass input gradient in one launch, and input gradients that would take two
  * passes only for the launches per filter row in the gather form; for comparisons
- * and tests; "whole-classes": automatic choice, but a class's rows are never cut
+ * and tests; "tap-columns": automatic choice, but the tap-product input gradient
+ * keeps one product per filter column in its workspace instead of summing the four
+ * columns of a filter row in the kernel; "whole-classes": automatic choice, but a class's rows are never cut
  * into ranges by where the filter rows' taps leave the signal; "class-launches":
  * like "classes", with a launch per class also where one launch would hold them).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */

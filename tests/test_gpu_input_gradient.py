@@ -163,3 +163,43 @@ def test_wide_mellin_layers_take_the_dense_two_pass_path(case):
     other, v2 = _grad_input(hip.AX_MCORR, w, go, (n, c_in) + ng, s, d, p, u, "generic")
     assert v2 == "generic", v2
     assert_close(other, exp, c_out * nf[0] * nf[1], "generic %s" % (case,))
+
+
+# Tap products with the four filter columns of a filter row summed in the kernel (Y, a quarter
+# of the tap products, goes through the workspace; a fold over x finishes): rows of exactly 64
+# positions per image pair (the last row's tail then takes a chunk of its own), left padding,
+# outputs past the valid size (grad_input narrower than the taps reach), the shortest rows the
+# form takes (three positions), and rows too short for it (the per-column form runs).
+YFOLD_CASES = [
+    # (kind, n, c_in, c_out, nf, ng, s, d, p, r, summed in the kernel)
+    (hip.AX_MCORR, 2, 3, 64, (8, 4), (64, 19), (1, 1), (1, 1), (0, 0), (0, 0), True),
+    (hip.AX_MCORR, 3, 2, 33, (3, 4), (30, 6), (1, 1), (1, 1), (1, 3), (0, 0), True),
+    (hip.AX_MCORR, 1, 5, 16, (5, 4), (40, 5), (1, 1), (1, 1), (0, 1), (0, 1), True),
+    (hip.AX_MCORR, 2, 1, 8, (2, 4), (21, 6), (1, 1), (1, 1), (0, 0), (0, 0), True),
+    (hip.AX_MCORR, 2, 3, 16, (2, 4), (20, 5), (1, 1), (1, 1), (0, 0), (0, 0), False),
+    (hip.AX_MCORR, 2, 3, 16, (2, 4), (20, 9), (1, 2), (1, 1), (0, 0), (0, 0), False),   # stride along y
+]
+
+
+@pytest.mark.parametrize("case", YFOLD_CASES, ids=[str(i) for i in range(len(YFOLD_CASES))])
+def test_tap_products_summed_over_filter_columns(case):
+    import mconv
+    kind, n, c_in, c_out, nf, ng, s, d, p, r, summed = case
+    u = (1, 1)
+    valid_x = mconv.mcorr_valid_size if kind == hip.AX_MCORR else mconv.lcorr_valid_size
+    nh = (valid_x(nf[0], ng[0], s[0], d[0], p[0], 1) + r[0], mconv.lcorr_valid_size(nf[1], ng[1], s[1], d[1], p[1], 1) + r[1])
+    assert min(nh) > 0
+    rng = np.random.default_rng(5100 + YFOLD_CASES.index(case))
+    w = rng.standard_normal((c_out, c_in) + nf).astype(np.float32)
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    bwd = oracle.mcorrlcorr_backward if kind == hip.AX_MCORR else oracle.lcorrlcorr_backward
+    exp, _, _ = bwd(np.zeros((n, c_in) + ng), w.astype(np.float64), go.astype(np.float64), s, d, p, u)
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, u)
+    need = hip.lib.mellin_corr2d_backward_input_workspace(kind, 4, *dims)
+    assert need == 4 * n * c_in * (nf[0] * nh[0] * ng[1] if summed else 32 * nh[0] * nh[1])
+    got, v = _grad_input(kind, w, go, (n, c_in) + ng, s, d, p, u, None)
+    assert v == "mfma-taps+fold", v
+    assert_close(got, exp, c_out * nf[0] * nf[1], "filter columns summed %s" % (case,))
+    other, v = _grad_input(kind, w, go, (n, c_in) + ng, s, d, p, u, "tap-columns")
+    assert v == "mfma-taps+fold", v
+    assert_close(other, exp, c_out * nf[0] * nf[1], "per column %s" % (case,))
