@@ -122,6 +122,17 @@ def test_large_forward_passes_take_the_classes_by_default():
     finally:
         hip.set_variant(None)
     assert bool(((got - ref).abs() <= 1e-5 * ref.abs() + 1e-5 * (c_in * 16) ** 0.5).all())
+    # (this layer keeps its 120 rows while the taps of filter rows 2 and 3 end at rows 79 and 59:
+    # by default a class's rows are cut there and all ranges share a launch; uncut, a launch per
+    # class -- the same products in the same order, the rows of zeros left out or not)
+    hip.set_variant("whole-classes")
+    try:
+        whole = torch.full_like(got, float("nan"))
+        hip.corr2d_forward(hip.AX_MCORR, x, w, b, whole, dims)
+        assert hip.last_variant() == "mfma-classes"
+    finally:
+        hip.set_variant(None)
+    assert torch.equal(whole, got)
 
 
 # Input gradients in two passes (layers that keep fewer rows than they are given): the first
