@@ -433,6 +433,7 @@ struct TwoPassInput {
   // out the c_in output channels of filter row fx[i], on the rows of grad_out that have a tap
   // of that filter row and on no others.
   int rows = 0;
+  bool rows_one_launch = false;    // the launches planned with one tile shape: they share a launch
   TilePlan row_plan[kMaxClasses];
   size_t row_lds[kMaxClasses], row_frag_off[kMaxClasses];    // (fragment regions: offsets from frag_off)
   int row_mt[kMaxClasses], row_nt[kMaxClasses], row_fx[kMaxClasses];
@@ -475,18 +476,43 @@ bool plan_first_pass_rows(const SepConv &first, i64 c_in, i64 nfx, i64 nfy, i64 
     ++n;
   }
   if (n == 0 || blocks * 5 > ((c_in * nfx + 31) / 32) * nhx * 4) return false;
+  // every launch with the tile shape it would pick by itself (force_mt = 0), or all with one
+  auto plan_all = [&](int force_mt, int force_nt, size_t &frag) {
+    frag = 0;
+    for (int i = 0; i < n; ++i) {
+      SepConv c = first;
+      c.x = make_axis(AX_MCORR, 1, nhx, hi[i] + 1, 1, 1, 0, 1);        // tap (h + 1)(0 + 1)/1 - 1 = h: rows pass through
+      c.c_out = c_in;
+      c.f_m = nfx * nfy;
+      c.h_m = nfx * nhx * ngy;
+      c.cls_stride = (int)q[i]; c.cls_first = (int)lo[i]; c.cls_nfx = 1; c.cls_fx = 0;
+      if (!c.in_half) c.math = MATH_BF16X3_ALWAYS;
+      if (!make_tile_plan(c, tp.row_plan[i], &tp.row_lds[i], &tp.row_mt[i], &tp.row_nt[i], force_nt, true, force_mt))
+        return false;
+      tp.row_frag_off[i] = frag;
+      frag += (tile_fragment_bytes(tp.row_plan[i], tp.row_mt[i]) + 255) & ~(size_t)255;
+    }
+    return true;
+  };
   size_t frag = 0;
-  for (int i = 0; i < n; ++i) {
-    SepConv c = first;
-    c.x = make_axis(AX_MCORR, 1, nhx, hi[i] + 1, 1, 1, 0, 1);          // tap (h + 1)(0 + 1)/1 - 1 = h: rows pass through
-    c.c_out = c_in;
-    c.f_m = nfx * nfy;
-    c.h_m = nfx * nhx * ngy;
-    c.cls_stride = (int)q[i]; c.cls_first = (int)lo[i]; c.cls_nfx = 1; c.cls_fx = 0;
-    if (!c.in_half) c.math = MATH_BF16X3_ALWAYS;
-    if (!make_tile_plan(c, tp.row_plan[i], &tp.row_lds[i], &tp.row_mt[i], &tp.row_nt[i])) return false;
-    tp.row_frag_off[i] = frag;
-    frag += (tile_fragment_bytes(tp.row_plan[i], tp.row_mt[i]) + 255) & ~(size_t)255;
+  if (!plan_all(0, 0, frag)) return false;
+  // One launch for all filter rows (tile_gemm_classes_kernel, the workgroups dealt to the
+  // filter rows by their work) where the plans allow it with the tile shape of the filter
+  // row that has the most rows: the launches of the filter rows with few rows are too
+  // short to fill the chip by themselves.
+  tp.rows_one_launch = false;
+  if (n >= 2 && !g_split_classes) {
+    int big = 0;
+    for (int i = 1; i < n; ++i)
+      if (tp.row_plan[i].Q > tp.row_plan[big].Q) big = i;
+    const int mt = tp.row_mt[big], nt = tp.row_nt[big];
+    size_t frag_one = 0;
+    if (plan_all(mt, nt, frag_one) && tile_classes_fit_one_launch(tp.row_plan, tp.row_mt, tp.row_nt, n)) {
+      tp.rows_one_launch = true;
+      frag = frag_one;
+    } else if (!plan_all(0, 0, frag)) {
+      return false;
+    }
   }
   tp.rows = n;
   tp.frag_bytes = frag;
@@ -500,6 +526,17 @@ hipError_t launch_first_pass(const TwoPassInput &tp, const void *weight, const v
   if (tp.rows == 0)
     return launch_tile_gemm(tp.plan, tp.lds, tp.mt, tp.nt, (const float *)weight, (const float *)grad_out, nullptr,
                             (float *)ws, stream, frag);
+  if (tp.rows_one_launch && frag && ((uintptr_t)frag & 15) == 0) {
+    long long f_bytes[kMaxClasses], h_bytes[kMaxClasses];
+    for (int i = 0; i < tp.rows; ++i) {
+      const TilePlan &pl = tp.row_plan[i];
+      f_bytes[i] = (long long)tp.row_fx[i] * pl.f_pitch * elem_bytes;
+      h_bytes[i] = (long long)tp.row_fx[i] * pl.ngx * pl.noy * 4;
+    }
+    return launch_tile_gemm_classes(tp.row_plan, tp.row_lds, tp.rows, tp.row_mt[0], tp.row_nt[0], (const float *)weight,
+                                    (const float *)grad_out, nullptr, (float *)ws, stream, frag, tp.row_frag_off, f_bytes,
+                                    h_bytes);
+  }
   for (int i = 0; i < tp.rows; ++i) {
     const TilePlan &pl = tp.row_plan[i];
     const i64 fx = tp.row_fx[i];
@@ -528,9 +565,10 @@ bool plan_two_pass_input(int kind_x, i64 batch, i64 c_in, i64 c_out, i64 nfx, i6
   // virtual row of zeros for each), given enough products per word of Y to pay for writing
   // and reading it: c_out * nfy from 256 on (measured on the 10-layer stack: 644 -> 594 us at
   // 256, 1157 -> 795 at 512, 3479 -> 1442 at 1024; 370 -> 451 at 128), in half precision,
-  // where the gather form is three times faster and Y is still fp32, from 1024 on
-  // (900 -> 744 us; 458 -> 570 at 512)
-  const bool mellin_rows = kind_x == AX_MCORR && c_in >= 16 && px >= 1 && c_out * nfy >= (half ? 1024 : 256);
+  // where the gather form is three times faster and Y is still fp32, from 512 on
+  // (with all filter rows in one launch: 453 -> 373 us at 512, 900 -> 549 at 1024;
+  // 291 -> 347 at 256)
+  const bool mellin_rows = kind_x == AX_MCORR && c_in >= 16 && px >= 1 && c_out * nfy >= (half ? 512 : 256);
   if ((c_in >= 16 && !mellin_wide && !mellin_rows) || nfx < 2) return false;
   if ((double)batch * m2 * nhx * ngy * 4.0 > (double)kMaxWorkspaceBytes) return false;
   const i64 pad = ((m2 + 31) / 32) * 32;

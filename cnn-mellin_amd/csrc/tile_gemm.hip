@@ -493,6 +493,7 @@ struct ClassLaunch {
   TilePlan pl[kMaxTileClasses];
   int n, wg_end[kMaxTileClasses];
   long long af_words[kMaxTileClasses];               // where the class's fragments start in AF (floats)
+  long long f_bytes[kMaxTileClasses], h_bytes[kMaxTileClasses];   // the class's filter and output: bytes past F and H
 };
 
 static_assert(sizeof(ClassLaunch) + 5 * sizeof(void *) <= 4096, "kernel arguments are limited to 4 KB");
@@ -505,8 +506,9 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 3 : 2)) void tile_gemm_classes
   ConstArgs *const a = (ConstArgs *)__builtin_amdgcn_kernarg_segment_ptr();
   int c = 0, first = 0;
   for (; c + 1 < a->n && (int)blockIdx.x >= a->wg_end[c]; ++c) first = a->wg_end[c];
-  tile_gemm_body<MT, NT, false, 0, HOUT, SPLIT>((ConstPlan *)&a->pl[c], (int)blockIdx.x - first, a->wg_end[c] - first, F,
-                                               G, bias, H, AF ? AF + a->af_words[c] : AF);
+  tile_gemm_body<MT, NT, false, 0, HOUT, SPLIT>((ConstPlan *)&a->pl[c], (int)blockIdx.x - first, a->wg_end[c] - first,
+                                               (const float *)((const char *)F + a->f_bytes[c]), G, bias,
+                                               (float *)((char *)H + a->h_bytes[c]), AF ? AF + a->af_words[c] : AF);
 }
 
 // The whole filter as fragments, once per launch, in the order the stages of the SPLIT
@@ -1010,7 +1012,7 @@ bool tile_classes_fit_one_launch(const TilePlan *pls, const int *mts, const int 
 
 hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes, int n, int mt, int nt, const float *f,
                                     const float *g, const float *bias, float *h, hipStream_t stream, float *frag_ws,
-                                    const size_t *frag_off) {
+                                    const size_t *frag_off, const long long *f_bytes, const long long *h_bytes) {
   if (!tile_classes_fit_one_launch(pls, std::vector<int>(n, mt).data(), std::vector<int>(n, nt).data(), n))
     return hipErrorInvalidValue;
   const int M_T = mt * 32;
@@ -1026,12 +1028,14 @@ hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes
     const int chunks = (pls[i].C + pls[i].CC - 1) / pls[i].CC;
     work[i] = (double)chunks * pls[i].KC16;
     args.af_words[i] = 0;
+    args.f_bytes[i] = f_bytes ? f_bytes[i] : 0;
+    args.h_bytes[i] = h_bytes ? h_bytes[i] : 0;
     if (frag_ws) {
       const i64 items = (i64)tile_fragment_bytes(pls[i], mt) / (f16 ? 16 : 48);
       float *ws = (float *)((char *)frag_ws + frag_off[i]);
       hipLaunchKernelGGL((f16 ? filter_fragments_kernel<true> : filter_fragments_kernel<false>),
-                         dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pls[i], M_T, chunks, (const void *)f,
-                         (uintx4 *)ws);
+                         dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pls[i], M_T, chunks,
+                         (const void *)((const char *)f + args.f_bytes[i]), (uintx4 *)ws);
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) return e;
       args.af_words[i] = (long long)(frag_off[i] / 4);

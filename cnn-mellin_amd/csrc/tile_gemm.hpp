@@ -86,11 +86,13 @@ hipError_t launch_tile_gemm(const TilePlan &pl, size_t lds_bytes, int mt, int nt
 // class for its whole life, the classes share the chip in proportion to their work.
 // tile_classes_fit_one_launch: the plans allow it (same tile shape, all staged in chunks on
 // the bf16 / f16 matrix cores).  frag_ws + frag_off[i]: class i's fragments (required for
-// half precision), or frag_ws null.
+// half precision), or frag_ws null.  f_bytes[i] / h_bytes[i]: class i's filter and output
+// start that many bytes past f and h (null: all at f and h).
 bool tile_classes_fit_one_launch(const TilePlan *pls, const int *mts, const int *nts, int n);
 hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes, int n, int mt, int nt, const float *f,
                                     const float *g, const float *bias, float *h, hipStream_t stream, float *frag_ws,
-                                    const size_t *frag_off);
+                                    const size_t *frag_off,
+                                    const long long *f_bytes = nullptr, const long long *h_bytes = nullptr);
 
 // Weight gradient (wgrad_gemm.hip): position tiling and signal staging of the
 // forward problem in `t`, plus the blocking of the (c_out) x (c_in * taps) output.

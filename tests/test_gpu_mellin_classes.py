@@ -149,7 +149,7 @@ ROW_CASES = [
     # 1-D, dilation 3 with p + 1 = 3: steps 1, 3, 3, 1
     (3, 64, 20, (4, 1), (100, 1), (1, 1), (3, 1), (2, 0), (0, 0)),
     # layers that keep their rows, as in the 10-layer stack: the form from 256 products per
-    # first-pass word on (c_out * nfy), in half precision from 1024 on
+    # first-pass word on (c_out * nfy), in half precision from 512 on
     (2, 64, 64, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
     (1, 32, 256, (4, 4), (40, 6), (1, 1), (1, 1), (1, 1), (20, 0)),
     # one output column under a dilated 8-wide filter: the first pass keeps filter columns 1-4
@@ -198,7 +198,7 @@ def test_half_first_pass_per_filter_row(case, classes_forced):
     wh, goh = torch.from_numpy(w).half().cuda(), torch.from_numpy(go).half().cuda()
     gi = torch.full((n, c_in) + ng, float("nan"), dtype=torch.float16, device="cuda")
     hip.corr2d_backward_input(hip.AX_MCORR, wh, goh, gi, dims)
-    if 8 * nh[0] > 7 * ng[0] and c_out * nf[1] < 1024:
+    if 8 * nh[0] > 7 * ng[0] and c_out * nf[1] < 512:
         assert hip.last_variant() in ("mfma-f16-classes", "mfma-f16-class-launches")   # the gather form
         return
     assert hip.last_variant() == "mfma-f16-filter-rows+fold"
@@ -240,7 +240,7 @@ def test_large_input_gradients_take_the_filter_rows_by_default():
     finally:
         hip.set_variant(None)
     assert bool(((got - ref).abs() <= 1e-5 * ref.abs() + 1e-5 * (c_out * 16) ** 0.5).all())
-    # half precision: 1024 products per first-pass word
+    # half precision, from 512 products per first-pass word on: 1024 here
     gh = torch.full((n, c_in) + ng, float("nan"), dtype=torch.float16, device="cuda")
     hip.corr2d_backward_input(hip.AX_MCORR, w.half(), go.half(), gh, dims)
     assert hip.last_variant() == "mfma-f16-filter-rows+fold"
