@@ -515,10 +515,9 @@ __global__ __launch_bounds__(kThreads, (NT == 1 ? 3 : 2)) void tile_gemm_classes
 // kernel copy them: AF[m_tile][chunk][part][group][row] (16-byte words).  One thread per
 // (m_tile, chunk, group, row): eight taps of one output channel, split, three stores.
 // F16: F is half-precision storage and a fragment is the eight values themselves (one part).
-template <bool F16>
-__global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int M_T, int chunks,
-                                                               const void *__restrict__ Fv,
-                                                               uintx4 *__restrict__ AF) {
+template <bool F16, class PL>
+__device__ __forceinline__ void filter_fragments_body(const PL &pl, int M_T, int chunks, const void *__restrict__ Fv,
+                                                      uintx4 *__restrict__ AF) {
   const int groups = pl.KC16 >> 3;
   const int per_block = groups * M_T;
   const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
@@ -545,6 +544,26 @@ __global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int 
   } else {
     store_frag(AF + (i64)blk * 3 * per_block, groups, M_T, g, m, x);
   }
+}
+
+template <bool F16>
+__global__ __launch_bounds__(256) void filter_fragments_kernel(TilePlan pl, int M_T, int chunks,
+                                                               const void *__restrict__ Fv,
+                                                               uintx4 *__restrict__ AF) {
+  filter_fragments_body<F16>(pl, M_T, chunks, Fv, AF);
+}
+
+// The same for every class of a launch at once: blockIdx.y is the class.
+template <bool F16>
+__global__ __launch_bounds__(256) void filter_fragments_classes_kernel(ClassLaunch args, int M_T,
+                                                                       const void *__restrict__ Fv,
+                                                                       float *__restrict__ AF) {
+  typedef const __attribute__((address_space(4))) ClassLaunch ConstArgs;
+  ConstArgs *const a = (ConstArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+  const int c = (int)blockIdx.y;
+  const auto &pl = a->pl[c];
+  filter_fragments_body<F16>(pl, M_T, (pl.C + pl.CC - 1) / pl.CC, (const char *)Fv + a->f_bytes[c],
+                             (uintx4 *)(AF + a->af_words[c]));
 }
 
 template <int MT, int NT, bool ACC, int MB, bool HOUT = false, int SPLIT = 0>
@@ -1022,6 +1041,7 @@ hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes
   args.n = n;
   size_t lds = 0;
   double work[kMaxTileClasses];                              // per tile
+  i64 max_items = 0;                                         // fragment items (eight taps of a channel) of the largest class
   for (int i = 0; i < n; ++i) {
     args.pl[i] = pls[i];
     lds = std::max(lds, lds_bytes[i]);
@@ -1031,15 +1051,18 @@ hipError_t launch_tile_gemm_classes(const TilePlan *pls, const size_t *lds_bytes
     args.f_bytes[i] = f_bytes ? f_bytes[i] : 0;
     args.h_bytes[i] = h_bytes ? h_bytes[i] : 0;
     if (frag_ws) {
-      const i64 items = (i64)tile_fragment_bytes(pls[i], mt) / (f16 ? 16 : 48);
-      float *ws = (float *)((char *)frag_ws + frag_off[i]);
-      hipLaunchKernelGGL((f16 ? filter_fragments_kernel<true> : filter_fragments_kernel<false>),
-                         dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, pls[i], M_T, chunks,
-                         (const void *)((const char *)f + args.f_bytes[i]), (uintx4 *)ws);
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) return e;
+      max_items = std::max(max_items, (i64)tile_fragment_bytes(pls[i], mt) / (f16 ? 16 : 48));
       args.af_words[i] = (long long)(frag_off[i] / 4);
     }
+  }
+  if (frag_ws && max_items > 0) {
+    // (wg_end is not read by this kernel)
+    for (int i = 0; i < kMaxTileClasses; ++i) args.wg_end[i] = 0;
+    hipLaunchKernelGGL((f16 ? filter_fragments_classes_kernel<true> : filter_fragments_classes_kernel<false>),
+                       dim3((unsigned)((max_items + 255) / 256), (unsigned)n), dim3(256), 0, stream, args, M_T,
+                       (const void *)f, frag_ws);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
   }
   // persistent workgroups: as many as fit at once, dealt to the classes by their work
   const int m_tiles = (pls[0].M + M_T - 1) / M_T;
