@@ -740,41 +740,54 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     const int gi_c = pl.ngx * pl.ngy, ws_c = (pl.strips - 1) * pl.nshared * 2 * pl.ngy;   // words per input channel
     T *GIn = GI + (i64)n * pl.c_in * gi_c;
     float *WSn = WS + (i64)n * pl.c_in * ws_c;
-    // four rows per trip: their table entries first, then all their reads, then the stores,
-    // so that the LDS round trips of the four overlap
-    for (int cc = 0; cc < pl.c_in; ++cc)
-      for (int pi = wave; pi < rp_t; pi += 4 * kWaves) {
-        int kind[4], dst[4], src[4], nw[4];
+    // four rows of every input channel per trip: their table entries first (the same for
+    // every channel), then all their reads, then the stores, so that the LDS round trips of a
+    // trip overlap and a wavefront makes three trips, not nine (lconv2d.grad_input of the
+    // benchmark 72 -> 67.5 us; eight rows per trip ran out of registers)
+    constexpr int kRowsTrip = 4;
+    // (a trip's table entries serve every input channel: the channels inside the trip)
+    for (int pi = wave; pi < rp_t; pi += kRowsTrip * kWaves) {
+      int kind[kRowsTrip], dst[kRowsTrip], src[kRowsTrip], nw[kRowsTrip];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int4 e = row_tab[min(pi + u * kWaves, rp_t - 1)];
-          kind[u] = pi + u * kWaves < rp_t ? __builtin_amdgcn_readfirstlane(e.x) : -1;
-          dst[u] = __builtin_amdgcn_readfirstlane(e.y);
-          src[u] = __builtin_amdgcn_readfirstlane(e.z);
-          nw[u] = __builtin_amdgcn_readfirstlane(e.w);
-        }
-        for (int gy = lane; gy < pl.ngy; gy += 64) {
-          // (no branches: all reads are requested together; a wavefront that does not reach the
-          // row, or a column past the image's, re-reads the first word and adds a zero)
-          const bool inside = gy + pl.py < pl.Wp;
-          const int col = inside ? gy : 0;
-          float x[4][kWaves];
+      for (int u = 0; u < kRowsTrip; ++u) {
+        const int4 e = row_tab[min(pi + u * kWaves, rp_t - 1)];
+        kind[u] = pi + u * kWaves < rp_t ? __builtin_amdgcn_readfirstlane(e.x) : -1;
+        dst[u] = __builtin_amdgcn_readfirstlane(e.y);
+        src[u] = __builtin_amdgcn_readfirstlane(e.z);
+        nw[u] = __builtin_amdgcn_readfirstlane(e.w);
+      }
+      for (int gy = lane; gy < pl.ngy; gy += 64) {
+        const bool inside = gy + pl.py < pl.Wp;
+        const int col = inside ? gy : 0;
+        for (int cc0 = 0; cc0 < pl.c_in; cc0 += 3) {
+          float x[3][kRowsTrip][kWaves];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const float *in = wplanes + src[u] + cc * wplane_words + pl.py;
+          for (int c3 = 0; c3 < 3; ++c3) {
+            const int cc = min(cc0 + c3, pl.c_in - 1);
 #pragma unroll
-            for (int k = 0; k < kWaves; ++k) x[u][k] = in[(k < nw[u] ? k * wave_step : 0) + col];
+            for (int u = 0; u < kRowsTrip; ++u) {
+              const float *in = wplanes + src[u] + cc * wplane_words + pl.py;
+#pragma unroll
+              for (int k = 0; k < kWaves; ++k) x[c3][u][k] = in[(k < nw[u] ? k * wave_step : 0) + col];
+            }
           }
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            float v = 0.f;
+          for (int c3 = 0; c3 < 3; ++c3) {
+            const int cc = cc0 + c3;
+            if (cc < pl.c_in) {
 #pragma unroll
-            for (int k = 0; k < kWaves; ++k) v += (inside && k < nw[u]) ? x[u][k] : 0.f;
-            if (kind[u] > 0) (WSn + cc * ws_c + dst[u])[gy] = v;
-            else if (kind[u] == 0) (GIn + cc * gi_c + dst[u])[gy] = (T)v;
+              for (int u = 0; u < kRowsTrip; ++u) {
+                float v = 0.f;
+#pragma unroll
+                for (int k = 0; k < kWaves; ++k) v += (inside && k < nw[u]) ? x[c3][u][k] : 0.f;
+                if (kind[u] > 0) (WSn + cc * ws_c + dst[u])[gy] = v;
+                else if (kind[u] == 0) (GIn + cc * gi_c + dst[u])[gy] = (T)v;
+              }
+            }
           }
         }
       }
+    }
   }
   // grad_input rows past the reach of the last grad_out row belong to the last strip: zeros
   if (strip == pl.strips - 1) {
