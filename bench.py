@@ -207,6 +207,59 @@ def cpu_baseline(layers, slice_n, reps=25):
             "frames_per_s": round(slice_n * CFG["ngx"] / med, 1)}
 
 
+def other_math_leg(args, dev, torch, hip, steps=30, reps=30):
+    """The same step once more under the other math mode (outside the main timed region):
+    wall-clock per step over `steps` steps after 10 warm-up steps, and per-pass medians."""
+    other = hip.MATH_FP32 if args.math == "bf16x3" else hip.MATH_BF16X3
+    hip.set_math(other)
+    try:
+        gen = torch.Generator().manual_seed(2)
+        layers = [Layer(hip.AX_MCORR, "mconv2d", gen, dev), Layer(hip.AX_LCORR, "lconv2d", gen, dev)]   # (workspaces of this mode)
+
+        def step():
+            for L in layers:
+                L.forward()
+                L.backward_input()
+                L.backward_weight()
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        per_pass, maths = {}, {}
+        for L in layers:
+            for pname, fn in L.passes():
+                key = "%s.%s" % (L.name, pname)
+                per_pass[key] = round(time_pass(fn, reps, torch), 2)
+                maths[key] = "bf16x3" if hip.last_math() == hip.MATH_BF16X3 else "fp32"
+        return {"ms_per_step": round(ms, 4), "steps": steps, "per_pass_us": per_pass, "per_pass_math": maths}
+    finally:
+        hip.set_math(hip.MATH_BF16X3 if args.math == "bf16x3" else hip.MATH_FP32)
+
+
+def other_configs(torch, reps=20):
+    """Per-pass times of BASELINE configuration 4 (wide layer, linear and Mellin x axis) and
+    forward + backward of the two 10-layer stacks of configuration 5, by time_layers.py's own
+    routines, `reps` timed calls each (outside the main timed region; not bench lines)."""
+    import time_layers
+    out = {"reps": reps, "cfg4": {}, "cfg5_stack_forward_backward_ms": {}}
+
+    def keep_layer(rec):
+        out["cfg4"][rec["layer"].split()[-1]] = {k: rec[k]["us"] for k in ("forward", "grad_input", "grad_weight")}
+
+    def keep_stack(rec):
+        if "stack" in rec:
+            out["cfg5_stack_forward_backward_ms"][rec["stack"]] = rec["forward_backward_ms"]
+    time_layers.run_cfg4(reps, torch.float32, emit=keep_layer)
+    time_layers.run_stack(reps, torch.float32, emit=keep_stack, per_layer=False)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,6 +268,9 @@ def main():
     ap.add_argument("--math", choices=["bf16x3", "fp32"], default="bf16x3",
                     help="how the matrix kernels form fp32 products (library default: bf16x3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the legs outside the timed region: the same step under the fp32 math mode and the "
+                         "other configurations (wide layer, 10-layer stacks)")
     ap.add_argument("--variant", default=None, help="force a kernel variant (e.g. generic)")
     ap.add_argument("--cpu-slice", type=int, default=32, help="utterances in the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -344,9 +400,9 @@ def main():
                    "algorithmic_MB_per_step": round(step_bytes / 1e6, 3),
                    "GFLOP_per_step": round(step_flops / 1e9, 3),
                    "arithmetic": ("fp32 storage, fp32 accumulation; products of the matrix kernels: every fp32 "
-                                  "operand as the exact sum of three bf16 parts, the six largest of the nine "
-                                  "cross products on the bf16 matrix cores (what is dropped is below 2^-24 of "
-                                  "a product)" if args.math == "bf16x3" else
+                                  "operand as the exact sum of three bf16 parts (rounded to nearest), the six "
+                                  "largest of the nine cross products on the bf16 matrix cores (what is dropped "
+                                  "is at most 1.01 * 2^-23 of a product, worst case)" if args.math == "bf16x3" else
                                   "fp32 storage, accumulation and matrix instructions")},
         "prewarm_ms": round(prewarm_ms, 1), "prewarm_steps": prewarm_steps,
         "frames_per_s": round(frames / (elapsed / args.steps), 1),
@@ -363,6 +419,9 @@ def main():
             "fp32_equivalent_TFLOPs": round(2 * (layers[0] if k.startswith("mconv2d") else layers[1]).macs_per_pass
                                             / v / 1e6, 2)}
         for k, v in per_pass.items()}
+    if not args.no_extras:
+        line["fp32_math" if args.math == "bf16x3" else "bf16x3_math"] = other_math_leg(args, dev, torch, hip)
+        line["other_configs"] = other_configs(torch)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(layers, args.cpu_slice)
     print(json.dumps(line))

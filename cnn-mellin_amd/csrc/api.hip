@@ -1347,20 +1347,27 @@ int mellin_get_math(void) { return g_math; }
 int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
-  const bool widen = name && !strcmp(name, "widen"), one = name && !strcmp(name, "one-launch");
-  const bool all = name && !strcmp(name, "classes"), each = name && !strcmp(name, "class-launches");
-  const bool whole = name && !strcmp(name, "whole-classes"), columns = name && !strcmp(name, "tap-columns");
-  g_widen = widen;
-  g_no_classes = one;
-  g_all_classes = all || each;
-  g_split_classes = each;
-  g_whole_classes = whole;
-  g_no_yfold = columns;
-  if (!name || !*name || widen || one || all || each || whole || columns) { g_forced = 0; return MELLIN_OK; }
-  if (!strcmp(name, "generic")) { g_forced = 1; return MELLIN_OK; }
-  if (!strcmp(name, "auto")) { g_forced = 0; return MELLIN_OK; }
-  if (!strcmp(name, "two-pass")) { g_forced = 2; return MELLIN_OK; }
-  return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
+  // the name is parsed first: an unknown one changes nothing
+  struct Setting { int forced, widen, no_classes, all_classes, split_classes, whole_classes, no_yfold;  };
+  Setting v = {0, 0, 0, 0, 0, 0, 0};
+  if (!name || !*name || !strcmp(name, "auto")) {}
+  else if (!strcmp(name, "generic")) v.forced = 1;
+  else if (!strcmp(name, "two-pass")) v.forced = 2;
+  else if (!strcmp(name, "widen")) v.widen = 1;
+  else if (!strcmp(name, "one-launch")) v.no_classes = 1;
+  else if (!strcmp(name, "classes")) v.all_classes = 1;
+  else if (!strcmp(name, "class-launches")) { v.all_classes = 1; v.split_classes = 1; }
+  else if (!strcmp(name, "whole-classes")) v.whole_classes = 1;
+  else if (!strcmp(name, "tap-columns")) v.no_yfold = 1;
+  else return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
+  g_widen = v.widen;
+  g_no_classes = v.no_classes;
+  g_all_classes = v.all_classes;
+  g_split_classes = v.split_classes;
+  g_whole_classes = v.whole_classes;
+  g_no_yfold = v.no_yfold;
+  g_forced = v.forced;
+  return MELLIN_OK;
 }
 
 #define DEFINE_1D(NAME, T, KX, KY)                                             \

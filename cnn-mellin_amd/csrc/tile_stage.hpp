@@ -425,30 +425,40 @@ __device__ __forceinline__ void multiply_taps(floatx16 (&acc)[MT][NT], const flo
 
 // ---- fp32 products on the bf16 matrix cores ------------------------------------------
 // An fp32 value is the exact sum of three bf16 values (8 + 8 + 8 significant bits):
-// hi = x with its low 16 bits cleared, mid = (x - hi) likewise, lo = x - hi - mid.  A
-// product x * y is then the sum of nine bf16 products, each exact in fp32; the six
-// largest (hi hi, hi mid, mid hi, hi lo, lo hi, mid mid) carry everything down to
-// 2^-24 of |x y|, i.e. what an fp32 multiply-add keeps.  v_mfma_f32_32x32x16_bf16
-// accumulates in fp32 and runs at sixteen times the rate of v_mfma_f32_32x32x2_f32
-// per product, so six of them cost three eighths of the fp32 instruction's time.
+// hi = x rounded to the nearest bf16, mid = (x - hi) rounded likewise, lo = x - hi - mid
+// (exact: what is left has at most 8 significant bits).  Both subtractions are exact in fp32.
+// With rounding to nearest |mid| <= 2^-8 |x| and |lo| <= 2^-16 |x| (up to a factor 1 + 2^-8).
+// A product x * y is then the sum of nine bf16 products, each exact in fp32; the six
+// largest (hi hi, hi mid, mid hi, hi lo, lo hi, mid mid) are issued, and the three dropped
+// ones (mid lo, lo mid, lo lo) are together below 1.01 * 2^-23 |x y|: two roundings of an
+// fp32 product.  v_mfma_f32_32x32x16_bf16 accumulates in fp32 and runs at sixteen times the
+// rate of v_mfma_f32_32x32x2_f32 per product, so six of them cost three eighths of the fp32
+// instruction's time.
+// Values that round to an infinite bf16 (infinities, and finite values above 3.3895e38)
+// give NaN parts (inf - inf) and hence NaN results; NaN stays NaN.
 __device__ __forceinline__ bf16x8 as_bf16x8(uintx4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// Two values -> their parts, x0's in the low half and x1's in the high half of each word.
+// v_cvt_pk_bf16_f32 rounds both to nearest even and packs them; a part back as fp32 is the
+// half moved to the top of a word.
+__device__ __forceinline__ void split_pair(float x0, float x1, unsigned &hi, unsigned &mid, unsigned &lo) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float floatx2 __attribute__((ext_vector_type(2)));
+  const floatx2 v = {x0, x1};
+  hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+  const floatx2 r1 = {x0 - __uint_as_float(hi << 16), x1 - __uint_as_float(hi & 0xFFFF0000u)};
+  mid = __builtin_bit_cast(unsigned, __builtin_convertvector(r1, bf16x2));
+  const floatx2 r2 = {r1.x - __uint_as_float(mid << 16), r1.y - __uint_as_float(mid & 0xFFFF0000u)};
+  lo = __builtin_bit_cast(unsigned, __builtin_convertvector(r2, bf16x2));
+}
 
 // x[0..8) -> packed hi / mid / lo parts (element i in half i & 1 of word i >> 1)
 __device__ __forceinline__ void split8(const float (&x)[8], uintx4 &hi, uintx4 &mid, uintx4 &lo) {
-  unsigned m[8], l[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float r1 = x[i] - __uint_as_float(__float_as_uint(x[i]) & 0xFFFF0000u);
-    const float r2 = r1 - __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
-    m[i] = __float_as_uint(r1);
-    l[i] = __float_as_uint(r2);
-  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    // the upper halves of two words: {a[31:16], b[31:16]} -> word (a high, b low)
-    hi[i] = __builtin_amdgcn_perm(__float_as_uint(x[2 * i + 1]), __float_as_uint(x[2 * i]), 0x07060302u);
-    mid[i] = __builtin_amdgcn_perm(m[2 * i + 1], m[2 * i], 0x07060302u);
-    lo[i] = __builtin_amdgcn_perm(l[2 * i + 1], l[2 * i], 0x07060302u);
+    unsigned h, m, l;
+    split_pair(x[2 * i], x[2 * i + 1], h, m, l);
+    hi[i] = h; mid[i] = m; lo[i] = l;
   }
 }
 

@@ -643,17 +643,7 @@ __global__ __launch_bounds__(kThreads, (MT == 1 ? 3 : 2)) void wgrad_stream_kern
       unsigned P[3][8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        unsigned h[2], m[2], l[2];
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          const float x = xr.v[k][2 * q + b];
-          const float r1 = x - __uint_as_float(__float_as_uint(x) & 0xFFFF0000u);
-          const float r2 = r1 - __uint_as_float(__float_as_uint(r1) & 0xFFFF0000u);
-          h[b] = __float_as_uint(x); m[b] = __float_as_uint(r1); l[b] = __float_as_uint(r2);
-        }
-        P[0][q] = __builtin_amdgcn_perm(h[1], h[0], 0x07060302u);
-        P[1][q] = __builtin_amdgcn_perm(m[1], m[0], 0x07060302u);
-        P[2][q] = __builtin_amdgcn_perm(l[1], l[0], 0x07060302u);
+        split_pair(xr.v[k][2 * q], xr.v[k][2 * q + 1], P[0][q], P[1][q], P[2][q]);
       }
       // positions the group before already covers become zeros (pairs 2 i, 2 i + 1 of the fragment)
       const int dead = t_dead[k];

@@ -415,17 +415,23 @@ const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).
  *   MELLIN_MATH_BF16X3 (default)  every fp32 operand is taken as the exact sum of three
- *     bf16 values (8 + 8 + 8 significant bits) and a product as the sum of the six largest
- *     of the nine bf16 cross products, which the bf16 matrix instructions form exactly and
- *     accumulate in fp32; what is dropped is below 2^-24 of the product, i.e. below the
- *     rounding of an fp32 multiply-add.  Storage, accumulation and results are fp32.
+ *     bf16 values (hi = the operand rounded to the nearest bf16, mid = the remainder rounded
+ *     likewise, lo = what is left, exactly) and a product as the sum of the six largest of the
+ *     nine bf16 cross products, which the bf16 matrix instructions form exactly and accumulate
+ *     in fp32.  The three dropped products (mid lo, lo mid, lo lo) are together at most
+ *     1.01 * 2^-23 of the product in the worst case: two roundings of an fp32 multiply.
+ *     Storage, accumulation and results are fp32.
  *   MELLIN_MATH_FP32  the fp32 matrix instructions (v_mfma_f32_32x32x2_f32), one sixth of
  *     the multiply rate.
  *   MELLIN_MATH_BF16X3_ALWAYS  as MELLIN_MATH_BF16X3, also for layers so small that the
  *     default leaves them on the fp32 instructions because those are faster there (layers
  *     staged in chunks of channels under 0.8 GMAC): for tests and comparisons.
- * Kernels that have no bf16 form yet run in fp32 under any setting.  Infinities in
- * the operands give NaN under the bf16 modes (inf - inf while splitting). */
+ * Kernels that have no bf16 form yet run in fp32 under any setting.
+ * Where the two modes differ on non-finite operands: an operand that rounds to an infinite
+ * bf16 (+-infinity, and finite values above 3.3895e38 in magnitude) gives NaN results under
+ * the bf16 modes (inf - inf while the operand is cut into parts), where fp32 multiply-add and
+ * the reference give +-infinity (or NaN only when infinities of both signs, or infinity and
+ * zero, meet).  NaN operands give NaN under every mode. */
 #define MELLIN_MATH_FP32 0
 #define MELLIN_MATH_BF16X3 1
 #define MELLIN_MATH_BF16X3_ALWAYS 2

@@ -8,8 +8,12 @@ against the float64 checker), and the bf16x3 mode must not be the less accurate 
 beyond noise: its error against the float64 checker is held to 2 x the fp32 mode's on the
 benchmark's layer (all three passes of both layer kinds; measured 0.7-1.1 x for the forward
 pass and the input gradient and 1.3-1.7 x for the weight gradient, whose 30 000-term sums
-are rounded in a different order, both an eighth of the tolerance or less).  Every call goes
-through the C ABI.
+are rounded in a different order, both an eighth of the tolerance or less).  The parts are
+rounded to nearest, which bounds what the three dropped cross products can amount to by
+1.01 * 2^-23 of a product; a second test feeds operands whose mantissas make the parts as
+large as they can be, all of one sign so that nothing cancels, and checks every output
+against that bound.  A third pins what the two modes do with infinite and NaN operands.
+Every call goes through the C ABI.
 """
 import numpy as np
 import pytest
@@ -125,3 +129,95 @@ def test_fp32_mode_keeps_every_kernel_covered(case, math):
     assert_close(out, exp, c_in * nf[0] * nf[1], "out")
     assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input")
     assert_close(gw, egw, n * nh[0] * nh[1], "grad_weight")
+
+
+def _adversarial(rng, shape, scale_exp):
+    """Positive fp32 values whose 24-bit mantissas maximise the mid and lo parts of the three-way
+    bf16 split (all ones; a half-way case after 8 bits and again after 16; alternating runs) mixed
+    with random ones, exponents spread over eight binades."""
+    patterns = np.array([0x7FFFFF, 0x00FFFF, 0x008080, 0x7F8080, 0x00807F, 0x7F7F7F, 0x00C0C0, 0x40FF7F,
+                         0x0080FF, 0x7FFF80, 0x3F80C0, 0x00FF80], dtype=np.uint32)
+    n = int(np.prod(shape))
+    mant = patterns[rng.integers(0, len(patterns), n)]
+    rnd = rng.integers(0, 1 << 23, n).astype(np.uint32)
+    mant = np.where(rng.random(n) < 0.25, rnd, mant)
+    expo = (127 + scale_exp + rng.integers(-4, 4, n)).astype(np.uint32)
+    return ((expo << 23) | mant).view(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("name", ["mconv2d", "lconv2d"])
+def test_worst_case_mantissas_stay_inside_the_stated_bound(name):
+    """All three passes on operands built to make the dropped cross products as large as the
+    split allows, every product positive.  Each result must meet the operator tolerance against
+    the float64 checker AND lie within (1.01 * 2^-23 + terms * 2^-24) * sum |w x| of it: the
+    dropped products plus one fp32 rounding per accumulated term.  The bf16x3 mode must also be
+    no less accurate than the fp32 instructions here (rms, factor 2)."""
+    kind_x, fwd, bwd = KINDS[name]
+    rng = np.random.default_rng(21)
+    n, c_in, c_out, nf, ng = 2, 3, 64, (8, 4), (80, 41)
+    x = _adversarial(rng, (n, c_in) + ng, 0)
+    w = _adversarial(rng, (c_out, c_in) + nf, -6)
+    b = np.zeros(c_out, np.float32)
+    exp = fwd(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64))
+    nh = exp.shape[2:]
+    go = _adversarial(rng, (n, c_out) + nh, 0)
+    egi, egw, _ = bwd(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64))
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), (0, 0), (1, 1))
+    fans = (c_in * 32, c_out * 32, n * nh[0] * nh[1])
+    rms = {}
+    for math in (hip.MATH_FP32, hip.MATH_BF16X3):
+        out, gi, gw, used = _run(kind_x, math, x, w, b, go, dims)
+        for got, e, fan, what in ((out, exp, fans[0], "out"), (gi, egi, fans[1], "grad_input"),
+                                  (gw, egw, fans[2], "grad_weight")):
+            assert_close(got, e, fan, "%s %s math %d" % (name, what, math))
+            err = np.abs(got.astype(np.float64) - e)
+            # every term is positive: sum |w x| is the exact result itself
+            bound = (1.01 * 2.0 ** -23 + fan * 2.0 ** -24) * e + 2.0 ** -149
+            worst = float(np.max(err / bound))
+            assert worst <= 1.0, (name, what, math, "error / bound = %.3f" % worst)
+            rms[(math, what)] = float(np.sqrt(np.mean((err / np.maximum(e, 1e-300)) ** 2)))
+    for what in ("out", "grad_input", "grad_weight"):
+        fp32, split = rms[(hip.MATH_FP32, what)], rms[(hip.MATH_BF16X3, what)]
+        assert split <= 2.0 * fp32 + 2.0 ** -24, (name, what, "relative rms fp32 %.3e bf16x3 %.3e" % (fp32, split))
+        print("%s %s: relative rms error against float64  fp32 %.3e  bf16x3 %.3e" % (name, what, fp32, split))
+
+
+@pytest.mark.parametrize("name", ["mconv2d", "lconv2d"])
+def test_infinite_and_nan_operands(name):
+    """Where the bf16x3 mode differs from the reference: an infinite input value.  The fp32
+    matrix instructions (and the reference's multiply-adds) carry it to +-inf in every output
+    that has a tap on it; cutting it into bf16 parts forms inf - inf, so the bf16x3 mode gives
+    NaN in exactly those outputs.  Outputs without a tap on it are untouched in both modes, and
+    a NaN input gives NaN in its outputs under both."""
+    kind_x, fwd, _ = KINDS[name]
+    rng = np.random.default_rng(22)
+    n, c_in, c_out, nf, ng = 2, 3, 64, (8, 4), (72, 41)
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float32)
+    w = rng.uniform(0.01, 0.1, (c_out, c_in) + nf).astype(np.float32)      # no zero weight: inf * w is never NaN
+    b = rng.standard_normal(c_out).astype(np.float32)
+    x[0, 1, 11, 7] = np.inf
+    x[1, 2, 23, 30] = -np.inf
+    x[1, 0, 5, 20] = np.nan
+    with np.errstate(invalid="ignore"):
+        exp = fwd(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64))
+    nh = exp.shape[2:]
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, (1, 1), (1, 1), (0, 0), (1, 1))
+    touched = ~np.isfinite(exp)
+    assert touched.any() and not touched.all()
+    for math in (hip.MATH_FP32, hip.MATH_BF16X3):
+        hip.set_math(math)
+        try:
+            out = torch.full(exp.shape, 7.0, device="cuda")
+            hip.corr2d_forward(kind_x, to_gpu(x), to_gpu(w), to_gpu(b), out, dims)
+            assert hip.last_math() == math
+            got = to_np(out)
+        finally:
+            hip.set_math(hip.MATH_BF16X3)
+        fan = c_in * nf[0] * nf[1]
+        np.testing.assert_allclose(got[~touched], exp[~touched].astype(np.float32), rtol=1e-5, atol=1e-5 * fan ** 0.5)
+        if math == hip.MATH_FP32:
+            # the reference's behaviour: the same infinities and NaNs in the same places
+            assert np.array_equal(np.isnan(got), np.isnan(exp))
+            assert np.array_equal(got[np.isinf(exp)], exp[np.isinf(exp)].astype(np.float32))
+        else:
+            assert np.isnan(got[touched]).all()

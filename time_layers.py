@@ -87,7 +87,11 @@ def run_cfg3(reps, dtype):
         print(json.dumps(rec), flush=True)
 
 
-def run_cfg4(reps, dtype):
+def _emit(rec):
+    print(json.dumps(rec), flush=True)
+
+
+def run_cfg4(reps, dtype, emit=_emit):
     import torch
     import _mellin_hip as hip
     gen = torch.Generator(device="cuda").manual_seed(3)
@@ -97,7 +101,7 @@ def run_cfg4(reps, dtype):
     b = ((torch.rand(256, device="cuda", generator=gen) * 2 - 1) * bound).to(dtype)
     for kind, name in ((hip.AX_LCORR, "lconv2d"), (hip.AX_MCORR, "mconv2d")):
         rec, _ = time_layer("cfg4 " + name, kind, x, w, b, (1, 1), (2, 1), (2, 1), (2, 1), reps)
-        print(json.dumps(rec), flush=True)
+        emit(rec)
 
 
 def run_cfg2(reps, dtype):
@@ -117,7 +121,7 @@ def run_cfg2(reps, dtype):
                     print(json.dumps(rec), flush=True)
 
 
-def run_stack(reps, dtype):
+def run_stack(reps, dtype, emit=_emit, per_layer=True):
     import time
     import torch
     import _mellin_hip as hip
@@ -144,15 +148,16 @@ def run_stack(reps, dtype):
             step()
         torch.cuda.synchronize()
         name = "mellin" if mellin else "linear"
-        print(json.dumps({"stack": name, "forward_backward_ms": round((time.perf_counter() - t0) / reps * 1e3, 2)}),
-              flush=True)
+        emit({"stack": name, "forward_backward_ms": round((time.perf_counter() - t0) / reps * 1e3, 2)})
+        if not per_layer:
+            continue
         h = x.detach().to(dtype)
         for no, (lay, conv) in enumerate(zip(stack.plan, stack.convs), 1):
             kind = hip.AX_MCORR if lay["kind"] == "mcorrlcorr" else hip.AX_LCORR
             rec, out = time_layer("%s stack layer %d" % (name, no), kind, h, conv.weight.detach().to(dtype),
                                   conv.bias.detach().to(dtype) if conv.bias is not None else None,
                                   lay["s"], lay["d"], lay["p"], lay["r"], reps)
-            print(json.dumps(rec), flush=True)
+            emit(rec)
             h = torch.relu(out)
             if lay["pool"]:
                 h = torch.nn.functional.max_pool2d(h, (1, 2))
