@@ -55,27 +55,34 @@ def test_cfg2_1d_forward_backward(s, d, p, variant):
     x = x * (torch.arange(L)[None, None, :] < lens[:, None, None])
     bound = (c_in * k) ** -0.5
     w, b = _uniform(gen, (c_out, c_in, k), bound), _uniform(gen, (c_out,), bound)
-    for op, nb in (("mcorr1d", n), ("lcorr1d", 8)):       # the linear case on 8 utterances
-        xs = x[:nb].contiguous()
-        xt = xs.to(dev()).requires_grad_(True)
+    for op in ("mcorr1d", "lcorr1d"):
+        # the GPU runs all 32 utterances of both layer kinds; for the linear one (eight times the
+        # outputs) the checker covers the output and the input gradient of the first 8 utterances
+        # and the weight / bias gradients (sums over the whole batch) of the first 16 channels
+        xt = x.to(dev()).requires_grad_(True)
         wt, bt = w.to(dev()).requires_grad_(True), b.to(dev()).requires_grad_(True)
         out = getattr(mconv, op)(xt, wt, bt, s, d, p)
         go = torch.randn(out.shape, generator=gen)
         out.backward(go.to(dev()))
-        if op == "mcorr1d":
-            exp = oracle.mcorr1d(xs.numpy(), w.numpy(), b.numpy(), s, d, p)
-            gi, gw, gb = oracle.mcorr1d_backward(*f64(xs.numpy(), w.numpy(), go.numpy()), s, d, p)
-        else:
-            exp = oracle.lcorrlcorr(xs.numpy()[..., None], w.numpy()[..., None], b.numpy(),
-                                    (s, 1), (d, 1), (p, 0))[..., 0]
-            gi, gw, gb = oracle.lcorrlcorr_backward(*f64(xs.numpy()[..., None], w.numpy()[..., None],
-                                                         go.numpy()[..., None]), (s, 1), (d, 1), (p, 0))
-            gi, gw = gi[..., 0], gw[..., 0]
         tag = "cfg2 %s s=%d d=%d p=%d" % (op, s, d, p)
-        assert_close(out, exp, c_in * k, tag + " out")
-        assert_close(xt.grad, gi, c_out * k, tag + " grad_input")
-        assert_close(wt.grad, gw, nb * exp.shape[2], tag + " grad_weight")
-        assert_close(bt.grad, gb, nb * exp.shape[2], tag + " grad_bias")
+        if op == "mcorr1d":
+            exp = oracle.mcorr1d(x.numpy(), w.numpy(), b.numpy(), s, d, p)
+            gi, gw, gb = oracle.mcorr1d_backward(*f64(x.numpy(), w.numpy(), go.numpy()), s, d, p)
+            nb, mc = n, c_out
+        else:
+            nb, mc = 8, 16
+            xs = x[:nb].numpy()
+            exp = oracle.lcorrlcorr(xs[..., None], w.numpy()[..., None], b.numpy(), (s, 1), (d, 1), (p, 0))[..., 0]
+            gi, _, _ = oracle.lcorrlcorr_backward(*f64(xs[..., None], w.numpy()[..., None],
+                                                       go[:nb].numpy()[..., None]), (s, 1), (d, 1), (p, 0))
+            _, gw, gb = oracle.lcorrlcorr_backward(*f64(x.numpy()[..., None], w[:mc].numpy()[..., None],
+                                                        go[:, :mc].contiguous().numpy()[..., None]), (s, 1), (d, 1), (p, 0))
+            gi, gw = gi[..., 0], gw[..., 0]
+        assert tuple(out.shape[:2]) == (n, c_out)
+        assert_close(out[:nb], exp, c_in * k, tag + " out")
+        assert_close(xt.grad[:nb], gi, c_out * k, tag + " grad_input")
+        assert_close(wt.grad[:mc], gw, n * exp.shape[2], tag + " grad_weight")
+        assert_close(bt.grad[:mc], gb, n * exp.shape[2], tag + " grad_bias")
 
 
 def _cfg3(gen):
