@@ -55,6 +55,7 @@ for _t in ("f32", "f16"):
     SYMBOLS["mellin_pool_pairs_forward_" + _t] = (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr])
     SYMBOLS["mellin_pool_pairs_backward_" + _t] = (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr])
 SYMBOLS["mellin_static_scratch_bytes"] = (_size_t, [])
+SYMBOLS["mellin_static_scratch_prepare"] = (_int, [])
 SYMBOLS["mellin_corr2d_backward_weight_static_f32"] = (_int, [_int, _ptr, _ptr] + _DIMS + [_ptr, _ptr])
 for _n in ("forward", "backward_input", "backward_weight"):
     SYMBOLS["mellin_corr2d_%s_f16_workspace" % _n] = (_size_t, [_int] + _DIMS)

@@ -802,13 +802,25 @@ const int kMaxDevices = 64;
 void *g_scratch_addr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-void *static_scratch(const char *fn) {
+// stream: the stream the caller is about to launch on, or null when only the lookup is asked
+// for; a lookup that has not been made yet is refused while that stream is capturing a graph
+// (it loads the code object, which a capture does not allow)
+void *static_scratch(const char *fn, hipStream_t stream = nullptr, bool check_capture = false) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) { fail(MELLIN_ERR_RUNTIME, "%s: hipGetDevice: %s", fn, hipGetErrorString(e)); return nullptr; }
   if (dev < 0 || dev >= kMaxDevices) { fail(MELLIN_ERR_RUNTIME, "%s: device index %d out of range", fn, dev); return nullptr; }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_addr[dev]) {
+    if (check_capture) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
+        fail(MELLIN_ERR_RUNTIME, "%s: the static scratch array of this device has not been looked up yet and the "
+             "stream is capturing a graph; call mellin_static_scratch_prepare() before the capture begins", fn);
+        return nullptr;
+      }
+      (void)hipGetLastError();
+    }
     void *ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr) {
@@ -1468,6 +1480,7 @@ int mellin_corr2d_backward_weight_f32(int kind_x, const float *input,
                                        grad_weight, workspace, workspace_bytes, stream);
 }
 size_t mellin_static_scratch_bytes(void) { return MELLIN_STATIC_SCRATCH_BYTES; }
+int mellin_static_scratch_prepare(void) { return static_scratch(__func__) ? MELLIN_OK : MELLIN_ERR_RUNTIME; }
 int mellin_corr2d_backward_weight_static_f32(int kind_x, const float *input, const float *grad_out,
                                              MELLIN_CORR2D_DIMS, float *grad_weight, void *stream) {
   const size_t need = mellin_corr2d_backward_weight_workspace(kind_x, 4, CORR2D_ARGS);
@@ -1476,7 +1489,7 @@ int mellin_corr2d_backward_weight_static_f32(int kind_x, const float *input, con
                 "%s: this layer needs %zu bytes of scratch memory, the static array holds %zu; use "
                 "mellin_corr2d_backward_weight_f32 with a workspace", __func__, need,
                 (size_t)MELLIN_STATIC_SCRATCH_BYTES);
-  void *ws = static_scratch(__func__);
+  void *ws = static_scratch(__func__, (hipStream_t)stream, true);
   if (!ws) return MELLIN_ERR_RUNTIME;
   return corr2d_backward_weight<float>(__func__, kind_x, input, grad_out, CORR2D_ARGS, grad_weight, ws,
                                        MELLIN_STATIC_SCRATCH_BYTES, stream);

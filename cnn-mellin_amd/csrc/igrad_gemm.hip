@@ -431,9 +431,9 @@ template <int KSTEPS, int NT, bool PIPE>
 hipError_t launch_instance(const IgradPlan &pl, const float *w, const float *go, float *gi,
                            float *ws, hipStream_t stream) {
   auto kern = igrad_kernel<KSTEPS, NT, PIPE>;
-  if (pl.lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)pl.lds_bytes);
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, pl.lds_bytes, lds_allowed);
     if (e != hipSuccess) return e;
   }
   const int groups = (pl.batch + pl.jobs - 1) / pl.jobs;
@@ -807,9 +807,9 @@ template <int MTT, int NT, bool F16 = false>
 hipError_t launch_stream_instance(const IgradPlan &pl, const void *w, const void *go, void *gi,
                                   float *ws, hipStream_t stream) {
   auto kern = igrad_stream_kernel<MTT, NT, F16>;
-  if (pl.lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)pl.lds_bytes);
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, pl.lds_bytes, lds_allowed);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)(pl.batch * pl.strips)), dim3(256), pl.lds_bytes, stream, pl, w, go, gi,
@@ -993,9 +993,9 @@ template <int KSTEPS>
 hipError_t launch_tap_product_instance(const TapProductPlan &pl, const float *w, const float *go,
                                        float *z, hipStream_t stream) {
   auto kern = pl.yfold ? tap_product_kernel<KSTEPS, true> : tap_product_kernel<KSTEPS, false>;
-  if (pl.lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)pl.lds_bytes);
+  {
+    static std::atomic<int> lds_allowed[2] = {{0}, {0}};   // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, pl.lds_bytes, lds_allowed[pl.yfold ? 1 : 0]);
     if (e != hipSuccess) return e;
   }
   const int groups_x = pl.yfold ? (pl.nhx + pl.rows_wg - 1) / pl.rows_wg : (pl.chunks_per_image + pl.cpw - 1) / pl.cpw;

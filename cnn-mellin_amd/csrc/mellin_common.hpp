@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace mellin {
 
 typedef int64_t i64;
@@ -117,6 +119,18 @@ inline Axis make_axis(int kind, i64 nf, i64 ng, i64 nh, i64 s, i64 d, i64 p, i64
   const i64 sup = support_size(kind, nf, ng, s, d, p, u);
   a.nh_eff = sup < nh ? sup : nh;
   return a;
+}
+
+// Opt a kernel in to more dynamic LDS than a launch gets by default (asked for from 48 KB on).  The attribute belongs to the
+// function, for the whole process, while launches come from any thread (PyTorch runs backward
+// passes on a thread of its own): it is set once per kernel instance, to all a CU has (160 KB on
+// gfx950), so that no later launch with another size on another thread can find it too small.
+// `done`: one flag per kernel instance.
+inline hipError_t allow_large_lds(const void *kernel, size_t lds_bytes, std::atomic<int> &done) {
+  if (lds_bytes <= 48 * 1024 || done.load(std::memory_order_acquire)) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess) done.store(1, std::memory_order_release);
+  return e;
 }
 
 // ---- launchers (each returns the hipError_t of the launch) ----------------

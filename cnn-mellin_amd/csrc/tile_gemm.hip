@@ -571,15 +571,10 @@ hipError_t launch_variant(const TilePlan &pl, size_t lds_bytes, dim3 grid, const
                           const float *g, const float *bias, float *h, hipStream_t stream,
                           const float *af = nullptr) {
   auto kern = tile_gemm_kernel<MT, NT, ACC, MB, HOUT, SPLIT>;
-  if (lds_bytes > 64 * 1024) {
-    // opt in to more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per CU)
-    static thread_local size_t granted = 0;
-    if (granted < lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, pl, f, g, bias, h, af);
   return hipGetLastError();
@@ -589,14 +584,10 @@ template <int MT, int NT, bool HOUT, int SPLIT>
 hipError_t launch_classes_variant(const ClassLaunch &args, size_t lds_bytes, dim3 grid, const float *f, const float *g,
                                   const float *bias, float *h, hipStream_t stream, const float *af) {
   auto kern = tile_gemm_classes_kernel<MT, NT, HOUT, SPLIT>;
-  if (lds_bytes > 64 * 1024) {
-    static thread_local size_t granted = 0;
-    if (granted < lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, args, f, g, bias, h, af);
   return hipGetLastError();

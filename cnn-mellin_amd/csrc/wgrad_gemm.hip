@@ -813,14 +813,10 @@ template <int MT, int JT, int NT>
 hipError_t launch_variant(const WgradPlan &wp, size_t lds_bytes, dim3 grid, const float *a,
                           const float *g, float *ws, hipStream_t stream) {
   auto kern = wgrad_gemm_kernel<MT, JT, NT>;
-  if (lds_bytes > 64 * 1024) {
-    static thread_local size_t granted = 0;
-    if (granted < lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, wp, a, g, ws);
   return hipGetLastError();
@@ -830,14 +826,10 @@ template <int MT, int JT>
 hipError_t launch_rows(const WgradPlan &wp, dim3 grid, const float *a, const float *g, float *ws,
                        hipStream_t stream) {
   auto kern = wgrad_rows_kernel<MT, JT>;
-  if (wp.lds_bytes > 64 * 1024) {
-    static thread_local size_t granted = 0;
-    if (granted < wp.lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)wp.lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = wp.lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, wp.lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
   return hipGetLastError();
@@ -847,14 +839,10 @@ template <int MT, int JT>
 hipError_t launch_stream(const WgradPlan &wp, dim3 grid, const float *a, const float *g, float *ws,
                          hipStream_t stream) {
   auto kern = wgrad_stream_kernel<MT, JT>;
-  if (wp.lds_bytes > 64 * 1024) {
-    static thread_local size_t granted = 0;
-    if (granted < wp.lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)wp.lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = wp.lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, wp.lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
   return hipGetLastError();

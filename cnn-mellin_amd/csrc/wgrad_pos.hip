@@ -288,14 +288,10 @@ template <int JT, bool F16>
 hipError_t launch_pos(const WgradPosPlan &wp, dim3 grid, const void *a, const void *g, float *ws,
                       hipStream_t stream) {
   auto kern = wgrad_pos_kernel<JT, F16>;
-  if (wp.lds_bytes > 64 * 1024) {
-    static thread_local size_t granted = 0;
-    if (granted < wp.lds_bytes) {
-      hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)wp.lds_bytes);
-      if (e != hipSuccess) return e;
-      granted = wp.lds_bytes;
-    }
+  {
+    static std::atomic<int> lds_allowed{0};                // (one per kernel instance)
+    hipError_t e = allow_large_lds((const void *)kern, wp.lds_bytes, lds_allowed);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), wp.lds_bytes, stream, wp, a, g, ws);
   return hipGetLastError();

@@ -170,12 +170,17 @@ int mellin_corr2d_backward_weight_f64(int kind_x, const double *input,
  * of a caller's workspace: the call allocates and frees nothing.  Layers whose
  * partial sums need more (mellin_corr2d_backward_weight_workspace() tells) are
  * rejected with MELLIN_ERR_WORKSPACE.  The array's address is looked up on the
- * first call made with a device current (not an allocation; make that call
- * before capturing a graph).  All calls on one GPU share the array: its
+ * first call made with a device current (not an allocation, but it loads the
+ * code object, which a graph capture does not allow):
+ * mellin_static_scratch_prepare() does only that lookup for the current device,
+ * for callers to run once before they capture; a first call on a stream that is
+ * already capturing is refused with MELLIN_ERR_RUNTIME and a message that says
+ * so.  All calls on one GPU share the array: its
  * contents never need clearing (every word read was written by the same
  * call), but two calls that overlap in time on one GPU (different streams or
  * threads) race and give wrong results; serialise them. */
 size_t mellin_static_scratch_bytes(void);
+int mellin_static_scratch_prepare(void);
 int mellin_corr2d_backward_weight_static_f32(int kind_x, const float *input,
                                              const float *grad_out,
                                              MELLIN_CORR2D_DIMS,
@@ -458,7 +463,10 @@ int mellin_last_math(void);
  * columns of a filter row in the kernel; "whole-classes": automatic choice, but a class's rows are never cut
  * into ranges by where the filter rows' taps leave the signal; "class-launches":
  * like "classes", with a launch per class also where one launch would hold them).
- * Unknown names are rejected with MELLIN_ERR_ARGUMENT. */
+ * Unknown names are rejected with MELLIN_ERR_ARGUMENT and change nothing.  The setting (like
+ * mellin_set_math's) is several process-wide words: change it while no operator-level call
+ * of the process is running, or a call may see part of the old and part of the new one (a
+ * workspace query and the call that follows it can then disagree: MELLIN_ERR_WORKSPACE). */
 int mellin_set_variant(const char *name);
 
 #ifdef __cplusplus

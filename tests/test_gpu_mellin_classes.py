@@ -258,3 +258,50 @@ def test_large_input_gradients_take_the_filter_rows_by_default():
 def test_some_input_gradient_took_the_classes():
     """(after the parametrized cases of this file: tests run in the order they are written)"""
     assert "mfma-classes" in seen_gi, seen_gi
+
+
+# Up-sampling on the Mellin axis (u > 1) together with strides and dilations above one: the
+# residue classes, where a class's rows are cut (h_f = floor((ng - 1 + u)(p + 1) / (f + d)) - s)
+# and the rows of a filter row's first pass all carry u.
+U_CASES = [
+    # (n, c_in, c_out, nf, ng, s, d, p, u, r)
+    (2, 40, 48, (4, 3), (50, 9), (2, 1), (2, 1), (2, 1), (2, 1), (6, 0)),      # u = 2, s = d = 2, three classes
+    (2, 64, 40, (5, 2), (40, 7), (3, 1), (1, 1), (3, 0), (3, 1), (0, 1)),      # u = 3, s = 3, four classes
+    (1, 32, 33, (6, 2), (45, 5), (2, 1), (3, 1), (1, 0), (3, 2), (4, 0)),      # u = (3, 2), d = 3, two classes
+    # rows far past the support of the later filter rows: the classes are cut into ranges
+    (2, 32, 64, (4, 4), (60, 6), (1, 1), (1, 1), (1, 1), (2, 1), (50, 0)),
+    (2, 48, 64, (4, 2), (70, 8), (2, 1), (2, 1), (1, 0), (3, 1), (40, 0)),
+]
+
+seen_u = []
+
+
+@pytest.mark.parametrize("case", U_CASES, ids=[str(i) for i in range(len(U_CASES))])
+def test_classes_with_upsampling_match_checker(case, classes_forced):
+    n, c_in, c_out, nf, ng, s, d, p, u, r = case
+    rng = np.random.default_rng(3300 + U_CASES.index(case))
+    x = rng.standard_normal((n, c_in) + ng).astype(np.float32)
+    w = (rng.standard_normal((c_out, c_in) + nf) * (c_in * nf[0] * nf[1]) ** -0.5).astype(np.float32)
+    b = rng.standard_normal(c_out).astype(np.float32)
+    exp = oracle.mcorrlcorr(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64), s, d, p, u, r)
+    nh = exp.shape[2:]
+    assert min(nh) > 0
+    go = rng.standard_normal((n, c_out) + nh).astype(np.float32)
+    egi, egw, _ = oracle.mcorrlcorr_backward(x.astype(np.float64), w.astype(np.float64), go.astype(np.float64),
+                                             s, d, p, u)
+    dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, p, u)
+    out = torch.full(exp.shape, float("nan"), device="cuda")                 # every word must be written
+    hip.corr2d_forward(hip.AX_MCORR, to_gpu(x), to_gpu(w), to_gpu(b), out, dims)
+    assert hip.last_variant() == "mfma-classes", case
+    assert_close(out, exp, c_in * nf[0] * nf[1], "forward %s" % (case,))
+    gi = torch.full(x.shape, float("nan"), device="cuda")
+    hip.corr2d_backward_input(hip.AX_MCORR, to_gpu(w), to_gpu(go), gi, dims)
+    seen_u.append(hip.last_variant())
+    assert_close(gi, egi, c_out * nf[0] * nf[1], "grad_input [%s] %s" % (hip.last_variant(), case))
+    gw = torch.full(w.shape, float("nan"), device="cuda")
+    hip.corr2d_backward_weight(hip.AX_MCORR, to_gpu(x), to_gpu(go), gw, dims)
+    assert_close(gw, egw, n * nh[0] * nh[1], "grad_weight [%s] %s" % (hip.last_variant(), case))
+
+
+def test_some_upsampled_input_gradient_took_the_filter_rows():
+    assert "mfma-filter-rows+fold" in seen_u, seen_u

@@ -52,6 +52,13 @@ def test_static_scratch_matches_workspace_entry_point_twice():
         assert_close(got, exp, n * nh[0] * nh[1], "static weight gradient, case %d" % seed)
 
 
+def test_prepare_does_the_lookup_alone():
+    """mellin_static_scratch_prepare(): the address lookup without a layer (what a caller runs
+    before capturing a graph); it may be called any number of times."""
+    assert hip.lib.mellin_static_scratch_prepare() == 0
+    assert hip.lib.mellin_static_scratch_prepare() == 0
+
+
 def test_layer_beyond_the_static_array_is_refused():
     # 1024 x 272 channels of 4 x 4 taps: the partial sums of one split alone pass 16 MiB
     n, c_in, c_out, nf, ng = 1, 272, 1024, (4, 4), (8, 8)
