@@ -13,6 +13,7 @@
 #include "mellin_common.hpp"
 #include "igrad_gemm.hpp"
 #include "tile_gemm.hpp"
+#include "gather_kernels.hpp"
 
 using namespace mellin;
 
@@ -34,6 +35,7 @@ std::atomic<int> g_split_classes{0};    // ... every class a launch of its own (
 std::atomic<int> g_all_classes{0};      // ... one per class whatever the layer's size ("classes": for tests)
 std::atomic<int> g_no_yfold{0};         // tap products stored per filter column, not summed over them ("tap-columns": for comparisons)
 std::atomic<int> g_whole_classes{0};    // ... a class's rows never cut into ranges ("whole-classes": for comparisons)
+std::atomic<int> g_gather{0};          // 1: the LDS-gather kernels (vector ALUs) wherever they apply ("lds-gather"); -1: never ("no-gather")
 std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
@@ -254,6 +256,12 @@ hipError_t launch_mellin_classes(const ClassPlans &cp, const void *f, const void
   return hipSuccess;
 }
 
+// Where the gather kernel is the faster forward pass (measured on the benchmark's layers): TBD
+bool gather_forward_wins(const SepConv &pr) {
+  (void)pr;
+  return false;
+}
+
 template <>
 hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
                               const float *bias, float *h, hipStream_t stream, void *frag_ws,
@@ -268,6 +276,15 @@ hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
       g_variant = "mfma-classes";
       g_last_math = MATH_BF16X3;
       return launch_mellin_classes(cp, f, g, bias, h, stream, frag_ws, frag_bytes);
+    }
+  }
+  if (g_forced == 0 && g_gather >= 0) {
+    // few input channels and a small layer: the vector-ALU gather kernel (gather_kernels.hip)
+    GatherPlan gp;
+    if ((g_gather > 0 || gather_forward_wins(pr)) && make_gather_forward_plan(pr, gp)) {
+      g_variant = "lds-gather";
+      g_last_math = MATH_FP32;
+      return launch_gather_forward(gp, f, g, bias, h, stream);
     }
   }
   if (g_forced != 1) {
@@ -1360,8 +1377,8 @@ int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
   // the name is parsed first: an unknown one changes nothing
-  struct Setting { int forced, widen, no_classes, all_classes, split_classes, whole_classes, no_yfold;  };
-  Setting v = {0, 0, 0, 0, 0, 0, 0};
+  struct Setting { int forced, widen, no_classes, all_classes, split_classes, whole_classes, no_yfold, gather; };
+  Setting v = {0, 0, 0, 0, 0, 0, 0, 0};
   if (!name || !*name || !strcmp(name, "auto")) {}
   else if (!strcmp(name, "generic")) v.forced = 1;
   else if (!strcmp(name, "two-pass")) v.forced = 2;
@@ -1371,6 +1388,8 @@ int mellin_set_variant(const char *name) {
   else if (!strcmp(name, "class-launches")) { v.all_classes = 1; v.split_classes = 1; }
   else if (!strcmp(name, "whole-classes")) v.whole_classes = 1;
   else if (!strcmp(name, "tap-columns")) v.no_yfold = 1;
+  else if (!strcmp(name, "lds-gather")) v.gather = 1;
+  else if (!strcmp(name, "no-gather")) v.gather = -1;
   else return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
   g_widen = v.widen;
   g_no_classes = v.no_classes;
@@ -1378,6 +1397,7 @@ int mellin_set_variant(const char *name) {
   g_split_classes = v.split_classes;
   g_whole_classes = v.whole_classes;
   g_no_yfold = v.no_yfold;
+  g_gather = v.gather;
   g_forced = v.forced;
   return MELLIN_OK;
 }

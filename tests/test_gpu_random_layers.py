@@ -192,3 +192,9 @@ def test_accumulate_into_h():
         done += 1
     print("accumulate: %d calls in %.1f s" % (done, time.time() - t0))
     assert done >= MIN_COUNT
+
+
+def test_lds_gather_kernels_forced():
+    """The vector-ALU gather kernels wherever they apply (few input channels, unit y stride and dilation)."""
+    v = _sweep(110, "few-channels", variant="lds-gather")
+    assert v.get("lds-gather", 0) >= 20, v
