@@ -320,42 +320,57 @@ __device__ __forceinline__ void tile_gemm_body(
   auto write_tile = [&](auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     char *Himg = (char *)H + ((i64)tg.n * pl.h_n + (i64)m0 * pl.h_m) * ES;
+    bool live[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int local = (wave * NT + t) * 32 + l32;
-      bool live = local < tg.count;
+      live[t] = local < tg.count;
       if (ACC) {
         int ox, oy;
         by_noy.divmod(lane_q[t], ox, oy);
-        live = live && ox < pl.nox_eff && oy < pl.noy_eff;
+        live[t] = live[t] && ox < pl.nox_eff && oy < pl.noy_eff;
       }
-      if (!live) continue;
-      if (FULL && !ACC && buffer_stores) {
-        // One descriptor for the block's channels of this image; a lane's offset is its
-        // position plus whole groups of eight channels, the four channels inside a group
-        // are scalar offsets: a store and a quarter of a 32-bit add per word, against a
-        // store and a 64-bit add with pointers.
-        const __amdgpu_buffer_rsrc_t h_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc((void *)Himg, 0, (int)(M_T * hm1), 0x00020000);
-        int voff = (half * 4) * (int)hm1 + lane_q[t] * ES;
-        auto put = [&](float v, int soff) {
-          if constexpr (HOUT)
-            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, (_Float16)v), h_rsrc, voff, soff, 0);
-          else
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), h_rsrc, voff, soff, 0);
-        };
+    }
+    if (FULL && !ACC && buffer_stores) {
+      // One descriptor for the block's channels of this image; a lane's offset is its
+      // position plus whole groups of eight channels, the four channels inside a group
+      // are scalar offsets: a store and a quarter of a 32-bit add per word, against a
+      // store and a 64-bit add with pointers.
+      // A channel's 32-position pieces of this wavefront's position tiles go out back to
+      // back (tile innermost): the pieces are neighbours in memory and none starts on a
+      // 128-byte line, so the line two of them share is completed while the first write to
+      // it is still on its way through the CU's write path.  With the channels innermost
+      // (each tile's 64 stores, then the next tile's) the shared lines were written twice,
+      // in two parts: a store-only launch of this pattern took 36 us for the benchmark's
+      // 157 MB against 28.6 us in this order.
+      const __amdgpu_buffer_rsrc_t h_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void *)Himg, 0, (int)(M_T * hm1), 0x00020000);
+      int voff[NT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+      for (int t = 0; t < NT; ++t) voff[t] = live[t] ? (half * 4) * (int)hm1 + lane_q[t] * ES : (int)0x7FFFFFF0;   // (past the descriptor: dropped)
+      auto put = [&](float v, int vo, int soff) {
+        if constexpr (HOUT)
+          __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, (_Float16)v), h_rsrc, vo, soff, 0);
+        else
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), h_rsrc, vo, soff, 0);
+      };
 #pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            put(acc[i][t][4 * g4 + 0], 0);
-            put(acc[i][t][4 * g4 + 1], (int)hm1);
-            put(acc[i][t][4 * g4 + 2], (int)hm2);
-            put(acc[i][t][4 * g4 + 3], (int)hm3);
-            voff += (int)hm8;
-          }
-        continue;
-      }
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              put(acc[i][t][4 * g4 + r], voff[t], r == 0 ? 0 : (r == 1 ? (int)hm1 : (r == 2 ? (int)hm2 : (int)hm3)));
+#pragma unroll
+          for (int t = 0; t < NT; ++t) voff[t] += (int)hm8;
+        }
+      return;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (!live[t]) continue;
       char *o = Himg + (half * 4) * hm1 + (i64)lane_q[t] * ES;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
