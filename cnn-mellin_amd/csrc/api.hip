@@ -14,6 +14,7 @@
 #include "igrad_gemm.hpp"
 #include "tile_gemm.hpp"
 #include "gather_kernels.hpp"
+#include "narrow_gemm.hpp"
 
 using namespace mellin;
 
@@ -36,6 +37,7 @@ std::atomic<int> g_all_classes{0};      // ... one per class whatever the layer'
 std::atomic<int> g_no_yfold{0};         // tap products stored per filter column, not summed over them ("tap-columns": for comparisons)
 std::atomic<int> g_whole_classes{0};    // ... a class's rows never cut into ranges ("whole-classes": for comparisons)
 std::atomic<int> g_gather{0};          // 1: the LDS-gather kernels (vector ALUs) wherever they apply ("lds-gather"); -1: never ("no-gather")
+std::atomic<int> g_no_narrow{0};       // 1: few-channel linear forward passes through the tiled kernel ("no-narrow": for comparisons); -1: their own kernel whatever the size ("narrow": for tests)
 std::atomic<int> g_widen{0};            // half-precision entry points: always through fp32 copies (mellin_set_variant "widen")
 std::atomic<int> g_math{MATH_BF16X3};   // how fp32 products are formed on the matrix cores (mellin_set_math)
 std::atomic<int> g_last_math{MATH_FP32};   // what the kernels of the most recent operator-level call multiplied with
@@ -287,6 +289,16 @@ hipError_t run_sepconv<float>(const SepConv &pr, const float *f, const float *g,
       return launch_gather_forward(gp, f, g, bias, h, stream);
     }
   }
+  if (g_forced == 0 && g_no_narrow <= 0) {
+    // few input channels, linear axes without padding: the signal cut into bf16 parts once per
+    // staged element (narrow_gemm.hip)
+    NarrowPlan np;
+    if (make_narrow_plan(pr, np, g_no_narrow < 0)) {
+      g_variant = "mfma-narrow";
+      g_last_math = MATH_BF16X3;
+      return launch_narrow_forward(np, f, g, bias, h, stream);
+    }
+  }
   if (g_forced != 1) {
     TilePlan pl;
     size_t lds = 0;
@@ -414,8 +426,12 @@ int corr2d_forward(const char *fn, int kind_x, const T *input, const T *weight,
     TilePlan pl;
     size_t lds = 0;
     int mt = 0, nt = 0;
+    // (not where the fp32 entry point would take the few-channel kernel, which has no half-precision
+    // store: the caller rounds that kernel's fp32 result instead, so that both give the same bits)
+    NarrowPlan narrow;
+    const bool few_channels = g_forced == 0 && g_no_narrow <= 0 && g_gather <= 0 && make_narrow_plan(pr, narrow, g_no_narrow < 0);
     pr.out_half = 1;
-    if (make_tile_plan(pr, pl, &lds, &mt, &nt)) {
+    if (!few_channels && make_tile_plan(pr, pl, &lds, &mt, &nt)) {
       g_variant = "mfma";
       g_last_math = pl.split ? MATH_BF16X3 : MATH_FP32;
       if (wrote_half) *wrote_half = true;
@@ -1377,8 +1393,8 @@ int mellin_last_math(void) { return g_last_math; }
 
 int mellin_set_variant(const char *name) {
   // the name is parsed first: an unknown one changes nothing
-  struct Setting { int forced, widen, no_classes, all_classes, split_classes, whole_classes, no_yfold, gather; };
-  Setting v = {0, 0, 0, 0, 0, 0, 0, 0};
+  struct Setting { int forced, widen, no_classes, all_classes, split_classes, whole_classes, no_yfold, gather, no_narrow; };
+  Setting v = {0, 0, 0, 0, 0, 0, 0, 0, 0};
   if (!name || !*name || !strcmp(name, "auto")) {}
   else if (!strcmp(name, "generic")) v.forced = 1;
   else if (!strcmp(name, "two-pass")) v.forced = 2;
@@ -1390,6 +1406,8 @@ int mellin_set_variant(const char *name) {
   else if (!strcmp(name, "tap-columns")) v.no_yfold = 1;
   else if (!strcmp(name, "lds-gather")) v.gather = 1;
   else if (!strcmp(name, "no-gather")) v.gather = -1;
+  else if (!strcmp(name, "no-narrow")) v.no_narrow = 1;
+  else if (!strcmp(name, "narrow")) v.no_narrow = -1;
   else return fail(MELLIN_ERR_ARGUMENT, "mellin_set_variant: unknown variant '%s'", name);
   g_widen = v.widen;
   g_no_classes = v.no_classes;
@@ -1398,6 +1416,7 @@ int mellin_set_variant(const char *name) {
   g_whole_classes = v.whole_classes;
   g_no_yfold = v.no_yfold;
   g_gather = v.gather;
+  g_no_narrow = v.no_narrow;
   g_forced = v.forced;
   return MELLIN_OK;
 }

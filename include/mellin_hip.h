@@ -415,7 +415,9 @@ int mellin_pool_pairs_backward_f16(const void *grad_y, const unsigned char *whic
  * classes of a half-precision layer sharing one launch) and
  * "mfma-f16-class-launches" (a launch each),
  * "mfma-f16-fused", "mfma-f16+fold" and "mfma-f16-filter-rows+fold"
- * (half-precision tensors on the f16 matrix cores). */
+ * (half-precision tensors on the f16 matrix cores), "mfma-narrow" (forward pass
+ * of a linear x linear layer with few input channels, bf16 matrix cores) and
+ * "lds-gather" (vector-ALU forward kernel, only under mellin_set_variant). */
 const char *mellin_last_variant(void);
 
 /* How the matrix-core kernels form their fp32 products (process-wide).
@@ -462,7 +464,16 @@ int mellin_last_math(void);
  * keeps one product per filter column in its workspace instead of summing the four
  * columns of a filter row in the kernel; "whole-classes": automatic choice, but a class's rows are never cut
  * into ranges by where the filter rows' taps leave the signal; "class-launches":
- * like "classes", with a launch per class also where one launch would hold them).
+ * like "classes", with a launch per class also where one launch would hold them);
+ * "lds-gather": automatic choice, but fp32 forward passes with at most eight input
+ * channels and unit stride and dilation along y take the vector-ALU kernel that gathers
+ * its taps from LDS (reported as "lds-gather", MELLIN_MATH_FP32: the non-matrix form the
+ * matrix kernels are measured against), "no-gather": never; "no-narrow": automatic choice,
+ * but linear x linear forward passes with few input channels go through the tiled kernel
+ * instead of their own ("mfma-narrow": both axes correlations without padding or
+ * up-sampling, unit stride and dilation along y, an even number of filter columns,
+ * c_in * nfx * nfy <= 128, at least 1024 tiles of 256 positions x 64 channels), "narrow":
+ * that kernel for layers of its class however small (for tests).
  * Unknown names are rejected with MELLIN_ERR_ARGUMENT and change nothing.  The setting (like
  * mellin_set_math's) is several process-wide words: change it while no operator-level call
  * of the process is running, or a call may see part of the old and part of the new one (a

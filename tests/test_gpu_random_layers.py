@@ -33,6 +33,18 @@ OPS = {"mcorrlcorr": (hip.AX_MCORR, oracle.mcorrlcorr, oracle.mcorrlcorr_backwar
 
 def _draw(rng, family):
     """One layer: (op, n, c_in, c_out, nf, ng, s, d, p, u, r)."""
+    if family == "narrow-class":
+        # linear x linear, no padding or up-sampling, unit y stride and dilation, an even number of
+        # filter columns, at most 128 taps in all
+        c_in = int(rng.integers(1, 17))
+        nfy = int(rng.choice([2, 4, 6]))
+        nfx = int(rng.integers(1, max(2, min(9, 128 // (c_in * nfy) + 1))))
+        if c_in * nfx * nfy > 128:
+            nfx = 1
+        c_out = int(rng.choice([1, 5, 32, 33, 64, 70, 130]))
+        ng = (int(rng.integers(8, 120)), int(rng.choice([6, 7, 13, 20, 33, 41, 64])))
+        return ("lcorrlcorr", int(rng.integers(1, 5)), c_in, c_out, (nfx, nfy), ng,
+                (int(rng.integers(1, 4)), 1), (int(rng.integers(1, 4)), 1), (0, 0), (1, 1), (0, 0))
     op = ["mcorrlcorr", "lcorrlcorr"][int(rng.integers(2))]
     n = int(rng.integers(1, 7))
     if family == "few-channels":
@@ -198,3 +210,10 @@ def test_lds_gather_kernels_forced():
     """The vector-ALU gather kernels wherever they apply (few input channels, unit y stride and dilation)."""
     v = _sweep(110, "few-channels", variant="lds-gather")
     assert v.get("lds-gather", 0) >= 20, v
+
+
+def test_narrow_forward_kernel_forced():
+    """The few-channel linear forward kernel on layers of its class however small (the automatic
+    choice takes it from 1024 tiles on): partial tiles, partial channel blocks, 1-16 input channels."""
+    v = _sweep(111, "narrow-class", math=hip.MATH_BF16X3_ALWAYS, variant="narrow")
+    assert v.get("mfma-narrow", 0) >= 40, v
