@@ -588,40 +588,47 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   // row when nfy is a multiple of 4; with dy = 1 they are four consecutive words of the image,
   // reached with immediate offsets from the first
   const bool quad = (pl.nfy & 3) == 0 && pl.dy == 1;
-  auto multiply = [&](auto first_tag, int ks, const BOp &o) {
-    constexpr bool kFirst = decltype(first_tag)::value;      // an iteration's first step starts the sums from zero
-    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // A step's operands as the matrix instructions take them: the filter's fragments of the step's
+  // 16 channels and the cut grad_out values (F16: one part each, the values themselves).
+  constexpr int kParts = F16 ? 1 : 3;
+  struct AOp { uintx4 p[kParts][MTT]; };
+  struct SOp { uintx4 p[kParts][NT]; };
+  auto stage = [&](int ks, const BOp &o, AOp &a, SOp &s) {
     const uintx4 *af = Af + (2 * ks + half) * ROWS + l32;
-    if constexpr (F16) {
-      uintx4 b[NT];
+#pragma unroll
+    for (int part = 0; part < kParts; ++part)
+#pragma unroll
+      for (int m = 0; m < MTT; ++m) a.p[part][m] = af[part * af_part + m * 32];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if constexpr (F16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s.p[0][t][i] = (unsigned)o.v[t][2 * i] | ((unsigned)o.v[t][2 * i + 1] << 16);
+      } else {
+        split8(o.v[t], s.p[0][t], s.p[1][t], s.p[2][t]);
+      }
+    }
+  };
+  auto multiply = [&](const AOp &a, const SOp &s) {
+#pragma unroll
+    for (int m = 0; m < MTT; ++m)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if constexpr (F16)
+          acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a.p[0][m]),
+                                                             __builtin_bit_cast(halfx8, s.p[0][t]), acc[m][t], 0, 0, 0);
+        else
+          mfma_split6(acc[m][t], a.p[0][m], a.p[kParts > 1 ? 1 : 0][m], a.p[kParts > 1 ? 2 : 0][m],
+                      s.p[0][t], s.p[kParts > 1 ? 1 : 0][t], s.p[kParts > 1 ? 2 : 0][t]);
+      }
+  };
+  auto clear_sums = [&] {
+#pragma unroll
+    for (int m = 0; m < MTT; ++m)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b[t][i] = (unsigned)o.v[t][2 * i] | ((unsigned)o.v[t][2 * i + 1] << 16);
-#pragma unroll
-      for (int a = 0; a < MTT; ++a) {
-        const uintx4 av = af[a * 32];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          if (kFirst) acc[a][t] = zero16;
-          acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, av),
-                                                             __builtin_bit_cast(halfx8, b[t]), acc[a][t], 0, 0, 0);
-        }
-      }
-    } else {
-      uintx4 bh[NT], bm[NT], bl[NT];
-#pragma unroll
-      for (int t = 0; t < NT; ++t) split8(o.v[t], bh[t], bm[t], bl[t]);
-#pragma unroll
-      for (int a = 0; a < MTT; ++a) {
-        const uintx4 ah = af[a * 32], am = af[af_part + a * 32], al = af[2 * af_part + a * 32];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          if (kFirst) acc[a][t] = zero16;
-          mfma_split6(acc[a][t], ah, am, al, bh[t], bm[t], bl[t]);
-        }
-      }
-    }
+        for (int r = 0; r < 16; ++r) acc[m][t][r] = 0.f;
   };
   auto fold_tiles = [&](int it) {
     {
@@ -675,22 +682,56 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     }
   };
   __syncthreads();                                       // fragments and zeros are in place
-  {
-    // two operand buffers alternate; the loads of a step are requested one step ahead
-    BOp b0, b1;
-    if (n_it > 0) load_b(0, 0, b0);
-    for (int it = 0; it < n_it; ++it) {
-      load_b(it, 1, b1);
-      multiply(std::true_type(), 0, b0);
-      for (int ks = 1; ks + 1 < ksteps; ks += 2) {
-        load_b(it, ks + 1, b0);
-        multiply(std::false_type(), ks, b1);
-        load_b(it, ks + 2, b1);
-        multiply(std::false_type(), ks + 1, b0);
+  if (n_it > 0) {
+    // Steps (tile, 16 output channels) in one sequence.  A step's grad_out values are requested
+    // three steps ahead into a ring of four register sets, cut (and its fragments read from LDS)
+    // while the step before it multiplies, and every part of that is pinned in place: left to
+    // itself the scheduler moves each load next to its first use, and a step then waits for the
+    // whole trip to memory.
+    constexpr int D = 4;
+    BOp ring[D];
+    AOp A[2];
+    SOp S[2];
+    int it_req = 0, ks_req = 0, ks_stage = 0;
+    auto request = [&](BOp &o) {
+      load_b(min(it_req, n_it - 1), ks_req, o);          // (past the last step: a valid address, never used)
+      if (++ks_req == ksteps) { ks_req = 0; ++it_req; }
+    };
+    auto stage_next = [&](const BOp &o, AOp &a, SOp &sv) {
+      stage(ks_stage, o, a, sv);
+      if (++ks_stage == ksteps) ks_stage = 0;
+    };
+    request(ring[0]);
+    request(ring[1]);
+    request(ring[2]);
+    stage_next(ring[0], A[0], S[0]);
+    clear_sums();
+    int it = 0, ks = 0;
+    for (int st = 0; st < total; st += D) {
+#pragma unroll
+      for (int u = 0; u < D; ++u) {
+        if (st + u < total) {
+          __builtin_amdgcn_sched_barrier(0);
+          request(ring[(u + 3) & 3]);
+          stage_next(ring[(u + 1) & 3], A[(u + 1) & 1], S[(u + 1) & 1]);   // (after the last step: cut and never used)
+          multiply(A[u & 1], S[u & 1]);
+          // the requests first, then after every matrix instruction a few of the next step's cuts and one fragment read
+          __builtin_amdgcn_sched_group_barrier(0x020, 8 * NT, 0);
+#pragma unroll
+          for (int k = 0; k < MTT * NT * (F16 ? 1 : 6); ++k) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, F16 ? 8 : 4, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (++ks == ksteps) {
+            fold_tiles(it);
+            clear_sums();
+            ks = 0;
+            ++it;
+          }
+        }
       }
-      if (it + 1 < n_it) load_b(it + 1, 0, b0);
-      multiply(std::false_type(), ksteps - 1, b1);
-      fold_tiles(it);
     }
   }
   __syncthreads();                                       // every wavefront's image is complete; the fragments are free
@@ -701,8 +742,8 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
   // goes (-1 nowhere: another strip owns it, or it lies outside grad_input; 0 straight to
   // grad_input; 1 a partial row in the workspace, upper strip's share first) at which word
   // of the image's grad_input or workspace slice, which wavefronts' images reach it and
-  // where their rows lie.  Then a wavefront takes rows wave, wave + 4, ... of every input
-  // channel with its lanes on the columns, and everything wave-uniform comes from the table.
+  // where their rows lie.  Then every thread takes words of the strip's image, reading its
+  // row's entry from the table.
   const int g0 = pl.sx * ha - pl.px;
   const int rp_t = max(pl.Rp, pl.sx * pl.Th);
   int4 *row_tab = (int4 *)lds;                           // kind, destination word, first image word, images
@@ -740,52 +781,45 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     const int gi_c = pl.ngx * pl.ngy, ws_c = (pl.strips - 1) * pl.nshared * 2 * pl.ngy;   // words per input channel
     T *GIn = GI + (i64)n * pl.c_in * gi_c;
     float *WSn = WS + (i64)n * pl.c_in * ws_c;
-    // four rows of every input channel per trip: their table entries first (the same for
-    // every channel), then all their reads, then the stores, so that the LDS round trips of a
-    // trip overlap and a wavefront makes three trips, not nine (lconv2d.grad_input of the
-    // benchmark 72 -> 67.5 us; eight rows per trip ran out of registers)
-    constexpr int kRowsTrip = 4;
-    // (a trip's table entries serve every input channel: the channels inside the trip)
-    for (int pi = wave; pi < rp_t; pi += kRowsTrip * kWaves) {
-      int kind[kRowsTrip], dst[kRowsTrip], src[kRowsTrip], nw[kRowsTrip];
+    // One word of the strip's image per thread and trip, (row, input channel, column) flattened with
+    // the column fastest, four words in flight per thread: everything is per-lane vector code (the
+    // row's table entry comes through an LDS read like the data), so nothing waits on a scalar.  A
+    // word is the sum of at most reach_w wavefronts' images; words of wavefronts that do not hold
+    // the row are read from the first one's and dropped.
+    const int cols = pl.c_in * pl.ngy, words = rp_t * cols;
+    const int reach_w = min(kWaves, (Rw + pl.sx * pl.rw - 1) / (pl.sx * pl.rw));   // images a row can lie in
+    const FastDiv by_cols(cols), by_ngy(pl.ngy);
+    constexpr int kFlight = 4;
+    for (int e0 = tid; e0 < words; e0 += kFlight * 256) {
+      int kind[kFlight], dst[kFlight];
+      float v[kFlight];
 #pragma unroll
-      for (int u = 0; u < kRowsTrip; ++u) {
-        const int4 e = row_tab[min(pi + u * kWaves, rp_t - 1)];
-        kind[u] = pi + u * kWaves < rp_t ? __builtin_amdgcn_readfirstlane(e.x) : -1;
-        dst[u] = __builtin_amdgcn_readfirstlane(e.y);
-        src[u] = __builtin_amdgcn_readfirstlane(e.z);
-        nw[u] = __builtin_amdgcn_readfirstlane(e.w);
-      }
-      for (int gy = lane; gy < pl.ngy; gy += 64) {
+      for (int u = 0; u < kFlight; ++u) {
+        const int e = min(e0 + u * 256, words - 1);
+        int pi, idx, cc, gy;
+        by_cols.divmod(e, pi, idx);
+        by_ngy.divmod(idx, cc, gy);
+        const int4 row = row_tab[pi];
         const bool inside = gy + pl.py < pl.Wp;
-        const int col = inside ? gy : 0;
-        for (int cc0 = 0; cc0 < pl.c_in; cc0 += 3) {
-          float x[3][kRowsTrip][kWaves];
-#pragma unroll
-          for (int c3 = 0; c3 < 3; ++c3) {
-            const int cc = min(cc0 + c3, pl.c_in - 1);
-#pragma unroll
-            for (int u = 0; u < kRowsTrip; ++u) {
-              const float *in = wplanes + src[u] + cc * wplane_words + pl.py;
-#pragma unroll
-              for (int k = 0; k < kWaves; ++k) x[c3][u][k] = in[(k < nw[u] ? k * wave_step : 0) + col];
-            }
-          }
-#pragma unroll
-          for (int c3 = 0; c3 < 3; ++c3) {
-            const int cc = cc0 + c3;
-            if (cc < pl.c_in) {
-#pragma unroll
-              for (int u = 0; u < kRowsTrip; ++u) {
-                float v = 0.f;
-#pragma unroll
-                for (int k = 0; k < kWaves; ++k) v += (inside && k < nw[u]) ? x[c3][u][k] : 0.f;
-                if (kind[u] > 0) (WSn + cc * ws_c + dst[u])[gy] = v;
-                else if (kind[u] == 0) (GIn + cc * gi_c + dst[u])[gy] = (T)v;
-              }
-            }
+        const float *in = wplanes + row.z + cc * wplane_words + pl.py + (inside ? gy : 0);
+        float sum = in[0];
+        if (reach_w > 1) {
+          const float x1 = in[1 < row.w ? wave_step : 0];
+          sum += 1 < row.w ? x1 : 0.f;
+          if (reach_w > 2) {
+            const float x2 = in[2 < row.w ? 2 * wave_step : 0], x3 = in[3 < row.w ? 3 * wave_step : 0];
+            sum += 2 < row.w ? x2 : 0.f;
+            sum += 3 < row.w ? x3 : 0.f;
           }
         }
+        v[u] = (inside && row.w > 0) ? sum : 0.f;
+        kind[u] = e0 + u * 256 < words ? row.x : -1;
+        dst[u] = cc * (row.x > 0 ? ws_c : gi_c) + row.y + gy;
+      }
+#pragma unroll
+      for (int u = 0; u < kFlight; ++u) {
+        if (kind[u] > 0) WSn[dst[u]] = v[u];
+        else if (kind[u] == 0) GIn[dst[u]] = (T)v[u];
       }
     }
   }
