@@ -788,40 +788,49 @@ __global__ __launch_bounds__(256, 2) void igrad_stream_kernel(const IgradPlan pl
     // the row are read from the first one's and dropped.
     const int cols = pl.c_in * pl.ngy, words = rp_t * cols;
     const int reach_w = min(kWaves, (Rw + pl.sx * pl.rw - 1) / (pl.sx * pl.rw));   // images a row can lie in
-    const FastDiv by_cols(cols), by_ngy(pl.ngy);
+    const float inv_cols = 1.0f / (float)cols, inv_ngy = 1.0f / (float)pl.ngy;
+    // x / d without a branch (x below 2^22: the float quotient is off by one at most)
+    auto quotient = [](int x, int d, float inv) {
+      const int q = (int)((float)x * inv), r = x - q * d;
+      return q + (r >= d ? 1 : 0) - (r < 0 ? 1 : 0);
+    };
     constexpr int kFlight = 4;
-    for (int e0 = tid; e0 < words; e0 += kFlight * 256) {
-      int kind[kFlight], dst[kFlight];
-      float v[kFlight];
+    auto write_out = [&](auto reach_tag) {
+      constexpr int kReach = decltype(reach_tag)::value;
+      for (int e0 = tid; e0 < words; e0 += kFlight * 256) {
+        int4 row[kFlight];
+        int cc[kFlight], gy[kFlight];
 #pragma unroll
-      for (int u = 0; u < kFlight; ++u) {
-        const int e = min(e0 + u * 256, words - 1);
-        int pi, idx, cc, gy;
-        by_cols.divmod(e, pi, idx);
-        by_ngy.divmod(idx, cc, gy);
-        const int4 row = row_tab[pi];
-        const bool inside = gy + pl.py < pl.Wp;
-        const float *in = wplanes + row.z + cc * wplane_words + pl.py + (inside ? gy : 0);
-        float sum = in[0];
-        if (reach_w > 1) {
-          const float x1 = in[1 < row.w ? wave_step : 0];
-          sum += 1 < row.w ? x1 : 0.f;
-          if (reach_w > 2) {
-            const float x2 = in[2 < row.w ? 2 * wave_step : 0], x3 = in[3 < row.w ? 3 * wave_step : 0];
-            sum += 2 < row.w ? x2 : 0.f;
-            sum += 3 < row.w ? x3 : 0.f;
-          }
+        for (int u = 0; u < kFlight; ++u) {
+          const int e = min(e0 + u * 256, words - 1);
+          const int pi = quotient(e, cols, inv_cols), idx = e - pi * cols;
+          cc[u] = quotient(idx, pl.ngy, inv_ngy);
+          gy[u] = idx - cc[u] * pl.ngy;
+          row[u] = row_tab[pi];
         }
-        v[u] = (inside && row.w > 0) ? sum : 0.f;
-        kind[u] = e0 + u * 256 < words ? row.x : -1;
-        dst[u] = cc * (row.x > 0 ? ws_c : gi_c) + row.y + gy;
-      }
+        float x[kFlight][kReach];
+        bool inside[kFlight];
 #pragma unroll
-      for (int u = 0; u < kFlight; ++u) {
-        if (kind[u] > 0) WSn[dst[u]] = v[u];
-        else if (kind[u] == 0) GIn[dst[u]] = (T)v[u];
+        for (int u = 0; u < kFlight; ++u) {
+          inside[u] = gy[u] + pl.py < pl.Wp;
+          const float *in = wplanes + row[u].z + cc[u] * wplane_words + pl.py + (inside[u] ? gy[u] : 0);
+#pragma unroll
+          for (int k = 0; k < kReach; ++k) x[u][k] = in[k < row[u].w ? k * wave_step : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < kFlight; ++u) {
+          float sum = 0.f;
+#pragma unroll
+          for (int k = 0; k < kReach; ++k) sum += (inside[u] && k < row[u].w) ? x[u][k] : 0.f;
+          const int kind = e0 + u * 256 < words ? row[u].x : -1;
+          const int dst = cc[u] * (kind > 0 ? ws_c : gi_c) + row[u].y + gy[u];
+          if (kind > 0) WSn[dst] = sum;
+          else if (kind == 0) GIn[dst] = (T)sum;
+        }
       }
-    }
+    };
+    if (reach_w <= 2) write_out(std::integral_constant<int, 2>());
+    else write_out(std::integral_constant<int, kWaves>());
   }
   // grad_input rows past the reach of the last grad_out row belong to the last strip: zeros
   if (strip == pl.strips - 1) {
