@@ -520,14 +520,29 @@ __device__ __forceinline__ void multiply_taps_split(floatx16 (&acc)[MT][NT], con
 #pragma unroll
       for (int t = 0; t < NT; ++t) mfma_split6(acc[i][t], o.ah[i], o.am[i], o.al[i], o.bh[t], o.bm[t], o.bl[t]);
   };
+  // A step's operands are fetched and cut while the step before it multiplies: after every matrix
+  // instruction one LDS read and a few of the vector instructions of the cut, pinned (left to
+  // itself the scheduler moves every read next to its first use and the step waits for LDS).  The
+  // loop body has no exit between a fetch and its use: the fetch past the last step reads the
+  // last step's operands again.
+  auto interleave = [] {
+#pragma unroll
+    for (int k = 0; k < MT * NT * 6; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       // one matrix instruction
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);       // two LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);       // six vector instructions
+    }
+  };
   Ops a, b;
   int s = 0;
   if (steps > 0) fetch(0, a);
   for (; s + 1 < steps; s += 2) {
     fetch(s + 1, b);
     multiply(a);
-    if (s + 2 < steps) fetch(s + 2, a);
+    interleave();
+    fetch(min(s + 2, steps - 1), a);
     multiply(b);
+    interleave();
   }
   if (s < steps) multiply(a);
 }
