@@ -218,6 +218,8 @@ __device__ __forceinline__ void tile_gemm_body(
   const int cc_last = pl.C - (chunks - 1) * pl.CC;
   __amdgpu_buffer_rsrc_t f_rsrc;
   if (SPLIT) f_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)F, 0, (int)pl.f_bytes, 0x00020000);
+  const bool dense = SPLIT == 1 && pl.f_dense;          // (one chunk, the filter's own tap order)
+  const int K_dense = pl.C * pl.nf;
   auto load_filter = [&](int ch, int first, FilterWords &fw) {
     const int *ko = tapoff + (ch + 1 == chunks ? 3 : 2) * pl.KC16;
     const int soff = (int)((unsigned)(ch * pl.CC) * (unsigned)pl.f_c * (unsigned)EB);
@@ -227,8 +229,22 @@ __device__ __forceinline__ void tile_gemm_body(
       const int idx = first + tid + j * kThreads;
       if (idx < f_groups * M_T) {
         int m, g;
-        by_groups.divmod(idx, m, g);
+        if (dense) { g = idx / M_T; m = idx - g * M_T; }   // channels fastest: the fragment writes are conflict-free
+        else by_groups.divmod(idx, m, g);
         const unsigned row = m0 + m < pl.M ? (unsigned)(m0 + m) * (unsigned)pl.f_m * (unsigned)EB : kDeadOffset;
+        if constexpr (!F16) {
+          if (dense) {
+            // the eight taps are 32 consecutive bytes of the channel's row (any 4-byte alignment)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const int k = 8 * g + 4 * h;
+              const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(f_rsrc, k < K_dense ? (int)(row + 4u * (unsigned)k) : (int)kDeadOffset, 0, 0);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) fw.x[j][4 * h + i] = __uint_as_float(v[i]);
+            }
+            continue;
+          }
+        }
         const int4 k0 = *(const int4 *)(ko + 8 * g), k1 = *(const int4 *)(ko + 8 * g + 4);
         const int off[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
 #pragma unroll
@@ -248,7 +264,8 @@ __device__ __forceinline__ void tile_gemm_body(
       const int idx = first + tid + j * kThreads;
       if (idx < f_groups * M_T) {
         int m, g;
-        by_groups.divmod(idx, m, g);
+        if (dense) { g = idx / M_T; m = idx - g * M_T; }
+        else by_groups.divmod(idx, m, g);
         if constexpr (F16) {
           uintx4 v;
 #pragma unroll
@@ -261,6 +278,9 @@ __device__ __forceinline__ void tile_gemm_body(
     }
   };
 
+  // (dense: the first round of the filter's words is requested before the tables are made; it needs none of them)
+  FilterWords fw_first;
+  if (dense && my_stages > 0) load_filter(0, 0, fw_first);
   {
     const FastDiv by_nf(pl.nf), by_nfy(pl.nfy);
     for (int k = tid; k < (SPLIT ? pl.KC16 : pl.KCp); k += kThreads) {
@@ -292,6 +312,7 @@ __device__ __forceinline__ void tile_gemm_body(
       // (a filter that is one chunk may have more items than one round of the threads)
       if (!single_chunk && (AF || SPLIT == 4)) copy_fragments(0, ws_word0);
       else for (int first = 0; first < f_groups * M_T; first += kFilterItems * kThreads) {
+        if (dense && first == 0) { store_filter(fw_first, 0, Ws0); continue; }
         FilterWords fw;
         load_filter(0, first, fw);
         store_filter(fw, first, Ws0);
@@ -807,6 +828,7 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
   // the bf16 matrix cores: the filter block as fragments (6 bytes per word, taps padded to
   // a multiple of 16), built by 256 threads of two 8-tap items each
   pl.split = 0;
+  pl.f_dense = 0;
   pl.f16 = 0;
   pl.KC16 = 0;
   pl.f_bytes = 0;
@@ -856,6 +878,8 @@ bool make_tile_plan(const SepConv &pr, TilePlan &pl, size_t *lds_bytes, int *mt,
     if (whole_split) {
       pl.split = 1;
       pl.KC16 = (int)(((pl.C * pl.nf + 15) / 16) * 16);
+      // (the kernel's taps are the filter's own, in its own order: fragments can be cut from 16-byte loads)
+      pl.f_dense = !cls && pl.f_off == 0 && pl.f_pitch == pl.nfy && pr.f_c == pl.nf && ((pl.C * pl.nf) & 3) == 0;
       *lds_bytes = split_lds(2, pl.C, true);
     } else if (pr.math == MATH_BF16X3_ALWAYS ||
                (!single && (double)pr.batch * (double)Q * (double)pr.c_out * (double)pr.c_in * (double)nf >= 8e8)) {

@@ -39,6 +39,7 @@ struct TilePlan {
   int KCp;                         // CC * nf rounded up to even
   int WSS;                         // stride of the K-major filter block (words)
   int split;                       // products on the bf16 matrix cores, operands as three bf16 parts each
+  int f_dense;                     // split, one chunk, fp32: a channel's taps are K consecutive words in the kernel's order, K a multiple of 4
   int f16;                         // (with split) half-precision operands on the f16 matrix cores instead: one part
   int KC16;                        // split: CC * nf rounded up to a multiple of 16
   unsigned f_bytes;                // split: bytes from the filter's first word to its last one's end
