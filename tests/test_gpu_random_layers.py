@@ -217,3 +217,36 @@ def test_narrow_forward_kernel_forced():
     choice takes it from 1024 tiles on): partial tiles, partial channel blocks, 1-16 input channels."""
     v = _sweep(111, "narrow-class", math=hip.MATH_BF16X3_ALWAYS, variant="narrow")
     assert v.get("mfma-narrow", 0) >= 40, v
+
+
+def test_narrow_forward_kernel_relu_and_no_bias():
+    """The few-channel linear forward kernel with the fused ReLU and without a bias: bit-identical
+    to relu(.) of its own plain result, and to the plain result with a zero bias."""
+    rng = np.random.default_rng(112)
+    hip.set_math(hip.MATH_BF16X3_ALWAYS)
+    hip.set_variant("narrow")
+    try:
+        for n, c_in, c_out, nf, ng, s, d in ((2, 3, 64, (8, 4), (70, 41), (1, 1), (1, 1)),
+                                             (3, 5, 33, (3, 2), (24, 13), (2, 1), (3, 1)),
+                                             (1, 8, 70, (2, 4), (14, 12), (1, 1), (2, 1))):
+            x = to_gpu(rng.standard_normal((n, c_in) + ng).astype(np.float32))
+            w = to_gpu((rng.standard_normal((c_out, c_in) + nf) * 0.2).astype(np.float32))
+            b = to_gpu(rng.standard_normal(c_out).astype(np.float32))
+            nh = ((ng[0] - d[0] * (nf[0] - 1) - 1) // s[0] + 1, ng[1] - nf[1] + 1)
+            dims = hip._dims(n, c_in, c_out, nf, ng, nh, s, d, (0, 0), (1, 1))
+            nan = float("nan")
+            plain = torch.full((n, c_out) + nh, nan, device="cuda")
+            act = torch.full_like(plain, nan)
+            hip.corr2d_forward(hip.AX_LCORR, x, w, b, plain, dims)
+            assert hip.last_variant() == "mfma-narrow"
+            hip.corr2d_forward(hip.AX_LCORR, x, w, b, act, dims, activation=hip.ACT_RELU)
+            assert hip.last_variant() == "mfma-narrow"
+            assert torch.equal(act, torch.relu(plain))
+            nobias = torch.full_like(plain, nan)
+            zero = torch.full_like(plain, nan)
+            hip.corr2d_forward(hip.AX_LCORR, x, w, None, nobias, dims)
+            hip.corr2d_forward(hip.AX_LCORR, x, w, torch.zeros_like(b), zero, dims)
+            assert torch.equal(nobias, zero) and not torch.isnan(nobias).any()
+    finally:
+        hip.set_variant(None)
+        hip.set_math(hip.MATH_BF16X3)
