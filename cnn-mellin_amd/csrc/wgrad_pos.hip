@@ -318,8 +318,9 @@ bool make_wgrad_pos_plan(const SepConv &fwd_in, WgradPosPlan &wp, bool half) {
   pl.contig = 0;
   pl.RS = (pl.ay * (pl.noy - 1) + pl.by_span + 1) | 1;
   wp.J = pl.C * pl.nf;
-  // (fp32: three-part operands take the registers of a fourth column tile)
-  wp.jt = std::min(half ? 4 : 3, (wp.J + 31) / 32);
+  // (four column tiles in both precisions; the fp32 instance then holds 244 registers, without spills:
+  //  grad_out is re-read once per block of 128 columns instead of 96)
+  wp.jt = std::min(4, (wp.J + 31) / 32);
   wp.mbw = pl.M > 128 ? 4 : (pl.M > 64 ? 2 : 1);
   const int M_T = 64 * wp.mbw, J_T = wp.jt * 32;
   wp.m_groups = (pl.M + M_T - 1) / M_T;
@@ -365,6 +366,7 @@ hipError_t launch_wgrad_pos(const WgradPosPlan &wp, const void *grad_out, const 
     if (wp.jt == 1) e = launch_pos<1, false>(wp, grid, grad_out, input, workspace, stream);
     if (wp.jt == 2) e = launch_pos<2, false>(wp, grid, grad_out, input, workspace, stream);
     if (wp.jt == 3) e = launch_pos<3, false>(wp, grid, grad_out, input, workspace, stream);
+    if (wp.jt == 4) e = launch_pos<4, false>(wp, grid, grad_out, input, workspace, stream);
   }
   if (e != hipSuccess) return e;
   return launch_wgrad_reduce(workspace, grad_weight, wp.half, wp.S * (kWaves / wp.mbw), wp.t.M, wp.J,
