@@ -457,11 +457,16 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
     }
   }
 
-  // ---- sum the four wavefronts in wave order, then write the partial block ------
+  // ---- sum the four wavefronts, then write the partial block -------------------------------
+  // Every workgroup of the one-round grid gets here at the same moment, so this is on the launch's
+  // critical path.  Two slabs: wavefronts 0 and 2 store their sums, 1 and 3 add theirs on top, and
+  // the block is slab 0 + slab 1, i.e. (w0 + w1) + (w2 + w3) whatever the timing; the write-out
+  // has several words in flight per thread.
   __syncthreads();
-  float *red = lds;                                   // [M_T][J_T]
-  for (int w = 0; w < kWaves; ++w) {
-    if (wave == w) {
+  float *red = lds;                                   // [2][M_T][J_T]
+  for (int phase = 0; phase < 2; ++phase) {
+    if ((wave & 1) == phase) {
+      float *slab = red + (wave >> 1) * (M_T * J_T);
 #pragma unroll
       for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -469,17 +474,24 @@ __global__ __launch_bounds__(kThreads) void wgrad_rows_kernel(
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int m = i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-            float *dst = red + m * J_T + t * 32 + l32;
-            if (w == 0) *dst = acc[i][t][r];
+            float *dst = slab + m * J_T + t * 32 + l32;
+            if (phase == 0) *dst = acc[i][t][r];
             else *dst += acc[i][t][r];
           }
     }
     __syncthreads();
   }
   float *out = ws + (i64)blockIdx.x * wp.M_pad * wp.J_pad + (i64)m0 * wp.J_pad + j0;
-  for (int e = tid; e < M_T * J_T; e += kThreads) {
-    const int m = e / J_T, jj = e - m * J_T;
-    out[(i64)m * wp.J_pad + jj] = red[e];
+  constexpr int kTrip = 4;                             // words a thread has in flight (M_T * J_T is a multiple of 1024)
+  for (int e0 = tid; e0 < M_T * J_T; e0 += kTrip * kThreads) {
+    float v[kTrip];
+#pragma unroll
+    for (int u = 0; u < kTrip; ++u) v[u] = red[e0 + u * kThreads] + red[M_T * J_T + e0 + u * kThreads];
+#pragma unroll
+    for (int u = 0; u < kTrip; ++u) {
+      const int e = e0 + u * kThreads, m = e / J_T, jj = e - m * J_T;
+      out[(i64)m * wp.J_pad + jj] = v[u];
+    }
   }
 }
 
@@ -967,10 +979,11 @@ static bool make_wgrad_plan_jt(const SepConv &fwd, WgradPlan &wp, bool g_allow_r
       // all channels in one workgroup (two 32-row tiles) only on request: fewer, fatter
       // workgroups have measured slower
       int mt_rows = (pl.M > 32 && rows_opt_mt == 2) ? 2 : 1;
-      size_t bytes = 4 * std::max(nbuf * (xw + (size_t)mt_rows * 32 * pitch), (size_t)mt_rows * 32 * J_T);
+      // (the second term: two slabs of sums at the end)
+      size_t bytes = 4 * std::max(nbuf * (xw + (size_t)mt_rows * 32 * pitch), 2 * (size_t)mt_rows * 32 * J_T);
       if (mt_rows == 2 && bytes > 150 * 1024) {
         mt_rows = 1;
-        bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), (size_t)32 * J_T);
+        bytes = 4 * std::max(nbuf * (xw + (size_t)32 * pitch), 2 * (size_t)32 * J_T);
       }
       if (Rr > 8192 || pitch * 32 * 4 >= 65536 || bytes > (mt_rows == 2 ? 150 : 78) * 1024) continue;
       const int m_groups = (pl.M + mt_rows * 32 - 1) / (mt_rows * 32);
